@@ -1,0 +1,423 @@
+// Block-scaled FP8 GEMM for gfx950:  C[m,n] = sum_kb (sum_{k in kb} Aq[m,k] Bq[n,k]) * As[m,kb] * Bs[n/128,kb].
+//
+// One 256-thread workgroup (4 waves, 2 x 2) owns a 128(M) x 128(N) tile of C and
+// walks K in steps of 128 = one scale block.  Per step the two operand tiles
+// (128 rows x 128 bytes each) are staged through LDS (double buffered, rows
+// padded to 144 bytes so that 128-bit reads and writes are bank-conflict free),
+// each wave issues v_mfma_f32_32x32x64_f8f6f4 with FP8 operands on its
+// 64 x 64 sub-tile into a zero-initialised partial accumulator, and the partial
+// is folded into the fp32 accumulator with one FMA per element by
+// As[m,kb] * Bs[n/128,kb].
+//
+// The weight tile is the MFMA "A" operand and the activation tile the "B"
+// operand, so the accumulator of a lane holds one activation row m (lane % 32)
+// and 16 weight rows n: the activation scale is then a single value per lane.
+//
+// The same tile routine serves the dense, split-K (skinny M) and grouped
+// (per-expert row ranges) entry points.
+#include "lowp_device.h"
+
+using namespace lowp;
+
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 128, TN = 128, TK = 128;
+constexpr int LDS_ROW = TK + 16;                 // bytes per staged row
+constexpr int TILE_BYTES = 128 * LDS_ROW;        // one operand tile in LDS
+
+struct Smem {
+    uint8_t a[2][TILE_BYTES];
+    uint8_t b[2][TILE_BYTES];
+    float as[2][TM];
+};
+
+struct TileArgs {
+    const uint8_t *Aq;   // [*, K] activation codes
+    const void *As;      // [*, K/128] activation scales
+    const uint8_t *Bq;   // [N, K] weight codes of this problem (expert)
+    const void *Bs;      // [N/128, K/128]
+    int scale_dtype;
+    int64_t K;
+    int64_t kblocks;     // K / 128
+    int64_t m0;          // first row of the tile
+    int64_t m_end;       // rows >= m_end are not read or written
+    int64_t n0;          // first weight row of the tile
+    int kb_begin, kb_end;
+};
+
+__device__ __forceinline__ float scale_at(const void *s, int dtype, int64_t idx)
+{
+    if (dtype == LP_F32) return ((const float *)s)[idx];
+    return e8m0_to_f32(((const uint8_t *)s)[idx]);
+}
+
+// accumulators of one wave: acc[mb][nb] is a 32(n) x 32(m) block
+struct Acc { f32x16 v[2][2]; };
+
+__device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc)
+{
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
+
+    // global -> register staging: 4 chunks of 16 bytes per operand per thread
+    u32x4 ga[4], gb[4];
+    float gas = 0.0f;
+    auto gload = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = t + 256 * i;
+            const int row = c >> 3, col = (c & 7) * 16;
+            const int64_t m = ta.m0 + row;
+            if (m < ta.m_end) ga[i] = *(const u32x4 *)(ta.Aq + m * ta.K + (int64_t)kb * TK + col);
+            else ga[i] = u32x4{0, 0, 0, 0};
+            gb[i] = *(const u32x4 *)(ta.Bq + (ta.n0 + row) * ta.K + (int64_t)kb * TK + col);
+        }
+        if (t < TM) {
+            const int64_t m = ta.m0 + t;
+            gas = m < ta.m_end ? scale_at(ta.As, ta.scale_dtype, m * ta.kblocks + kb) : 0.0f;
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = t + 256 * i;
+            const int row = c >> 3, col = (c & 7) * 16;
+            *(u32x4 *)(sm.a[buf] + row * LDS_ROW + col) = ga[i];
+            *(u32x4 *)(sm.b[buf] + row * LDS_ROW + col) = gb[i];
+        }
+        if (t < TM) sm.as[buf][t] = gas;
+    };
+
+    gload(ta.kb_begin);
+    sstore(0);
+    __syncthreads();
+
+    for (int kb = ta.kb_begin; kb < ta.kb_end; ++kb) {
+        const int buf = (kb - ta.kb_begin) & 1;
+        const bool more = kb + 1 < ta.kb_end;
+        if (more) gload(kb + 1);
+
+        const float bscale = scale_at(ta.Bs, ta.scale_dtype, (ta.n0 >> 7) * ta.kblocks + kb);
+
+        // operand fragments: lane reads 32 bytes of its row per 64-wide K half
+        i32x8 wf[2][2], af[2][2];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int kh = 0; kh < 2; ++kh) {
+                const int koff = kh * 64 + lhi * 32;
+                const uint8_t *wp = sm.b[buf] + (wn * 64 + blk * 32 + l32) * LDS_ROW + koff;
+                const uint8_t *ap = sm.a[buf] + (wm * 64 + blk * 32 + l32) * LDS_ROW + koff;
+                u32x4 w0 = *(const u32x4 *)wp, w1 = *(const u32x4 *)(wp + 16);
+                u32x4 a0 = *(const u32x4 *)ap, a1 = *(const u32x4 *)(ap + 16);
+                wf[blk][kh] = i32x8{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+                af[blk][kh] = i32x8{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+            }
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            const float sc = sm.as[buf][wm * 64 + mb * 32 + l32] * bscale;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                f32x16 p = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                p = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][0], af[mb][0], p, 0, 0, 0, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][1], af[mb][1], p, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = __builtin_fmaf(p[r], sc, acc.v[mb][nb][r]);
+            }
+        }
+        if (more) sstore(buf ^ 1);
+        __syncthreads();
+    }
+}
+
+// element (mb, nb, r) of a lane's accumulator sits at
+//   m = m0 + wm*64 + mb*32 + lane%32
+//   n = n0 + wn*64 + nb*32 + 8*(r/4) + 4*(lane/32) + r%4
+template <typename F>
+__device__ __forceinline__ void for_each_quad(const Acc &acc, int64_t m0, int64_t n0, F &&f)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        const int64_t m = m0 + wm * 64 + mb * 32 + (lane & 31);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int64_t n = n0 + wn * 64 + nb * 32 + 8 * g + 4 * (lane >> 5);
+                f(m, n, acc.v[mb][nb][4 * g], acc.v[mb][nb][4 * g + 1], acc.v[mb][nb][4 * g + 2], acc.v[mb][nb][4 * g + 3]);
+            }
+    }
+}
+
+__device__ __forceinline__ void store_tile(const Acc &acc, int64_t m0, int64_t m_end, int64_t n0, int64_t N, void *C,
+                                           int out_dtype)
+{
+    for_each_quad(acc, m0, n0, [&](int64_t m, int64_t n, float a, float b, float c, float d) {
+        if (m >= m_end) return;
+        if (out_dtype == LP_BF16) {
+            u32x2 o = {pack_bf16(a, b), pack_bf16(c, d)};
+            *(u32x2 *)((uint16_t *)C + m * N + n) = o;
+        } else {
+            u32x4 o = {f2u(a), f2u(b), f2u(c), f2u(d)};
+            *(u32x4 *)((float *)C + m * N + n) = o;
+        }
+    });
+}
+
+// Tile order: tiles are numbered so that 32 consecutive numbers form a block of
+// 8 M-tiles x 4 N-tiles (shared operand panels), and each XCD (workgroup id
+// modulo 8) is handed whole blocks, so panels are re-used out of one L2.
+constexpr int GROUP_M = 8, GROUP_N = 4, CHUNK = GROUP_M * GROUP_N;
+
+__device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t tiles_n, int64_t &tm, int64_t &tn)
+{
+    const int64_t xcd = b & 7, s = b >> 3;
+    const int64_t lin = ((s / CHUNK) * 8 + xcd) * CHUNK + s % CHUNK;
+    if (lin >= tiles_m * tiles_n) return false;
+    // groups of GROUP_M m-tiles (the last may be short); inside a group, blocks of
+    // GROUP_N n-tiles (the last may be narrow); inside a block m runs fastest
+    const int64_t per_group = GROUP_M * tiles_n;
+    const int64_t grp = lin / per_group, in_grp = lin - grp * per_group;
+    const int64_t left = tiles_m - grp * GROUP_M;
+    const int64_t gm = left < GROUP_M ? left : GROUP_M;
+    const int64_t per_nblock = gm * GROUP_N;
+    const int64_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
+    tm = grp * GROUP_M + in_blk % gm;
+    tn = nblk * GROUP_N + in_blk / gm;
+    return true;
+}
+
+__global__ __launch_bounds__(256) void gemm_dense(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                  const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                  int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
+                                                  int64_t tiles_n, void *__restrict__ C, int out_dtype)
+{
+    __shared__ Smem sm;
+    int64_t tm, tn;
+    if (!tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    TileArgs ta;
+    ta.Aq = Aq; ta.As = As; ta.Bq = Bq; ta.Bs = Bs; ta.scale_dtype = scale_dtype;
+    ta.K = K; ta.kblocks = K / TK; ta.m0 = tm * TM; ta.m_end = M; ta.n0 = tn * TN;
+    ta.kb_begin = 0; ta.kb_end = (int)(K / TK);
+    Acc acc;
+    gemm_tile(ta, sm, acc);
+    store_tile(acc, ta.m0, M, ta.n0, N, C, out_dtype);
+}
+
+int64_t padded_grid(int64_t tiles_m, int64_t tiles_n)
+{
+    const int64_t chunks = (tiles_m * tiles_n + CHUNK - 1) / CHUNK;
+    return ((chunks + 7) / 8) * 8 * CHUNK;
+}
+
+
+// ------------------------------------------------------------------ split-K
+// Skinny problems (few output tiles) are weight-streaming bound: K is cut into
+// `splits` contiguous ranges so that every CU pulls HBM; each range writes an
+// fp32 partial tile to the workspace and a second kernel adds the ranges in a
+// fixed order (deterministic) and narrows.
+
+__global__ __launch_bounds__(256) void gemm_splitk(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                   int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
+                                                   int64_t tiles_n, int splits, int kb_per_split, float *__restrict__ ws)
+{
+    __shared__ Smem sm;
+    const int64_t tile = blockIdx.x / splits;
+    const int split = (int)(blockIdx.x - tile * splits);
+    const int64_t tn = tile / tiles_m, tm = tile - tn * tiles_m;
+    TileArgs ta;
+    ta.Aq = Aq; ta.As = As; ta.Bq = Bq; ta.Bs = Bs; ta.scale_dtype = scale_dtype;
+    ta.K = K; ta.kblocks = K / TK; ta.m0 = tm * TM; ta.m_end = M; ta.n0 = tn * TN;
+    ta.kb_begin = split * kb_per_split;
+    const int kb_all = (int)(K / TK);
+    ta.kb_end = ta.kb_begin + kb_per_split < kb_all ? ta.kb_begin + kb_per_split : kb_all;
+    Acc acc;
+    if (ta.kb_begin < ta.kb_end) {
+        gemm_tile(ta, sm, acc);
+    } else {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
+    }
+    store_tile(acc, ta.m0, M, ta.n0, N, ws + (int64_t)split * M * N, LP_F32);
+}
+
+__global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ ws, int splits, int64_t mn,
+                                                     void *__restrict__ C, int out_dtype)
+{
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= mn) return;
+    f32x4 s = *(const f32x4 *)(ws + i);
+    for (int k = 1; k < splits; ++k) {
+        f32x4 v = *(const f32x4 *)(ws + (int64_t)k * mn + i);
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    if (out_dtype == LP_BF16) {
+        u32x2 o = {pack_bf16(s.x, s.y), pack_bf16(s.z, s.w)};
+        *(u32x2 *)((uint16_t *)C + i) = o;
+    } else {
+        *(f32x4 *)((float *)C + i) = s;
+    }
+}
+
+// how many K ranges to use: aim at >= 2 workgroups per CU (256 CUs)
+int choose_splits(int64_t tiles, int64_t kblocks)
+{
+    if (tiles >= 256 || kblocks < 8) return 1;
+    int64_t s = (512 + tiles - 1) / tiles;
+    if (s > kblocks / 4) s = kblocks / 4;     // keep >= 4 K steps per range
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : (int)s;
+}
+
+// ------------------------------------------------------------------ grouped
+// Rows are sorted by expert; expert e owns rows m_offsets[e] .. m_offsets[e+1]-1.
+// The grid is sized from an upper bound on the number of 128-row tiles; every
+// workgroup finds its (expert, tile) from the offsets with a block-wide scan.
+
+__global__ __launch_bounds__(256) void gemm_grouped(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                    const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                    int scale_dtype, const int32_t *__restrict__ m_offsets, int E,
+                                                    int64_t N, int64_t K, int64_t max_mtiles, int64_t tiles_n,
+                                                    void *__restrict__ C, int out_dtype)
+{
+    __shared__ Smem sm;
+    __shared__ int scan[256];
+    __shared__ int found_e, found_first;
+    int64_t gmt, tn;
+    const bool in_range = tile_coords(blockIdx.x, max_mtiles, tiles_n, gmt, tn);
+    const int t = threadIdx.x;
+    if (t == 0) found_e = -1;
+    __syncthreads();
+    // inclusive scan of per-expert tile counts, 256 experts per round
+    int base = 0;
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int e = e0 + t;
+        int cnt = 0;
+        if (e < E) cnt = (m_offsets[e + 1] - m_offsets[e] + TM - 1) / TM;
+        scan[t] = cnt;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            int v = t >= off ? scan[t - off] : 0;
+            __syncthreads();
+            scan[t] += v;
+            __syncthreads();
+        }
+        const int incl = base + scan[t], excl = incl - cnt;
+        if (in_range && e < E && gmt >= excl && gmt < incl) { found_e = e; found_first = excl; }
+        base += scan[255];
+        __syncthreads();
+    }
+    if (!in_range || found_e < 0) return;
+    const int e = found_e;
+    const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
+    const int64_t kblocks = K / TK;
+    TileArgs ta;
+    ta.Aq = Aq; ta.As = As; ta.scale_dtype = scale_dtype;
+    ta.Bq = Bq + (int64_t)e * N * K;
+    ta.Bs = (const char *)Bs + (int64_t)e * (N / 128) * kblocks * (scale_dtype == LP_F32 ? 4 : 1);
+    ta.K = K; ta.kblocks = kblocks;
+    ta.m0 = row_begin + (gmt - found_first) * TM; ta.m_end = row_end; ta.n0 = tn * TN;
+    ta.kb_begin = 0; ta.kb_end = (int)kblocks;
+    Acc acc;
+    gemm_tile(ta, sm, acc);
+    store_tile(acc, ta.m0, row_end, ta.n0, N, C, out_dtype);
+}
+
+}  // namespace
+
+extern "C" int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+    const int64_t tiles = ((M + TM - 1) / TM) * (N / TN);
+    const int splits = choose_splits(tiles, K / TK);
+    return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
+}
+
+static int check_gemm_args(const char *name, const void *Aq, const void *As, const void *Bq, const void *Bs,
+                           int scale_dtype, int64_t M, int64_t N, int64_t K, const void *C, int out_dtype)
+{
+    LP_REQUIRE(scale_dtype == LP_F32 || scale_dtype == LP_E8M0, "%s: scale_dtype must be LP_F32 or LP_E8M0", name);
+    LP_REQUIRE(out_dtype == LP_BF16 || out_dtype == LP_F32, "%s: out_dtype must be LP_BF16 or LP_F32", name);
+    LP_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative dimension", name);
+    LP_REQUIRE(K % 128 == 0, "%s: K (%lld) must be a multiple of 128", name, (long long)K);
+    LP_REQUIRE(N % 128 == 0, "%s: N (%lld) must be a multiple of 128", name, (long long)N);
+    if (M == 0 || N == 0) return 1;
+    LP_REQUIRE(K > 0, "%s: K must be positive", name);
+    LP_REQUIRE(Aq && As && Bq && Bs && C, "%s: null pointer", name);
+    LP_REQUIRE((uintptr_t)Aq % 16 == 0 && (uintptr_t)Bq % 16 == 0 && (uintptr_t)C % 16 == 0,
+               "%s: operands must be 16-byte aligned", name);
+    return LP_OK;
+}
+
+extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                                 int64_t M, int64_t N, int64_t K, void *C, int out_dtype, void *workspace,
+                                 int64_t workspace_bytes, lp_stream_t stream)
+{
+    int rc = check_gemm_args("lp_gemm_fp8_block", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
+    int splits = choose_splits(tiles_m * tiles_n, K / TK);
+    if (splits > 1 && (!workspace || workspace_bytes < (int64_t)splits * M * N * 4 || (uintptr_t)workspace % 16)) splits = 1;
+    if (splits > 1) {
+        const int kb_all = (int)(K / TK);
+        const int per = (kb_all + splits - 1) / splits;
+        splits = (kb_all + per - 1) / per;
+        hipLaunchKernelGGL(gemm_splitk, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(256), 0, st, (const uint8_t *)Aq,
+                           As, (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, splits, per, (float *)workspace);
+        rc = check_launch("lp_gemm_fp8_block(split-K)");
+        if (rc) return rc;
+        const int64_t mn = M * N;
+        hipLaunchKernelGGL(splitk_reduce, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, st, (const float *)workspace,
+                           splits, mn, C, out_dtype);
+        return check_launch("lp_gemm_fp8_block(reduce)");
+    }
+    const int64_t grid = padded_grid(tiles_m, tiles_n);
+    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");
+    hipLaunchKernelGGL(gemm_dense, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                       (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
+    return check_launch("lp_gemm_fp8_block");
+}
+
+extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                                   const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C,
+                                   int out_dtype, lp_stream_t stream)
+{
+    LP_REQUIRE(E >= 0, "lp_gemm_fp8_grouped: negative expert count");
+    int rc = check_gemm_args("lp_gemm_fp8_grouped", Aq, As, Bq, Bs, scale_dtype, M_total, N, K, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    if (E == 0) return LP_OK;
+    LP_REQUIRE(m_offsets, "lp_gemm_fp8_grouped: null m_offsets");
+    const int64_t max_mtiles = M_total / TM + E, tiles_n = N / TN;
+    const int64_t grid = padded_grid(max_mtiles, tiles_n);
+    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_grouped: problem too large");
+    hipLaunchKernelGGL(gemm_grouped, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
+                       (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+    return check_launch("lp_gemm_fp8_grouped");
+}
+
+extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M, int64_t N, int64_t K, void *C,
+                          int out_dtype, lp_stream_t stream)
+{
+    (void)A; (void)B; (void)in_dtype; (void)M; (void)N; (void)K; (void)C; (void)out_dtype; (void)stream;
+    return lowp::fail(LP_ERR_UNSUPPORTED, "lp_gemm_nt: not built yet");
+}

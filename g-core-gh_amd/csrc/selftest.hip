@@ -1,0 +1,121 @@
+// On-device checks of the gfx950 conversion instructions against the software
+// casts in lowp_math.h, plus bulk casts used by tests.
+#include "lowp_device.h"
+
+using namespace lowp;
+
+namespace {
+
+__device__ __forceinline__ void count(uint64_t *out, bool bad)
+{
+    unsigned long long b = __ballot(bad);
+    if ((threadIdx.x & 63) == 0 && b) atomicAdd((unsigned long long *)out, (unsigned long long)__popcll(b));
+}
+
+// which 0: every fp32 pattern; patterns with |x| > 448 (or NaN) are skipped
+__global__ __launch_bounds__(256) void st_cvt_fp8(uint64_t *out)
+{
+    const uint32_t base = (blockIdx.x * 256u + threadIdx.x) * 16u;
+    bool bad = false;
+    for (uint32_t i = 0; i < 16u; i += 2) {
+        uint32_t u0 = base + i, u1 = base + i + 1;
+        float a = u2f(u0), b = u2f(u1);
+        bool ok0 = (u0 & 0x7FFFFFFFu) <= 0x43E00000u, ok1 = (u1 & 0x7FFFFFFFu) <= 0x43E00000u;
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(ok0 ? a : 0.0f, ok1 ? b : 0.0f, 0, false);
+        int w2 = __builtin_amdgcn_cvt_pk_fp8_f32(ok1 ? b : 0.0f, ok0 ? a : 0.0f, 0, true);
+        if (ok0) bad |= (uint8_t)w != sw_f32_to_e4m3fn(a) || (uint8_t)(w2 >> 24) != sw_f32_to_e4m3fn(a);
+        if (ok1) bad |= (uint8_t)(w >> 8) != sw_f32_to_e4m3fn(b) || (uint8_t)(w2 >> 16) != sw_f32_to_e4m3fn(b);
+    }
+    count(out, bad);
+}
+
+// which 1: 256 codes through all four byte positions
+__global__ __launch_bounds__(256) void st_cvt_from_fp8(uint64_t *out)
+{
+    const uint32_t c = threadIdx.x;
+    bool bad = false;
+    if ((c & 0x7Fu) != 0x7Fu) {
+        uint32_t w = c | ((c ^ 0x55u) << 8) | (c << 16) | ((c ^ 0x33u) << 24);
+        f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+        f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+        bad |= f2u(lo.x) != f2u(sw_e4m3fn_to_f32((uint8_t)c));
+        bad |= f2u(hi.x) != f2u(sw_e4m3fn_to_f32((uint8_t)c));
+        uint32_t c1 = c ^ 0x55u, c3 = c ^ 0x33u;
+        if ((c1 & 0x7Fu) != 0x7Fu) bad |= f2u(lo.y) != f2u(sw_e4m3fn_to_f32((uint8_t)c1));
+        if ((c3 & 0x7Fu) != 0x7Fu) bad |= f2u(hi.y) != f2u(sw_e4m3fn_to_f32((uint8_t)c3));
+    }
+    count(out, bad);
+}
+
+// which 2: packed fp32 -> bf16 over every non-NaN fp32
+__global__ __launch_bounds__(256) void st_cvt_bf16(uint64_t *out)
+{
+    const uint32_t base = (blockIdx.x * 256u + threadIdx.x) * 16u;
+    bool bad = false;
+    for (uint32_t i = 0; i < 16u; i += 2) {
+        uint32_t u0 = base + i, u1 = base + i + 1;
+        bool ok0 = (u0 & 0x7FFFFFFFu) <= 0x7F800000u, ok1 = (u1 & 0x7FFFFFFFu) <= 0x7F800000u;
+        uint32_t p = pack_bf16(ok0 ? u2f(u0) : 0.0f, ok1 ? u2f(u1) : 0.0f);
+        if (ok0) bad |= (p & 0xFFFFu) != sw_f32_to_bf16(u2f(u0));
+        if (ok1) bad |= (p >> 16) != sw_f32_to_bf16(u2f(u1));
+    }
+    count(out, bad);
+}
+
+// which 3: every packed byte in every byte position, scale operand 1.0
+__global__ __launch_bounds__(256) void st_cvt_fp4(uint64_t *out)
+{
+    const uint32_t b = threadIdx.x;
+    bool bad = false;
+    for (int pos = 0; pos < 4; ++pos) {
+        uint32_t w = (b << (8 * pos)) | (0xA5C3961Eu & ~(0xFFu << (8 * pos)));
+        float v[8];
+        fp4_decode8(w, v);
+        bad |= f2u(v[2 * pos]) != f2u(sw_e2m1_to_f32(b & 0xFu, true));
+        bad |= f2u(v[2 * pos + 1]) != f2u(sw_e2m1_to_f32(b >> 4, true));
+        float z[8];
+        fp4_decode8(fp4_pos_zero(w), z);
+        bad |= f2u(z[2 * pos]) != f2u(sw_e2m1_to_f32(b & 0xFu, false));
+        bad |= f2u(z[2 * pos + 1]) != f2u(sw_e2m1_to_f32(b >> 4, false));
+    }
+    count(out, bad);
+}
+
+__global__ __launch_bounds__(256) void debug_cast(int kind, const float *__restrict__ x, void *__restrict__ out, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        float v = x[i];
+        if (kind == 0) ((uint8_t *)out)[i] = sw_f32_to_e4m3fn(v);
+        else if (kind == 1) ((uint8_t *)out)[i] = (uint8_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v), 0.0f, 0, false);
+        else if (kind == 2) ((uint8_t *)out)[i] = f32_to_e8m0(v);
+        else ((uint16_t *)out)[i] = sw_f32_to_bf16(v);
+    }
+}
+
+}  // namespace
+
+extern "C" int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream)
+{
+    LP_REQUIRE(mismatches, "lp_selftest: null pointer");
+    LP_REQUIRE(which >= 0 && which <= 3, "lp_selftest: which must be 0..3");
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = hipMemsetAsync(mismatches, 0, sizeof(uint64_t), st);
+    if (e != hipSuccess) return fail(LP_ERR_HIP, "lp_selftest: %s", hipGetErrorString(e));
+    const unsigned all = (1u << 20);   // 2^20 workgroups x 256 threads x 16 patterns = 2^32
+    if (which == 0) hipLaunchKernelGGL(st_cvt_fp8, dim3(all), dim3(256), 0, st, mismatches);
+    else if (which == 1) hipLaunchKernelGGL(st_cvt_from_fp8, dim3(1), dim3(256), 0, st, mismatches);
+    else if (which == 2) hipLaunchKernelGGL(st_cvt_bf16, dim3(all), dim3(256), 0, st, mismatches);
+    else hipLaunchKernelGGL(st_cvt_fp4, dim3(1), dim3(256), 0, st, mismatches);
+    return check_launch("lp_selftest");
+}
+
+extern "C" int lp_debug_cast(int kind, const float *x, void *out, int64_t n, lp_stream_t stream)
+{
+    LP_REQUIRE(kind >= 0 && kind <= 3, "lp_debug_cast: kind must be 0..3");
+    LP_REQUIRE(n >= 0, "lp_debug_cast: negative length");
+    if (n == 0) return LP_OK;
+    LP_REQUIRE(x && out, "lp_debug_cast: null pointer");
+    unsigned wgs = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    hipLaunchKernelGGL(debug_cast, dim3(wgs), dim3(256), 0, (hipStream_t)stream, kind, x, out, n);
+    return check_launch("lp_debug_cast");
+}

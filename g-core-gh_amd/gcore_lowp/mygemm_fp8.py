@@ -1,0 +1,76 @@
+"""MI355X drop-in for gfused/mygemm_fp8.py: block-scaled FP8 GEMM and the plain NT GEMM.
+
+The reference functions are TileLang JIT kernels whose keyword arguments pick
+tile sizes; they are accepted here for signature compatibility and otherwise
+ignored (tiling is chosen by the HIP kernels).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _abi as A
+from . import ops
+
+__all__ = ["gemm_fp8_block_scaling_impl", "gemm_impl"]
+
+_workspace: dict = {}
+
+
+def _get_workspace(dev: torch.device, nbytes: int) -> torch.Tensor | None:
+    if nbytes <= 0:
+        return None
+    ws = _workspace.get(dev)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _workspace[dev] = ws
+    return ws
+
+
+def _scale_arg(s: torch.Tensor, dev) -> tuple[torch.Tensor, int]:
+    s = s.to(dev)
+    if s.dtype == ops.E8M0:
+        return s.contiguous(), A.E8M0
+    return s.to(torch.float32).contiguous(), A.F32
+
+
+def gemm_fp8_block_scaling_impl(Aq, As, Bq, Bs, BLK_M=64, BLK_N=128, BLK_K=128, FP8_BLK_SZ=128,
+                                dtype=torch.float8_e4m3fn, scale_dtype=torch.float8_e8m0fnu,
+                                out_dtype=torch.bfloat16, accum_dtype=torch.float32):
+    """gfused/mygemm_fp8.py:44-97.  Aq [M,K] e4m3fn, As [M,K/128], Bq [N,K] e4m3fn,
+    Bs [N/128,K/128] -> C [M,N] of out_dtype; the scales may be e8m0 or any real
+    float dtype (read as fp32)."""
+    assert max(BLK_N, FP8_BLK_SZ) % min(BLK_N, FP8_BLK_SZ) == 0
+    assert BLK_K == FP8_BLK_SZ
+    assert FP8_BLK_SZ == 128, "only 128-wide scale blocks are built"
+    assert dtype == torch.float8_e4m3fn and accum_dtype == torch.float32
+    assert Aq.dtype == torch.float8_e4m3fn and Bq.dtype == torch.float8_e4m3fn
+    assert Aq.ndim == 2 and Bq.ndim == 2 and Aq.shape[1] == Bq.shape[1]
+    M, K = Aq.shape
+    N = Bq.shape[0]
+    assert K % FP8_BLK_SZ == 0 and N % FP8_BLK_SZ == 0
+    assert tuple(As.shape) == (M, K // FP8_BLK_SZ), (tuple(As.shape), (M, K // FP8_BLK_SZ))
+    assert tuple(Bs.shape) == (N // FP8_BLK_SZ, K // FP8_BLK_SZ)
+    assert out_dtype in (torch.bfloat16, torch.float32)
+    a, home = A.to_device(Aq)
+    dev = a.device
+    a = a.contiguous()
+    b = Bq.to(dev).contiguous()
+    sa, ca = _scale_arg(As, dev)
+    sb, cb = _scale_arg(Bs, dev)
+    if ca != cb:
+        sa, sb, ca = sa.to(torch.float32), sb.to(torch.float32), A.F32
+    C = torch.empty((M, N), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        nws = A.lib().lp_gemm_workspace_bytes(M, N, K)
+        ws = _get_workspace(dev, nws)
+        A.check(A.lib().lp_gemm_fp8_block(
+            a.data_ptr(), sa.data_ptr(), b.data_ptr(), sb.data_ptr(), ca, M, N, K, C.data_ptr(),
+            A.BF16 if out_dtype == torch.bfloat16 else A.F32,
+            ws.data_ptr() if ws is not None else None, nws, A.stream_ptr()))
+    return C.to(home)
+
+
+def gemm_impl(A_, B_, block_M=128, block_N=128, block_K=64, dtype=torch.bfloat16, out_dtype=torch.bfloat16,
+              accum_dtype=torch.float32):
+    """gfused/mygemm_fp8.py:12-41: C = A B^T, fp8 or bf16 operands, fp32 accumulation."""
+    raise A.LowpError("gemm_impl: the unscaled GEMM is not built yet")

@@ -1,0 +1,196 @@
+/*
+ * lowp -- C ABI of the MI355X (gfx950) low-precision weight / GEMM path.
+ *
+ * One shared library, plain pointers and sizes.  Every pointer marked "device"
+ * must be device memory on the GPU that is current on the calling thread; all
+ * work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ * default stream) and the call returns without waiting.  The caller owns and
+ * allocates every buffer.  Return value: 0 on success, a negative lp_status
+ * otherwise, with a message available from lp_last_error() (thread local).
+ * Arguments are validated on the host before anything is launched.
+ *
+ * File:line citations name the reference (Tencent/G-Core-GH) interface that an
+ * entry point stands in for.
+ */
+#ifndef LOWP_H
+#define LOWP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *lp_stream_t;
+
+enum lp_status {
+    LP_OK = 0,
+    LP_ERR_INVALID = -1,      /* bad shape / dtype / null pointer            */
+    LP_ERR_UNSUPPORTED = -2,  /* valid request this build has no kernel for */
+    LP_ERR_HIP = -3           /* the HIP runtime reported an error           */
+};
+
+enum lp_dtype {
+    LP_F32 = 0,
+    LP_BF16 = 1,
+    LP_E8M0 = 2,   /* float8_e8m0fnu: one byte, value 2^(b-127)            */
+    LP_E4M3 = 3    /* float8_e4m3fn (OCP)                                   */
+};
+
+/* How the per-block scale is derived from the block's amax. */
+enum lp_scale_mode {
+    /* s = 2^ceil(log2(max(amax, FLT_MIN)/448)), q = cast(clamp(x / s));
+     * gpatch_v4/kernel/quantize/eager_quant_kernels.py:132-181 */
+    LP_SCALE_POW2 = 0,
+    /* s = max(amax, amax_floor)/448, q = cast(clamp(x / s));
+     * tests/test_gfused/test_te_gemm_fp8.py:82-101,
+     * tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:29-72 */
+    LP_SCALE_DIV = 1,
+    /* f = fl(fl(1/amax) * 448), q = cast(clamp(x * f)), stored scale = fl(1/f);
+     * tools/convert_fp8/qwen3_5/qwen3_mtp_fp8_postprocess.py:138-149 */
+    LP_SCALE_MUL = 2
+};
+
+enum lp_zero_rule {
+    LP_ZERO_NONE = 0,          /* no special case                              */
+    LP_ZERO_AMAX_TO_ONE = 1,   /* amax == 0      -> scale 1                    */
+    LP_ZERO_SCALE_TO_ONE = 2   /* computed s == 0 -> scale 1                   */
+};
+
+/* Table flavour for FP4 code 8: */
+enum lp_fp4_zero {
+    LP_FP4_POS_ZERO = 0,  /* +0.0: tools/convert_deepseek_v4_fp4_to_bf16.py:15-18,
+                             tools/dsv4_quant_and_dequant/kernels.py:46-66      */
+    LP_FP4_NEG_ZERO = 1   /* -0.0: gpatch_v4/kernel/quantize/eager_quant_kernels.py:56-58 */
+};
+
+int lp_version(void);
+const char *lp_last_error(void);
+
+/*
+ * Block quantiser to e4m3fn.  x: device, [rows, cols] row-major, LP_BF16 or
+ * LP_F32 (leading dims of the reference's [..., M, N] are folded into rows).
+ * One scale per bm x bn block; rows % bm == 0, cols % bn == 0.
+ * q_out: device u8 [rows, cols].  scale_out: device [rows/bm, cols/bn] of
+ * scale_dtype (LP_F32, LP_BF16 or LP_E8M0).  nan_count: optional device
+ * int32 that is incremented once per block that holds a NaN (caller zeroes it).
+ * Replaces quant_fp8_e4m3_scale_e8m0 (eager_quant_kernels.py:132-181),
+ * quantize_fp8_blockwise (qwen3_mtp_fp8_postprocess.py:102-151) and the
+ * 1 x 128 / 128 x 128 fp32-scale quantisers used around the GEMM
+ * (test_te_gemm_fp8.py:82-101, test_deep_gemm_grouped_gemm_fp8.py:29-72).
+ */
+int lp_quant_fp8_block(const void *x, int x_dtype, int64_t rows, int64_t cols, int bm, int bn,
+                       int scale_mode, float amax_floor, int zero_rule,
+                       void *q_out, void *scale_out, int scale_dtype,
+                       int32_t *nan_count, lp_stream_t stream);
+
+/*
+ * Block dequantiser: out = cast(fl32(fl32(code) * fl32(scale))).
+ * q: device [rows, cols] e4m3fn bytes (q_dtype LP_E4M3).  scale: device
+ * [rows/bm, cols/bn] of scale_dtype.  out: device [rows, cols], LP_BF16 or LP_F32.
+ * Replaces the FP8 branch of dequant_fp4_e2m1_fp8_scale_e8m0_packed
+ * (eager_quant_kernels.py:200-233) and cast_e4m3fn_to_bf16
+ * (tools/convert_deepseek_v4_fp4_to_bf16.py:51-63).
+ */
+int lp_dequant_fp8_block(const void *q, const void *scale, int scale_dtype,
+                         int64_t rows, int64_t cols, int bm, int bn,
+                         void *out, int out_dtype, lp_stream_t stream);
+
+/*
+ * Packed FP4 (e2m1, two codes per byte, low nibble = even column) with one
+ * scale per bm x bn block of logical elements -> bf16 / fp32.
+ * packed: device u8 [rows, cols/2]; scale: device [rows/bm, cols/bn] of
+ * scale_dtype; out: device [rows, cols].
+ * Replaces cast_e2m1fn_to_bf16 (tools/convert_deepseek_v4_fp4_to_bf16.py:24-46;
+ * bm=1, bn=32, LP_E8M0, LP_FP4_POS_ZERO) and the FP4 branch of
+ * dequant_fp4_e2m1_fp8_scale_e8m0_packed (eager_quant_kernels.py:190-233;
+ * LP_FP4_NEG_ZERO).
+ */
+int lp_dequant_fp4_block(const void *packed, const void *scale, int scale_dtype,
+                         int64_t rows, int64_t cols, int bm, int bn, int fp4_zero,
+                         void *out, int out_dtype, lp_stream_t stream);
+
+/*
+ * Lossless FP4 (1 x 32 e8m0 scales) -> e4m3fn with one 128 x 128 outer scale
+ * = (max e8m0 scale of the tile) / 64; no clamp.
+ * packed: device u8 [rows, cols/2]; scale: device u8 (e8m0) [rows, cols/32];
+ * q_out: device u8 [rows, cols]; scale_out: device [rows/128, cols/128] of
+ * scale_dtype (LP_E8M0 or LP_F32).
+ * Replaces cast_e2m1fn_to_e4m3fn / official_expert_to_sgl
+ * (tools/dsv4_quant_and_dequant/kernels.py:91-133).
+ */
+int lp_fp4_to_fp8_rebase(const void *packed, const void *scale, int64_t rows, int64_t cols,
+                         void *q_out, void *scale_out, int scale_dtype, lp_stream_t stream);
+
+/*
+ * Fused FP4 (1 x 32 e8m0) -> bf16 -> e4m3fn with a 128 x 128 fp32 scale: the
+ * result is byte-identical to lp_dequant_fp4_block (bf16, LP_FP4_POS_ZERO)
+ * followed by lp_quant_fp8_block on 128 x 128 blocks with the given scale
+ * mode, without the bf16 tensor touching HBM unless bf16_out is non-NULL.
+ * Stands in for running tools/convert_deepseek_v4_fp4_to_bf16.py:24-46 and then
+ * the tools/convert_fp8 quantiser.
+ */
+int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t rows, int64_t cols,
+                       int scale_mode, float amax_floor, int zero_rule,
+                       void *q_out, void *scale_out, int scale_dtype, void *bf16_out,
+                       lp_stream_t stream);
+
+/*
+ * Block-scaled FP8 GEMM: C[i,j] = cast(sum_kb (sum_{k in kb} Aq[i,k] Bq[j,k]) * As[i,kb] * Bs[j/128,kb]).
+ * Aq: device e4m3fn [M,K]; As: device [M,K/128]; Bq: device e4m3fn [N,K];
+ * Bs: device [N/128,K/128]; scales of scale_dtype (LP_F32 or LP_E8M0);
+ * C: device [M,N] LP_BF16 or LP_F32.  K % 128 == 0, N % 128 == 0, any M.
+ * workspace: optional device scratch of at least lp_gemm_workspace_bytes(M,N,K)
+ * bytes (16-byte aligned); with it, problems with few output tiles split K
+ * across workgroups (fixed summation order).  NULL / too small = no split.
+ * Replaces gemm_fp8_block_scaling_impl (gfused/mygemm_fp8.py:44-97).
+ */
+int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                      int64_t M, int64_t N, int64_t K, void *C, int out_dtype,
+                      void *workspace, int64_t workspace_bytes, lp_stream_t stream);
+
+/* Scratch bytes lp_gemm_fp8_block can use for this shape (0 = none needed). */
+int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Unscaled C = A B^T with fp32 accumulation.  A [M,K], B [N,K], both of
+ * in_dtype (LP_E4M3 or LP_BF16); C [M,N] of out_dtype (LP_E4M3, LP_BF16, LP_F32).
+ * Replaces gemm_impl (gfused/mygemm_fp8.py:12-41).
+ */
+int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M, int64_t N, int64_t K,
+               void *C, int out_dtype, lp_stream_t stream);
+
+/*
+ * Grouped block-scaled FP8 GEMM for MoE experts.  Rows of Aq are sorted by
+ * expert; expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 (zero rows
+ * allowed).  Aq [M_total,K], As [M_total,K/128], Bq [E,N,K], Bs [E,N/128,K/128],
+ * C [M_total,N].  m_offsets: device int32 [E+1], non-decreasing, m_offsets[0]=0.
+ * Rows at or beyond m_offsets[E] are left untouched.
+ * Replaces MyTeGroupedLinearFp8.forward (gpatch_v4/models/deepseek_v4/fp8.py:346-394)
+ * and the DeepGEMM-style contiguous grouped GEMM called at
+ * tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:106-109.
+ */
+int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                        const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K,
+                        void *C, int out_dtype, lp_stream_t stream);
+
+/*
+ * On-device self tests of the gfx950 conversion instructions against the
+ * library's software casts.  Each writes the number of mismatching inputs to
+ * *mismatches (device uint64, zeroed by the call).  No reference counterpart.
+ *   which = 0: v_cvt_pk_fp8_f32 over every fp32 with |x| <= 448 (and +-0)
+ *   which = 1: v_cvt_pk_f32_fp8 over all 256 codes except the two NaNs
+ *   which = 2: fp32 -> bf16 conversion over every non-NaN fp32
+ *   which = 3: v_cvt_scalef32_pk_f32_fp4 over 256 bytes x the scale exponents used
+ */
+int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream);
+
+/* Bulk element-wise casts through the library's device code paths (debug aid
+ * for tests): kind 0 = fp32 -> e4m3fn software, 1 = fp32 -> e4m3fn hardware
+ * (inputs clamped to +-448 first), 2 = fp32 -> e8m0, 3 = fp32 -> bf16. */
+int lp_debug_cast(int kind, const float *x, void *out, int64_t n, lp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LOWP_H */

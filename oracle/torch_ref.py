@@ -1,0 +1,231 @@
+"""Eager-PyTorch CPU oracle for the low-precision weight / GEMM path.
+
+TEST INFRASTRUCTURE ONLY.  This module restates, op for op, the arithmetic the
+reference performs with eager torch ops, so that it (a) serves as the checker
+in parity tests and (b) stands in for "the reference's PyTorch CPU path" in the
+benchmark's cpu-baseline leg.  The product package never imports it.
+
+Each function names the reference lines it follows.  What pins each one
+independently of its own formula is listed in oracle/lowp_oracle.c's header;
+the tests additionally require this module and the scalar C oracle -- two
+independent restatements -- to agree byte for byte.
+"""
+from __future__ import annotations
+
+import torch
+
+E4M3_MAX = 448.0
+_E4M3 = torch.float8_e4m3fn
+_E8M0 = torch.float8_e8m0fnu
+
+# e2m1 code point -> value; index 8 differs between the two reference tables.
+_MAG = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
+LUT_NEG_ZERO = torch.tensor(_MAG + tuple(-m for m in _MAG), dtype=torch.float32)  # eager_quant_kernels.py:56-58
+LUT_POS_ZERO = LUT_NEG_ZERO.clone()                                                # convert_deepseek_v4_fp4_to_bf16.py:15-18
+LUT_POS_ZERO[8] = 0.0
+
+
+def _tiles(v: torch.Tensor, bm: int, bn: int) -> torch.Tensor:
+    """[..., M, N] -> [..., M/bm, bm, N/bn, bn] view."""
+    *lead, m, n = v.shape
+    return v.reshape(*lead, m // bm, bm, n // bn, bn)
+
+
+def _tile_amax(t: torch.Tensor) -> torch.Tensor:
+    return t.abs().amax(dim=(-3, -1))
+
+
+def _bcast(s: torch.Tensor) -> torch.Tensor:
+    return s.unsqueeze(-1).unsqueeze(-3)
+
+
+def _to_e4m3_clamped(t: torch.Tensor) -> torch.Tensor:
+    return t.clamp(min=-E4M3_MAX, max=E4M3_MAX).to(_E4M3)
+
+
+# --------------------------------------------------------------------- a1
+
+def quant_fp8_e4m3_scale_e8m0(value: torch.Tensor, block_size=(128, 128)):
+    """gpatch_v4/kernel/quantize/eager_quant_kernels.py:132-181."""
+    m, n = value.shape[-2:]
+    bm, bn = block_size
+    assert m % bm == 0 and n % bn == 0, f"value shape ({m}, {n}) not divisible by block ({bm}, {bn})"
+    assert not torch.isnan(value).any(), "quant_fp8_e4m3_scale_e8m0: input contains NaN"
+    t = _tiles(value.float(), bm, bn)
+    amax = _tile_amax(t)
+    r = amax.clamp(min=torch.finfo(torch.float32).tiny) / E4M3_MAX
+    s = torch.pow(2.0, torch.ceil(torch.log2(r)))
+    s = torch.where(amax > 0, s, torch.ones_like(s))
+    q = _to_e4m3_clamped(t / _bcast(s)).reshape(value.shape).contiguous()
+    return q, s.to(_E8M0)
+
+
+# --------------------------------------------------------------------- a2
+
+def quantize_fp8_blockwise(weight: torch.Tensor, block_size, *, device=None, scale_dtype=torch.bfloat16):
+    """tools/convert_fp8/qwen3_5/qwen3_mtp_fp8_postprocess.py:102-151 (multiply form)."""
+    if weight.ndim != 2:
+        raise ValueError(f"Expected a 2D weight, got shape={tuple(weight.shape)}")
+    bm, bn = block_size
+    rows, cols = weight.shape
+    if rows % bm or cols % bn:
+        raise ValueError(f"Matrix dimensions ({rows}, {cols}) must be divisible by block sizes ({bm}, {bn})")
+    t = _tiles(weight.to(dtype=torch.float32), bm, bn)
+    amax = t.abs().amax(dim=(1, 3))
+    one = torch.ones_like(amax)
+    f = E4M3_MAX / torch.where(amax > 0, amax, one)
+    f = torch.where(amax > 0, f, one)
+    q = _to_e4m3_clamped(t * f[:, None, :, None]).reshape(rows, cols)
+    return q, (1.0 / f).to(scale_dtype)
+
+
+# ---------------------------------------------------------------- a3 / a4
+
+def quant_block_fp32_scale(x: torch.Tensor, block_size, *, amax_floor=1e-12, zero_scale_to_one=False):
+    """Divide form with an fp32 scale = amax/448.
+
+    amax_floor=1e-12: tests/test_gfused/test_te_gemm_fp8.py:82-101,
+    tests/test_gfused/test_deepseek_tilekernels_quant.py:22-58.
+    amax_floor=None, zero_scale_to_one=True:
+    tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:29-72.
+    Works for 1 x 128 activation groups and 128 x 128 weight tiles alike.
+    """
+    bm, bn = block_size
+    t = _tiles(x.float(), bm, bn)
+    amax = _tile_amax(t)
+    if amax_floor is not None:
+        amax = amax.clamp(min=amax_floor)
+    s = amax / E4M3_MAX
+    if zero_scale_to_one:
+        s = torch.where(s == 0, torch.ones_like(s), s)
+    q = _to_e4m3_clamped(t / _bcast(s)).reshape(x.shape).contiguous()
+    return q, s.to(torch.float32)
+
+
+def quant_block_pow2_scale(x: torch.Tensor, block_size, *, amax_floor=1e-12):
+    """round_sf=True branch of tests/test_gfused/test_deepseek_tilekernels_quant.py:22-58."""
+    bm, bn = block_size
+    t = _tiles(x.float(), bm, bn)
+    amax = _tile_amax(t).clamp(min=amax_floor)
+    s = torch.pow(2.0, torch.ceil(torch.log2(amax / E4M3_MAX)))
+    q = _to_e4m3_clamped(t / _bcast(s)).reshape(x.shape).contiguous()
+    return q, s
+
+
+# ---------------------------------------------------------------- a5 / a6
+
+def unpack_fp4(packed: torch.Tensor, lut: torch.Tensor) -> torch.Tensor:
+    """Low nibble -> even column, high nibble -> odd column
+    (eager_quant_kernels.py:190-197)."""
+    b = packed.contiguous().view(torch.uint8)
+    lo = (b & 0xF).long()
+    hi = ((b >> 4) & 0xF).long()
+    return torch.stack((lut[lo], lut[hi]), dim=-1).reshape(*packed.shape[:-1], 2 * packed.shape[-1])
+
+
+def dequant_fp4_e2m1_fp8_scale_e8m0_packed(quantized: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """eager_quant_kernels.py:200-233: block = shape ratio, fp32 product, result in
+    scales.dtype when that is a float of >= 2 bytes, else bf16."""
+    fp4x2 = getattr(torch, "float4_e2m1fn_x2", None)
+    if quantized.dtype == torch.int8 or (fp4x2 is not None and quantized.dtype == fp4x2):
+        qf = unpack_fp4(quantized, LUT_NEG_ZERO)
+    else:
+        qf = quantized.to(torch.float32)
+    rows, cols = qf.shape[-2:]
+    sr, sc = scales.shape[-2:]
+    if rows % sr or cols % sc:
+        raise ValueError(f"Weight shape ({rows}, {cols}) not divisible by scale grid ({sr}, {sc}).")
+    out_dtype = scales.dtype if scales.dtype.is_floating_point and scales.element_size() >= 2 else torch.bfloat16
+    t = qf.reshape(-1, sr, rows // sr, sc, cols // sc)
+    s = scales.to(torch.float32).reshape(-1, sr, sc)[:, :, None, :, None]
+    return (t * s).to(out_dtype).reshape(qf.shape)
+
+
+def cast_e4m3fn_to_bf16(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """tools/convert_deepseek_v4_fp4_to_bf16.py:51-63."""
+    assert x.dtype == _E4M3 and x.ndim == 2
+    o, i = x.shape
+    assert o % 128 == 0 and i % 128 == 0
+    assert tuple(scale.shape) == (o // 128, i // 128)
+    s = scale.float().repeat_interleave(128, 0).repeat_interleave(128, 1)
+    return (x.float() * s).bfloat16()
+
+
+# --------------------------------------------------------------------- a7
+
+def cast_e2m1fn_to_bf16(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """tools/convert_deepseek_v4_fp4_to_bf16.py:24-46."""
+    assert x.dtype == torch.int8 and x.ndim == 2
+    o, half = x.shape
+    i = half * 2
+    assert i % 32 == 0
+    assert scale.size(0) == o and scale.size(1) == i // 32
+    v = unpack_fp4(x, LUT_POS_ZERO)
+    return (v * scale.float().repeat_interleave(32, dim=-1)).bfloat16()
+
+
+# --------------------------------------------------------------------- a8
+
+def cast_e2m1fn_to_e4m3fn(x: torch.Tensor, scale: torch.Tensor):
+    """tools/dsv4_quant_and_dequant/kernels.py:91-126."""
+    assert x.dtype == torch.int8 and x.ndim == 2
+    o, half = x.shape
+    i = half * 2
+    assert i % 128 == 0 and o % 128 == 0
+    assert scale.size(0) == o and scale.size(1) == i // 32
+    v = unpack_fp4(x, LUT_POS_ZERO)                                    # [o, i]
+    bo, bi = o // 128, i // 128
+    vt = v.view(bo, 128, bi, 128).transpose(1, 2)                      # [bo, bi, 128, 128]
+    st = scale.float().view(bo, 128, bi, 4).transpose(1, 2).flatten(2)  # [bo, bi, 512]
+    outer = st.amax(dim=-1, keepdim=True) / 64.0
+    off = (st / outer).unflatten(-1, (128, 4)).repeat_interleave(32, dim=-1)
+    y = (vt * off).transpose(1, 2).reshape(o, i)
+    return y.to(_E4M3), outer.squeeze(-1).to(_E8M0)
+
+
+def official_expert_to_sgl(weight: torch.Tensor, scale: torch.Tensor):
+    """tools/dsv4_quant_and_dequant/kernels.py:129-133."""
+    q, s = cast_e2m1fn_to_e4m3fn(weight, scale)
+    return q, s.float().contiguous()
+
+
+# --------------------------------------------------------------------- a9
+
+def fp4_to_fp8_amax(x: torch.Tensor, scale: torch.Tensor, *, amax_floor=1e-12, zero_scale_to_one=False):
+    """FP4 -> bf16 -> e4m3fn with a 128 x 128 fp32 scale = amax/448: the two-step
+    composition cast_e2m1fn_to_bf16 followed by the divide-form block quantiser."""
+    w = cast_e2m1fn_to_bf16(x, scale)
+    return quant_block_fp32_scale(w, (128, 128), amax_floor=amax_floor, zero_scale_to_one=zero_scale_to_one)
+
+
+# -------------------------------------------------------------- a10 - a12
+
+def dequant_act_f32(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+    m, k = q.shape
+    return (q.float().reshape(m, k // 128, 128) * s.float().unsqueeze(-1)).reshape(m, k)
+
+
+def dequant_weight_f32(q: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+    *lead, n, k = q.shape
+    t = q.float().reshape(*lead, n // 128, 128, k // 128, 128)
+    return (t * s.float().unsqueeze(-1).unsqueeze(-3)).reshape(q.shape)
+
+
+def gemm_fp8_block_scaling_ref(Aq, As, Bq, Bs) -> torch.Tensor:
+    """fp32 dequant then fp32 matmul: the numeric reference of gfused/mygemm_fp8.py:44-97
+    (tests/test_gfused/test_my_gemm_fp8.py:176-186 does the same in bf16)."""
+    return dequant_act_f32(Aq, As) @ dequant_weight_f32(Bq, Bs).T
+
+
+def grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits) -> torch.Tensor:
+    """tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:75-89 with rows given
+    as consecutive per-expert counts."""
+    x = dequant_act_f32(xq, xs)
+    w = dequant_weight_f32(wq, ws)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.float32)
+    r = 0
+    for e, cnt in enumerate(m_splits):
+        if cnt:
+            out[r:r + cnt] = x[r:r + cnt] @ w[e].T
+        r += cnt
+    return out

@@ -1,0 +1,88 @@
+"""The C-ABI library loads without a GPU, exports every symbol include/lowp.h declares,
+and rejects bad arguments on the host before anything is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from gcore_lowp import _abi
+    if not os.path.exists(_abi.LIB_PATH):
+        pytest.fail(f"{_abi.LIB_PATH} missing: run `python g-core-gh_amd/build.py`")
+    return _abi
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "lowp.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    names = _declared()
+    assert len(names) >= 12
+    L = lib.lib()
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/lowp.h but not exported"
+        assert n in lib.PROTOTYPES, f"{n} has no ctypes prototype"
+    assert sorted(lib.PROTOTYPES) == names
+    assert L.lp_version() >= 100
+
+
+def test_host_side_validation(lib):
+    L = lib.lib()
+    one = ctypes.c_void_p(16)       # never dereferenced: validation fails first
+    # shape not divisible by the block
+    rc = L.lp_quant_fp8_block(one, lib.BF16, 100, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, one, one, lib.F32, None, None)
+    assert rc == -1 and "not divisible" in lib.last_error()
+    rc = L.lp_quant_fp8_block(one, 7, 128, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, one, one, lib.F32, None, None)
+    assert rc == -1 and "x_dtype" in lib.last_error()
+    rc = L.lp_quant_fp8_block(None, lib.BF16, 128, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, one, one, lib.F32, None, None)
+    assert rc == -1 and "null" in lib.last_error()
+    rc = L.lp_dequant_fp8_block(one, one, lib.F32, 128, 100, 128, 128, one, lib.BF16, None)
+    assert rc == -1 and "not divisible" in lib.last_error()
+    rc = L.lp_fp4_to_fp8_rebase(one, one, 128, 64, one, one, lib.E8M0, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
+    rc = L.lp_gemm_fp8_block(one, one, one, one, lib.F32, 64, 128, 100, one, lib.BF16, None, 0, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
+    rc = L.lp_gemm_fp8_grouped(one, one, one, one, lib.F32, None, 4, 64, 128, 128, one, lib.BF16, None)
+    assert rc == -1 and "m_offsets" in lib.last_error()
+    # empty problems succeed without touching the device
+    assert L.lp_quant_fp8_block(None, lib.BF16, 0, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, None, None, lib.F32, None, None) == 0
+    assert L.lp_gemm_fp8_block(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None, 0, None) == 0
+
+
+def test_wrappers_keep_reference_exceptions(lib):
+    """Shape / dtype errors are raised as the reference raises them, before any GPU work."""
+    import torch
+    import gcore_lowp as G
+
+    with pytest.raises(AssertionError):
+        G.quant_fp8_e4m3_scale_e8m0(torch.zeros(100, 128), (128, 128))
+    with pytest.raises(ValueError):
+        G.quantize_fp8_blockwise(torch.zeros(2, 128, 128), (128, 128))
+    with pytest.raises(ValueError):
+        G.quantize_fp8_blockwise(torch.zeros(100, 128), (128, 128))
+    with pytest.raises(AssertionError):
+        G.cast_e2m1fn_to_bf16(torch.zeros(4, 16, dtype=torch.uint8), torch.zeros(4, 1))
+    with pytest.raises(AssertionError):
+        G.cast_e4m3fn_to_bf16(torch.zeros(128, 128).to(torch.float8_e4m3fn), torch.zeros(2, 1))
+    with pytest.raises(AssertionError):
+        G.cast_e2m1fn_to_e4m3fn(torch.zeros(128, 32, dtype=torch.int8), torch.zeros(128, 2))
+    with pytest.raises(AssertionError):
+        G.gemm_fp8_block_scaling_impl(torch.zeros(4, 128).to(torch.float8_e4m3fn), torch.zeros(4, 2),
+                                      torch.zeros(128, 128).to(torch.float8_e4m3fn), torch.zeros(1, 1))
+
+
+@pytest.mark.skipif(__import__("torch").cuda.is_available(), reason="GPU present")
+def test_no_cpu_fallback_without_gpu(lib):
+    import torch
+    import gcore_lowp as G
+
+    with pytest.raises(lib.LowpError, match="no GPU"):
+        G.quant_2d(torch.zeros(128, 128, dtype=torch.bfloat16))

@@ -1,0 +1,165 @@
+"""GPU parity of the block-scaled FP8 GEMMs against fp32 dequant-then-matmul.
+
+Bars: max relative error <= 2e-2 (relative to the largest |reference| entry) and cosine
+>= 0.9999, plus the reference's own bars: avg_abs < 1e-2 * scale, calc_diff < 1e-5
+(tests/test_gfused/test_my_gemm_fp8.py:239-243), cos > 0.999 and max_err < 1.0
+(tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:118-119).
+"""
+import pytest
+import torch
+
+from oracle import torch_ref as T
+from tests import _inputs as I
+
+pytestmark = pytest.mark.gpu
+
+E4M3, E8M0 = torch.float8_e4m3fn, torch.float8_e8m0fnu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gcore_lowp
+    return gcore_lowp
+
+
+def calc_diff(x, y):
+    x, y = x.double(), y.double()
+    return float(1 - 2 * (x * y).sum() / (x * x + y * y).sum())
+
+
+def check(out, ref, what):
+    out, ref = out.float().cpu(), ref.float().cpu()
+    assert torch.isfinite(out).all(), what
+    denom = ref.abs().max().item()
+    max_rel = ((out - ref).abs().max().item()) / max(denom, 1e-30)
+    cos = torch.nn.functional.cosine_similarity(out.flatten().double(), ref.flatten().double(), dim=0).item()
+    cd = calc_diff(out, ref)
+    print(f"    {what}: max_rel={max_rel:.3e} cos={cos:.7f} calc_diff={cd:.3e}", flush=True)
+    assert max_rel <= 2e-2, (what, max_rel)
+    assert cos >= 0.9999, (what, cos)
+    assert cd < 1e-5, (what, cd)
+
+
+def quantized_problem(M, N, K, seed, pow2=False):
+    x = I.act_like(M, K, seed)
+    w = I.weight_like(N, K, seed + 1, outliers=False)
+    if pow2:
+        xq, xs = T.quant_fp8_e4m3_scale_e8m0(x, (1, 128))
+        wq, ws = T.quant_fp8_e4m3_scale_e8m0(w, (128, 128))
+    else:
+        xq, xs = T.quant_block_fp32_scale(x, (1, 128))
+        wq, ws = T.quant_block_fp32_scale(w, (128, 128))
+    return xq, xs, wq, ws
+
+
+def ref_gemm(xq, xs, wq, ws):
+    # fp32 dequant then matmul, on the GPU for speed (fp32 accumulate, no TF32 on ROCm)
+    a = T.dequant_act_f32(xq.cuda(), xs.float().cuda())
+    b = T.dequant_weight_f32(wq.cuda(), ws.float().cuda())
+    return (a.double() @ b.double().T).float() if a.numel() * b.shape[0] < 2 ** 27 else a @ b.T
+
+
+DENSE_SHAPES = [
+    (128, 128, 128), (128, 256, 256), (256, 128, 512), (64, 4096, 7168), (1, 128, 128), (7, 256, 384),
+    (200, 384, 1024), (512, 1024, 2048), (2048, 4096, 7168), (128, 4096, 4096), (1024, 4096, 1024),
+    (333, 640, 896),
+]
+
+
+@pytest.mark.parametrize("shape", DENSE_SHAPES, ids=lambda s: "M%d_N%d_K%d" % s)
+@pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
+def test_gemm_dense(G, shape, pow2):
+    M, N, K = shape
+    xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + N + K, pow2=pow2)
+    say("gemm dense", shape, "pow2" if pow2 else "f32")
+    out = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N)
+    check(out, ref_gemm(xq, xs, wq, ws), f"dense {shape}")
+
+
+def test_gemm_small_exact_vs_c_oracle(G, corc):
+    """Small case against the double-precision scalar oracle, fp32 output: catches scale indexing
+    (As[i, kb], Bs[j // 128, kb]) with distinct scales per block."""
+    torch.manual_seed(0)
+    M, N, K = 70, 256, 384
+    aq = (torch.randn(M, K) * 40).to(E4M3)
+    bq = (torch.randn(N, K) * 40).to(E4M3)
+    a_s = torch.rand(M, K // 128) * 2 + 0.25
+    b_s = torch.rand(N // 128, K // 128) * 2 + 0.25
+    say("gemm small vs C oracle")
+    out = G.gemm_fp8_block_scaling_impl(aq.cuda(), a_s.cuda(), bq.cuda(), b_s.cuda(), out_dtype=torch.float32)
+    want = torch.from_numpy(corc.gemm_fp8_block(aq.view(torch.uint8).numpy(), a_s.numpy(),
+                                                bq.view(torch.uint8).numpy(), b_s.numpy()))
+    assert torch.allclose(out.cpu(), want, rtol=1e-5, atol=want.abs().max().item() * 1e-6)
+
+
+def test_gemm_cpu_inputs_round_trip(G):
+    xq, xs, wq, ws = quantized_problem(64, 128, 256, 3)
+    say("gemm CPU inputs")
+    out = G.gemm_fp8_block_scaling_impl(xq, xs, wq, ws)
+    assert not out.is_cuda
+    check(out, ref_gemm(xq, xs, wq, ws), "cpu-in")
+
+
+def _grouped_problem(E, N, K, m_splits, seed):
+    M = sum(m_splits)
+    x = I.act_like(max(M, 1), K, seed)[:M]
+    g = torch.Generator().manual_seed(seed + 1)
+    w = (torch.randn(E, N, K, generator=g) * 0.02).to(torch.bfloat16)
+    xq, xs = T.quant_block_fp32_scale(x, (1, 128), amax_floor=None, zero_scale_to_one=True)
+    wq, ws = T.quant_block_fp32_scale(w, (128, 128), amax_floor=None, zero_scale_to_one=True)
+    return xq, xs, wq, ws
+
+
+GROUPED = [
+    (8, 256, 512, [256] * 8),
+    (16, 512, 1024, [128] * 16),
+    (4, 2048, 7168, [256] * 4),
+    (6, 256, 256, [0, 5, 130, 0, 257, 1]),
+    (5, 128, 384, [0, 0, 0, 0, 0]),
+    (3, 384, 512, [300, 0, 77]),
+    (300, 128, 128, [i % 7 for i in range(300)]),
+]
+
+
+@pytest.mark.parametrize("case", GROUPED, ids=lambda c: "E%d_N%d_K%d" % c[:3])
+def test_gemm_grouped(G, case):
+    E, N, K, m_splits = case
+    xq, xs, wq, ws = _grouped_problem(E, N, K, m_splits, seed=E + N)
+    M = sum(m_splits)
+    say("gemm grouped", E, N, K, "M=", M)
+    offs = torch.zeros(E + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+    out = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda())
+    assert tuple(out.shape) == (M, N) and out.dtype == torch.bfloat16
+    if M == 0:
+        return
+    ref = T.grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits)
+    check(out, ref, f"grouped {case[:3]}")
+    assert (out.float().cpu() - ref).abs().max().item() < 1.0
+    say("deepgemm-style call")
+    m_indices = torch.repeat_interleave(torch.arange(E), torch.tensor(m_splits)).to(torch.int32)
+    out2 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    G.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((xq.cuda(), xs.cuda()), (wq.cuda(), ws.cuda()), out2, m_indices.cuda())
+    assert torch.equal(out2, out)
+
+
+def test_grouped_linear_module(G):
+    E, N, K = 4, 256, 512
+    m_splits = [100, 0, 31, 200]
+    x = I.act_like(sum(m_splits), K, 5).cuda()
+    w = (torch.randn(E, N, K, generator=torch.Generator().manual_seed(6)) * 0.02).to(torch.bfloat16).cuda()
+    say("MyTeGroupedLinearFp8 bf16 weights")
+    lin = G.MyTeGroupedLinearFp8(E)
+    out = lin(x, w, m_splits)
+    ref = torch.cat([x[sum(m_splits[:e]):sum(m_splits[:e + 1])].float() @ w[e].float().T for e in range(E)])
+    rel = (out.float() - ref).norm() / ref.norm()
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (sum(m_splits), N) and rel.item() < 0.05
+    say("MyTeGroupedLinearFp8 pre-quantised weights")
+    wq, ws = G.quant_fp8_e4m3_scale_e8m0(w)
+    out2 = lin(x, (wq, ws), m_splits)
+    assert torch.equal(out2, out)

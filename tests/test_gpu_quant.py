@@ -1,0 +1,298 @@
+"""GPU parity: HIP quantise / dequantise / FP4 kernels vs the CPU oracles, bit for bit.
+
+Every case prints its name before touching the GPU so that a fault names its case.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import torch_ref as T
+from tests import _inputs as I
+
+pytestmark = pytest.mark.gpu
+
+E4M3, E8M0 = torch.float8_e4m3fn, torch.float8_e8m0fnu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def u8(t):
+    return t.detach().cpu().contiguous().view(torch.uint8)
+
+
+def bits_equal(a, b):
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    assert a.dtype == b.dtype and a.shape == b.shape, (a.dtype, b.dtype, a.shape, b.shape)
+    return torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gcore_lowp
+    return gcore_lowp
+
+
+@pytest.mark.parametrize("which", [0, 1, 2, 3])
+def test_hardware_conversions_match_software(G, which):
+    """v_cvt_pk_fp8_f32 over all |x| <= 448, v_cvt_pk_f32_fp8 over all codes, fp32->bf16 over all
+    non-NaN fp32, e2m1 decode over all bytes: zero mismatches against the library's software casts."""
+    from gcore_lowp import ops
+    say("selftest", which)
+    assert ops.selftest(which) == 0
+
+
+def test_software_casts_match_oracle(G, corc):
+    from gcore_lowp import ops
+    rng = np.random.default_rng(1)
+    u = np.concatenate([np.arange(0, 1 << 32, 1 << 10, dtype=np.uint64).astype(np.uint32),
+                        rng.integers(0, 1 << 32, 1 << 22, dtype=np.uint64).astype(np.uint32)])
+    f = torch.from_numpy(u.view(np.float32).copy())
+    isnan = np.isnan(f.numpy())
+    say("debug_cast e4m3 sw")
+    got = ops.debug_cast(0, f).numpy()
+    want = corc.f32_to_e4m3fn(f.numpy())
+    assert np.array_equal(got[~isnan], want[~isnan]) and ((got[isnan] & 0x7F) == 0x7F).all()
+    say("debug_cast e4m3 hw (clamped)")
+    got = ops.debug_cast(1, f).numpy()
+    want = corc.f32_to_e4m3fn(np.clip(f.numpy(), -448, 448))
+    assert np.array_equal(got[~isnan], want[~isnan])
+    say("debug_cast e8m0")
+    assert np.array_equal(ops.debug_cast(2, f).numpy(), corc.f32_to_e8m0(f.numpy()))
+    say("debug_cast bf16")
+    got = ops.debug_cast(3, f).numpy().view(np.uint16)
+    assert np.array_equal(got[~isnan], corc.f32_to_bf16(f.numpy())[~isnan])
+
+
+def _ref(name, x, block):
+    if name == "pow2":
+        return T.quant_fp8_e4m3_scale_e8m0(x, block)
+    if name == "div_floor":
+        return T.quant_block_fp32_scale(x, block, amax_floor=1e-12)
+    if name == "div_zero1":
+        return T.quant_block_fp32_scale(x, block, amax_floor=None, zero_scale_to_one=True)
+    return T.quantize_fp8_blockwise(x, block, scale_dtype=torch.float32)
+
+
+def _hip(G, name, x, block):
+    from gcore_lowp import _abi as A, ops
+    if name == "pow2":
+        return G.quant_fp8_e4m3_scale_e8m0(x, block)
+    if name == "div_floor":
+        q, s, _ = ops.quant_fp8_block(x, block, scale_mode=A.SCALE_DIV, scale_dtype=torch.float32, amax_floor=1e-12)
+        return q, s
+    if name == "div_zero1":
+        q, s, _ = ops.quant_fp8_block(x, block, scale_mode=A.SCALE_DIV, scale_dtype=torch.float32,
+                                      zero_rule=A.ZERO_SCALE_TO_ONE)
+        return q, s
+    return G.quantize_fp8_blockwise(x, block, scale_dtype=torch.float32)
+
+
+def _inputs_for(block):
+    xs = {
+        "weight_bf16": I.weight_like(512, 768, 1),
+        "act_bf16": I.act_like(384, 1024, 2),
+        "edge_tiles": I.edge_tiles(),
+        "weight_f32": I.weight_like(256, 512, 3, dtype=torch.float32),
+        "act_f32_wide": (I.act_like(256, 256, 4, dtype=torch.float32) * torch.logspace(-30, 30, 256)),
+        "with_zero_tile": I.weight_like(256, 256, 5),
+        "ragged_rows": I.act_like(37, 384, 6),
+    }
+    xs["with_zero_tile"][:128, 128:] = 0
+    if block[0] != 1:
+        xs.pop("ragged_rows")
+    return xs
+
+
+@pytest.mark.parametrize("name", ["pow2", "div_floor", "div_zero1", "mul"])
+@pytest.mark.parametrize("block", [(128, 128), (1, 128), (2, 2), (64, 32)])
+def test_quant_parity(G, corc, name, block):
+    for label, x in _inputs_for(block).items():
+        if x.shape[0] % block[0] or x.shape[1] % block[1]:
+            continue
+        say("quant", name, block, label, tuple(x.shape), x.dtype)
+        rq, rs = _ref(name, x, block)
+        hq, hs = _hip(G, name, x.cuda(), block)
+        assert hq.dtype == rq.dtype and hs.dtype == rs.dtype and hq.is_cuda and hs.is_cuda
+        assert bits_equal(hs, rs), f"scales differ: {name} {block} {label}"
+        assert bits_equal(hq, rq), f"codes differ: {name} {block} {label}: {(u8(hq) != u8(rq)).sum().item()} bytes"
+        # and against the scalar C oracle
+        kw = {"pow2": dict(mode=0), "div_floor": dict(mode=1, amax_floor=1e-12),
+              "div_zero1": dict(mode=1, zero_rule=2), "mul": dict(mode=2)}[name]
+        cq, cs, csb, _ = corc.quant_fp8_block(x.float().numpy(), block[0], block[1], **kw)
+        assert np.array_equal(u8(hq).numpy(), cq)
+
+
+def test_quant_leading_dims_and_cpu_inputs(G):
+    x = I.weight_like(3 * 256, 256, 8).reshape(3, 256, 256)
+    say("quant 3-D input on GPU")
+    q, s = G.quant_fp8_e4m3_scale_e8m0(x.cuda())
+    rq, rs = T.quant_fp8_e4m3_scale_e8m0(x)
+    assert tuple(s.shape) == (3, 2, 2) and bits_equal(q, rq) and bits_equal(s, rs)
+    say("quant CPU input -> CPU output")
+    q, s = G.quant_fp8_e4m3_scale_e8m0(x)
+    assert not q.is_cuda and not s.is_cuda and bits_equal(q, rq) and bits_equal(s, rs)
+    say("quant non-contiguous input")
+    xt = I.weight_like(256, 128, 9).t()
+    q, s = G.quant_fp8_e4m3_scale_e8m0(xt.cuda())
+    rq, rs = T.quant_fp8_e4m3_scale_e8m0(xt)
+    assert bits_equal(q, rq) and bits_equal(s, rs)
+    say("quantize_fp8_blockwise bf16 scales, CPU return")
+    q, s = G.quantize_fp8_blockwise(x[0], (128, 128))
+    rq, rs = T.quantize_fp8_blockwise(x[0], (128, 128))
+    assert not q.is_cuda and s.dtype == torch.bfloat16 and bits_equal(q, rq) and bits_equal(s, rs)
+
+
+def test_quant_nan_is_rejected(G):
+    x = I.weight_like(128, 256, 10).cuda()
+    x[5, 200] = float("nan")
+    say("quant NaN assert")
+    with pytest.raises(AssertionError, match="NaN"):
+        G.quant_fp8_e4m3_scale_e8m0(x)
+    say("quant NaN divide form: NaN scale and NaN codes in that tile only")
+    q, s = G.quant_2d(x)
+    assert torch.isnan(s[0, 1]).item() and not torch.isnan(s[0, 0]).item()
+    assert ((u8(q)[:, 128:] & 0x7F) == 0x7F).all()
+    rq, rs = T.quant_block_fp32_scale(x.cpu(), (128, 128))
+    assert torch.equal(u8(q)[:, :128], u8(rq)[:, :128])
+
+
+def test_quant_inf_follows_ieee(G):
+    x = I.weight_like(128, 128, 12, dtype=torch.float32)
+    x[3, 3] = float("inf")
+    for name in ("pow2", "div_floor"):
+        say("quant inf", name)
+        rq, rs = _ref(name, x, (128, 128))
+        hq, hs = _hip(G, name, x.cuda(), (128, 128))
+        assert bits_equal(hs, rs)
+        a, b = u8(hq), u8(rq)
+        nan = (b & 0x7F) == 0x7F
+        assert torch.equal(a[~nan], b[~nan]) and ((a[nan] & 0x7F) == 0x7F).all()
+
+
+@pytest.mark.parametrize("sdt", [torch.float32, torch.bfloat16, E8M0])
+@pytest.mark.parametrize("block", [(128, 128), (1, 128), (1, 32), (2, 2), (64, 8)])
+def test_dequant_fp8_parity(G, sdt, block):
+    torch.manual_seed(20)
+    rows, cols = 256, 384
+    q = torch.randint(0, 256, (rows, cols), dtype=torch.int32).to(torch.uint8)
+    q[(q & 0x7F) == 0x7F] = 0x45
+    s = (torch.rand(rows // block[0], cols // block[1]) * 8 + 2.0 ** -20)
+    s = s.to(sdt)
+    say("dequant fp8", sdt, block)
+    want = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q.view(E4M3), s)
+    got = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q.view(E4M3).cuda(), s.cuda())
+    assert got.is_cuda and bits_equal(got, want)
+
+
+def test_dequant_fp8_special_values(G):
+    """NaN codes, e8m0 NaN / extreme scales, products that overflow bf16."""
+    q = torch.arange(256, dtype=torch.int32).to(torch.uint8).repeat(128, 1)[:, :256].contiguous()
+    for sb in (0, 1, 100, 127, 200, 250, 254, 255):
+        s = torch.full((1, 2), sb, dtype=torch.uint8).view(E8M0)
+        say("dequant fp8 special scale byte", sb)
+        want = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q.view(E4M3), s)
+        got = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q.view(E4M3).cuda(), s.cuda()).cpu()
+        nan = torch.isnan(want.float())
+        assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
+        assert torch.isnan(got.float()[nan]).all()
+    say("cast_e4m3fn_to_bf16")
+    w = (torch.randn(256, 384) * 3).to(E4M3)
+    s = torch.pow(2.0, torch.randint(-8, 9, (2, 3)).float()).to(E8M0)
+    assert bits_equal(G.cast_e4m3fn_to_bf16(w.cuda(), s.cuda()), T.cast_e4m3fn_to_bf16(w, s))
+    say("official_wo_a_to_sgl / sgl_wo_a_to_official")
+    assert bits_equal(G.official_wo_a_to_sgl(w.cuda(), s.cuda()), T.cast_e4m3fn_to_bf16(w, s))
+    bf = I.act_like(256, 256, 21)
+    hq, hs = G.sgl_wo_a_to_official(bf.cuda())
+    rq, rs = T.quant_fp8_e4m3_scale_e8m0(bf.float())
+    assert bits_equal(hq, rq) and bits_equal(hs, rs)
+
+
+def test_fp4_dequant_parity(G):
+    sbytes = [0, 1, 2, 3] + list(range(117, 128)) + [200, 252, 253, 254, 255]
+    packed = torch.arange(256, dtype=torch.int32).to(torch.uint8).repeat_interleave(16).reshape(256, 16)
+    for sb in sbytes:
+        scale = torch.full((256, 1), sb, dtype=torch.uint8).view(E8M0)
+        say("fp4 dequant all bytes, scale byte", sb)
+        want = T.cast_e2m1fn_to_bf16(packed.view(torch.int8), scale)
+        got = G.cast_e2m1fn_to_bf16(packed.view(torch.int8).cuda(), scale.cuda()).cpu()
+        nan = torch.isnan(want.float())
+        assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan]), sb
+        assert torch.isnan(got.float()[nan]).all()
+        want = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(packed.view(torch.int8), scale)
+        got = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(packed.view(torch.int8).cuda(), scale.cuda()).cpu()
+        assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan]), sb
+    for (rows, cols), seed in [((128, 256), 1), ((2048, 7168), 2), ((7168, 2048), 3), ((5, 64), 4)]:
+        p, s = I.fp4_expert(rows, cols, seed)
+        say("fp4 -> bf16", rows, cols)
+        assert bits_equal(G.cast_e2m1fn_to_bf16(p.cuda(), s.cuda()), T.cast_e2m1fn_to_bf16(p, s))
+    say("fp4 dequant with 2 x 64 blocks and fp32 scales")
+    p, _ = I.fp4_expert(64, 256, 5)
+    s = torch.rand(32, 4) + 0.25
+    want = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(p, s)
+    got = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(p.cuda(), s.cuda())
+    assert got.dtype == torch.float32 and bits_equal(got, want)
+
+
+def test_fp4_rebase_parity(G):
+    for (rows, cols), seed, (lo, hi) in [((128, 128), 1, (125, 129)), ((256, 256), 2, (119, 135)),
+                                         ((256, 384), 3, (117, 127)), ((2048, 7168), 4, (117, 127)),
+                                         ((7168, 2048), 5, (117, 127)), ((128, 640), 6, (60, 200)),
+                                         ((128, 256), 7, (0, 20)), ((128, 256), 8, (235, 254))]:
+        p, s = I.fp4_expert(rows, cols, seed, lo, hi)
+        say("fp4 rebase", rows, cols, lo, hi)
+        rq, rs = T.cast_e2m1fn_to_e4m3fn(p, s)
+        hq, hs = G.cast_e2m1fn_to_e4m3fn(p.cuda(), s.cuda())
+        assert bits_equal(hs, rs) and bits_equal(hq, rq)
+        rq, rs = T.official_expert_to_sgl(p, s)
+        hq, hs = G.official_expert_to_sgl(p.cuda(), s.cuda())
+        assert hs.dtype == torch.float32 and bits_equal(hs, rs) and bits_equal(hq, rq)
+
+
+def test_fp4_fused_amax_parity(G):
+    for (rows, cols), seed, (lo, hi) in [((128, 128), 1, (117, 127)), ((256, 384), 2, (117, 127)),
+                                         ((2048, 7168), 3, (117, 127)), ((7168, 2048), 4, (117, 127)),
+                                         ((128, 640), 5, (2, 252)), ((256, 256), 6, (0, 6)),
+                                         ((256, 256), 7, (248, 254)), ((128, 512), 8, (100, 140))]:
+        p, s = I.fp4_expert(rows, cols, seed, lo, hi)
+        if seed == 2:
+            p.view(torch.uint8)[:128, :64] = 0x80          # a tile of zeros (codes 0 and 8 only)
+        say("fp4 fused amax", rows, cols, lo, hi)
+        w = T.cast_e2m1fn_to_bf16(p, s)
+        rq, rs = T.quant_block_fp32_scale(w, (128, 128))
+        hq, hs, hw = G.fp4_to_fp8_blockwise(p.cuda(), s.cuda(), return_bf16=True)
+        assert bits_equal(hw, w)
+        assert bits_equal(hs, rs)
+        a, b = u8(hq), u8(rq)
+        nan = (b & 0x7F) == 0x7F
+        assert torch.equal(a[~nan], b[~nan]) and ((a[nan] & 0x7F) == 0x7F).all()
+        hq2, hs2 = G.fp4_to_fp8_blockwise(p.cuda(), s.cuda())
+        assert bits_equal(hq2, hq) and bits_equal(hs2, hs)
+
+
+def test_full_size_round_trip_properties(G):
+    """Benchmark config 1 at full size: [4096, 4096] bf16, N(0, 0.02) + 0.1 % outliers."""
+    x = I.weight_like(4096, 4096, 100).cuda()
+    say("C1 full size quant (divide form)")
+    q, s = G.quant_2d(x)
+    deq = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q, s)             # fp32 scales -> fp32 result
+    assert deq.dtype == torch.float32
+    # requantising the dequantised tensor reproduces codes and scales (idempotence on the grid)
+    q2, s2 = G.quant_2d(deq)
+    assert bits_equal(q2, q)
+    assert torch.allclose(s2, s, rtol=2e-7, atol=0)
+    amax = x.float().reshape(32, 128, 32, 128).abs().amax(dim=(1, 3))
+    assert torch.equal(s, amax / 448.0)
+    assert (u8(q).reshape(32, 128, 32, 128).__and__(0x7F).amax(dim=(1, 3)) == 0x7E).all()
+    err = (deq - x.float()).abs()
+    assert (err <= x.float().abs() * 2.0 ** -4 + s.repeat_interleave(128, 0).repeat_interleave(128, 1) * 2.0 ** -10).all()
+    say("C1 full size pow2 + bf16 dequant == oracle on a 512-row slab")
+    q, s = G.quant_fp8_e4m3_scale_e8m0(x)
+    d = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q, s)
+    rq, rs = T.quant_fp8_e4m3_scale_e8m0(x[:512].cpu())
+    rd = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(rq, rs)
+    assert bits_equal(q[:512], rq) and bits_equal(s[:4], rs) and bits_equal(d[:512], rd)
+    # checksum over the whole tensor vs the oracle's (cheap: byte sum)
+    rq_all, rs_all = T.quant_fp8_e4m3_scale_e8m0(x.cpu())
+    assert int(u8(q).long().sum()) == int(u8(rq_all).long().sum()) and bits_equal(s, rs_all)
