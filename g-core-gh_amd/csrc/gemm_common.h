@@ -1,0 +1,52 @@
+// Pieces shared by the FP8 GEMM translation units.
+#pragma once
+#include "lowp_device.h"
+
+namespace lowp {
+namespace gemm {
+
+template <int SDT>
+__device__ __forceinline__ float scale_at(const void *s, int64_t idx)
+{
+    if (SDT == LP_F32) return ((const float *)s)[idx];
+    // e8m0: 2^(b-127); byte 0 is the fp32 subnormal 2^-127 and 0xFF is NaN
+    const uint32_t b = ((const uint8_t *)s)[idx];
+    return u2f(b == 0u ? 0x00400000u : (b == 0xFFu ? 0x7FC00000u : b << 23));
+}
+
+// Tile order: tiles are numbered so that 32 consecutive numbers form a block of
+// 8 M-tiles x 4 N-tiles (shared operand panels), and each XCD (workgroup id
+// modulo 8) is handed whole blocks, so panels are re-used out of one L2.
+constexpr int GROUP_M = 8, GROUP_N = 4, CHUNK = GROUP_M * GROUP_N;
+
+__device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t tiles_n, int64_t &tm, int64_t &tn)
+{
+    const int64_t xcd = b & 7, s = b >> 3;
+    const int64_t lin = ((s / CHUNK) * 8 + xcd) * CHUNK + s % CHUNK;
+    if (lin >= tiles_m * tiles_n) return false;
+    // groups of GROUP_M m-tiles (the last may be short); inside a group, blocks of
+    // GROUP_N n-tiles (the last may be narrow); inside a block m runs fastest
+    const int64_t per_group = GROUP_M * tiles_n;
+    const int64_t grp = lin / per_group, in_grp = lin - grp * per_group;
+    const int64_t left = tiles_m - grp * GROUP_M;
+    const int64_t gm = left < GROUP_M ? left : GROUP_M;
+    const int64_t per_nblock = gm * GROUP_N;
+    const int64_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
+    tm = grp * GROUP_M + in_blk % gm;
+    tn = nblk * GROUP_N + in_blk / gm;
+    return true;
+}
+
+inline int64_t padded_grid(int64_t tiles_m, int64_t tiles_n)
+{
+    const int64_t chunks = (tiles_m * tiles_n + CHUNK - 1) / CHUNK;
+    return ((chunks + 7) / 8) * 8 * CHUNK;
+}
+
+// gemm_fp8_big.hip
+int choose_big_tn(int64_t M, int64_t N);
+int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
+               int64_t K, void *C, int out_dtype, int tn, hipStream_t st);
+
+}  // namespace gemm
+}  // namespace lowp

@@ -15,9 +15,14 @@
 //
 // The same tile routine serves the dense, split-K (skinny M) and grouped
 // (per-expert row ranges) entry points.
-#include "lowp_device.h"
+#include <stdlib.h>
+
+#include "gemm_common.h"
 
 using namespace lowp;
+using lowp::gemm::scale_at;
+using lowp::gemm::tile_coords;
+using lowp::gemm::padded_grid;
 
 namespace {
 
@@ -28,7 +33,7 @@ constexpr int TM = 128, TN = 128, TK = 128;
 constexpr int LDS_ROW = TK + 16;                 // bytes per staged row
 constexpr int TILE_BYTES = 128 * LDS_ROW;        // one operand tile in LDS
 
-struct Smem {
+struct alignas(16) Smem {
     uint8_t a[2][TILE_BYTES];
     uint8_t b[2][TILE_BYTES];
     float as[2][TM];
@@ -48,15 +53,10 @@ struct TileArgs {
     int kb_begin, kb_end;
 };
 
-__device__ __forceinline__ float scale_at(const void *s, int dtype, int64_t idx)
-{
-    if (dtype == LP_F32) return ((const float *)s)[idx];
-    return e8m0_to_f32(((const uint8_t *)s)[idx]);
-}
-
 // accumulators of one wave: acc[mb][nb] is a 32(n) x 32(m) block
 struct Acc { f32x16 v[2][2]; };
 
+template <int SDT>
 __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc)
 {
     const int t = threadIdx.x;
@@ -86,7 +86,7 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
         }
         if (t < TM) {
             const int64_t m = ta.m0 + t;
-            gas = m < ta.m_end ? scale_at(ta.As, ta.scale_dtype, m * ta.kblocks + kb) : 0.0f;
+            gas = m < ta.m_end ? scale_at<SDT>(ta.As, m * ta.kblocks + kb) : 0.0f;
         }
     };
     auto sstore = [&](int buf) {
@@ -109,7 +109,7 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
         const bool more = kb + 1 < ta.kb_end;
         if (more) gload(kb + 1);
 
-        const float bscale = scale_at(ta.Bs, ta.scale_dtype, (ta.n0 >> 7) * ta.kblocks + kb);
+        const float bscale = scale_at<SDT>(ta.Bs, (ta.n0 >> 7) * ta.kblocks + kb);
 
         // operand fragments: lane reads 32 bytes of its row per 64-wide K half
         i32x8 wf[2][2], af[2][2];
@@ -125,18 +125,26 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
                 wf[blk][kh] = i32x8{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
                 af[blk][kh] = i32x8{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
             }
+        // four 32 x 32 blocks; the fold of block i is issued after the MFMAs of block i+1
+        // so that VALU work overlaps the matrix pipe
+        const float sc0 = sm.as[buf][wm * 64 + l32] * bscale;
+        const float sc1 = sm.as[buf][wm * 64 + 32 + l32] * bscale;
+        const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        f32x16 p[4];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            const float sc = sm.as[buf][wm * 64 + mb * 32 + l32] * bscale;
+        for (int blk = 0; blk < 4; ++blk) {
+            const int mb = blk >> 1, nb = blk & 1;
+            p[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][0], af[mb][0], zero, 0, 0, 0, 0, 0, 0);
+            p[blk] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][1], af[mb][1], p[blk], 0, 0, 0, 0, 0, 0);
+            if (blk > 0) {
+                const int pm = (blk - 1) >> 1, pn = (blk - 1) & 1;
+                const float sc = pm ? sc1 : sc0;
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                f32x16 p = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-                p = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][0], af[mb][0], p, 0, 0, 0, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[nb][1], af[mb][1], p, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = __builtin_fmaf(p[r], sc, acc.v[mb][nb][r]);
+                for (int r = 0; r < 16; ++r) acc.v[pm][pn][r] = __builtin_fmaf(p[blk - 1][r], sc, acc.v[pm][pn][r]);
             }
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc.v[1][1][r] = __builtin_fmaf(p[3][r], sc1, acc.v[1][1][r]);
         if (more) sstore(buf ^ 1);
         __syncthreads();
     }
@@ -178,30 +186,8 @@ __device__ __forceinline__ void store_tile(const Acc &acc, int64_t m0, int64_t m
     });
 }
 
-// Tile order: tiles are numbered so that 32 consecutive numbers form a block of
-// 8 M-tiles x 4 N-tiles (shared operand panels), and each XCD (workgroup id
-// modulo 8) is handed whole blocks, so panels are re-used out of one L2.
-constexpr int GROUP_M = 8, GROUP_N = 4, CHUNK = GROUP_M * GROUP_N;
-
-__device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t tiles_n, int64_t &tm, int64_t &tn)
-{
-    const int64_t xcd = b & 7, s = b >> 3;
-    const int64_t lin = ((s / CHUNK) * 8 + xcd) * CHUNK + s % CHUNK;
-    if (lin >= tiles_m * tiles_n) return false;
-    // groups of GROUP_M m-tiles (the last may be short); inside a group, blocks of
-    // GROUP_N n-tiles (the last may be narrow); inside a block m runs fastest
-    const int64_t per_group = GROUP_M * tiles_n;
-    const int64_t grp = lin / per_group, in_grp = lin - grp * per_group;
-    const int64_t left = tiles_m - grp * GROUP_M;
-    const int64_t gm = left < GROUP_M ? left : GROUP_M;
-    const int64_t per_nblock = gm * GROUP_N;
-    const int64_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
-    tm = grp * GROUP_M + in_blk % gm;
-    tn = nblk * GROUP_N + in_blk / gm;
-    return true;
-}
-
-__global__ __launch_bounds__(256) void gemm_dense(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+template <int SDT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_dense(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                   int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
                                                   int64_t tiles_n, void *__restrict__ C, int out_dtype)
@@ -214,16 +200,9 @@ __global__ __launch_bounds__(256) void gemm_dense(const uint8_t *__restrict__ Aq
     ta.K = K; ta.kblocks = K / TK; ta.m0 = tm * TM; ta.m_end = M; ta.n0 = tn * TN;
     ta.kb_begin = 0; ta.kb_end = (int)(K / TK);
     Acc acc;
-    gemm_tile(ta, sm, acc);
+    gemm_tile<SDT>(ta, sm, acc);
     store_tile(acc, ta.m0, M, ta.n0, N, C, out_dtype);
 }
-
-int64_t padded_grid(int64_t tiles_m, int64_t tiles_n)
-{
-    const int64_t chunks = (tiles_m * tiles_n + CHUNK - 1) / CHUNK;
-    return ((chunks + 7) / 8) * 8 * CHUNK;
-}
-
 
 // ------------------------------------------------------------------ split-K
 // Skinny problems (few output tiles) are weight-streaming bound: K is cut into
@@ -231,7 +210,8 @@ int64_t padded_grid(int64_t tiles_m, int64_t tiles_n)
 // fp32 partial tile to the workspace and a second kernel adds the ranges in a
 // fixed order (deterministic) and narrows.
 
-__global__ __launch_bounds__(256) void gemm_splitk(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+template <int SDT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_splitk(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                    const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                    int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
                                                    int64_t tiles_n, int splits, int kb_per_split, float *__restrict__ ws)
@@ -248,7 +228,7 @@ __global__ __launch_bounds__(256) void gemm_splitk(const uint8_t *__restrict__ A
     ta.kb_end = ta.kb_begin + kb_per_split < kb_all ? ta.kb_begin + kb_per_split : kb_all;
     Acc acc;
     if (ta.kb_begin < ta.kb_end) {
-        gemm_tile(ta, sm, acc);
+        gemm_tile<SDT>(ta, sm, acc);
     } else {
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
@@ -293,7 +273,8 @@ int choose_splits(int64_t tiles, int64_t kblocks)
 // The grid is sized from an upper bound on the number of 128-row tiles; every
 // workgroup finds its (expert, tile) from the offsets with a block-wide scan.
 
-__global__ __launch_bounds__(256) void gemm_grouped(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+template <int SDT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_grouped(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                     const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                     int scale_dtype, const int32_t *__restrict__ m_offsets, int E,
                                                     int64_t N, int64_t K, int64_t max_mtiles, int64_t tiles_n,
@@ -338,7 +319,7 @@ __global__ __launch_bounds__(256) void gemm_grouped(const uint8_t *__restrict__ 
     ta.m0 = row_begin + (gmt - found_first) * TM; ta.m_end = row_end; ta.n0 = tn * TN;
     ta.kb_begin = 0; ta.kb_end = (int)kblocks;
     Acc acc;
-    gemm_tile(ta, sm, acc);
+    gemm_tile<SDT>(ta, sm, acc);
     store_tile(acc, ta.m0, row_end, ta.n0, N, C, out_dtype);
 }
 
@@ -382,8 +363,12 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
         const int kb_all = (int)(K / TK);
         const int per = (kb_all + splits - 1) / splits;
         splits = (kb_all + per - 1) / per;
-        hipLaunchKernelGGL(gemm_splitk, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(256), 0, st, (const uint8_t *)Aq,
-                           As, (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, splits, per, (float *)workspace);
+        if (scale_dtype == LP_F32)
+            hipLaunchKernelGGL(gemm_splitk<LP_F32>, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(256), 0, st, (const uint8_t *)Aq,
+                               As, (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, splits, per, (float *)workspace);
+        else
+            hipLaunchKernelGGL(gemm_splitk<LP_E8M0>, dim3((unsigned)(tiles_m * tiles_n * splits)), dim3(256), 0, st, (const uint8_t *)Aq,
+                               As, (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, splits, per, (float *)workspace);
         rc = check_launch("lp_gemm_fp8_block(split-K)");
         if (rc) return rc;
         const int64_t mn = M * N;
@@ -391,10 +376,22 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
                            splits, mn, C, out_dtype);
         return check_launch("lp_gemm_fp8_block(reduce)");
     }
+    // prefill-sized problems go to the 256-row kernel; LP_GEMM_FORCE_SMALL=1 keeps the 128 x 128 kernel (tests)
+    static const bool force_small = getenv("LP_GEMM_FORCE_SMALL") != nullptr;
+    if (!force_small && M >= 192 && tiles_m * tiles_n >= 512)
+    {
+        const char *force_tn = getenv("LP_GEMM_TN");      // tuning aid: 128 / 192 / 256
+        const int tn = force_tn ? atoi(force_tn) : gemm::choose_big_tn(M, N);
+        return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, tn, st);
+    }
     const int64_t grid = padded_grid(tiles_m, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");
-    hipLaunchKernelGGL(gemm_dense, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
-                       (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
+    if (scale_dtype == LP_F32)
+        hipLaunchKernelGGL(gemm_dense<LP_F32>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
+    else
+        hipLaunchKernelGGL(gemm_dense<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
     return check_launch("lp_gemm_fp8_block");
 }
 
@@ -410,8 +407,12 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
     const int64_t max_mtiles = M_total / TM + E, tiles_n = N / TN;
     const int64_t grid = padded_grid(max_mtiles, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_grouped: problem too large");
-    hipLaunchKernelGGL(gemm_grouped, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
-                       (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+    if (scale_dtype == LP_F32)
+        hipLaunchKernelGGL(gemm_grouped<LP_F32>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+    else
+        hipLaunchKernelGGL(gemm_grouped<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
     return check_launch("lp_gemm_fp8_grouped");
 }
 

@@ -1,0 +1,349 @@
+// Large-tile block-scaled FP8 GEMM for gfx950 (the kernel that carries prefill-sized problems).
+//
+// Workgroup: 512 threads = 8 waves (4 along M x 2 along N), C tile 256(M) x TN(N)
+// with TN = 128 / 192 / 256 chosen at launch to balance the last round of
+// tiles over the 256 CUs.  K advances in steps of 128 = one scale block.
+//
+// Data movement: each step's operand tiles (256 x 128 B of activations, TN x
+// 128 B of weights) are copied HBM/L2 -> LDS by global_load_lds_dwordx4, with
+// no VGPR staging, into one of two stages (the copy of step k+1 overlaps the
+// math of step k).  A row holds 8 chunks of 16 bytes; chunk c of row r is
+// stored in slot c ^ ((r >> 1) & 7), which makes both the linear 1 KB DMA
+// writes and the fragment reads (16 lanes = 16 consecutive rows, same chunk)
+// conflict free across the 64 LDS banks without padding.
+//
+// Math: v_mfma_f32_16x16x128_f8f6f4 -- one instruction covers the whole 128-wide
+// scale block, so every MFMA starts from a zero accumulator and its 4 results
+// per lane are folded into the fp32 accumulators with 4 FMAs by
+// As[m,kb] * Bs[n/128,kb].  The weight fragment is the MFMA A operand and the
+// activation fragment the B operand: a lane then owns one activation row
+// (lane % 16) per block, so the activation scale is one register per block
+// row, and the weight scale is wave-uniform.
+#include <stdlib.h>
+
+#include "gemm_common.h"
+
+using namespace lowp;
+
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 256;             // tile rows (activations)
+constexpr int KB = 128;             // bytes per row per step
+constexpr int THREADS = 512;
+
+#define LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
+#define GLB_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
+
+#ifndef LP_SWZ
+#define LP_SWZ 0
+#endif
+__device__ __forceinline__ int swz(int row, int chunk)
+{
+#if LP_SWZ == 0
+    return chunk ^ ((row >> 1) & 7);
+#elif LP_SWZ == 1
+    return chunk ^ (row & 7);
+#else
+    return chunk ^ ((row >> 2) & 7);
+#endif
+}
+
+// NB = 16-column blocks per wave; TN = 2 * 16 * NB
+template <int SDT, int NB>
+__global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                    const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                    int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                    void *__restrict__ C, int out_dtype)
+{
+    constexpr int TN = 32 * NB;
+    constexpr int A_BYTES = BM * KB, B_BYTES = TN * KB, STAGE = A_BYTES + B_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * STAGE];
+
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    const int64_t m0 = tm * BM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int kblocks = (int)(K / KB);
+
+    // ---- DMA plan: wave w, instruction i moves rows 8*(w + 8*i) .. +7 (1 KB)
+    const int ld_row = lane >> 3, ld_slot = lane & 7;
+    // Rows past the end of a matrix are clamped to its last row: the copies stay branch free,
+    // the duplicated data only feeds accumulator rows / columns that are never stored.
+    const uint8_t *a_src[BM / 64];
+    const uint8_t *b_src[TN / 64];
+#pragma unroll
+    for (int i = 0; i < BM / 64; ++i) {
+        const int row = 8 * (wave + 8 * i) + ld_row;
+        const int64_t m = m0 + row < M ? m0 + row : M - 1;
+        a_src[i] = Aq + m * K + swz(row, ld_slot) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < TN / 64; ++i) {
+        const int row = 8 * (wave + 8 * i) + ld_row;
+        const int64_t n = n0 + row < N ? n0 + row : N - 1;
+        b_src[i] = Bq + n * K + swz(row, ld_slot) * 16;
+    }
+    auto issue_stage = [&](int kb, int stage) {
+        uint8_t *sa = smem + stage * STAGE, *sb = sa + A_BYTES;
+#pragma unroll
+        for (int i = 0; i < BM / 64; ++i)
+            __builtin_amdgcn_global_load_lds(GLB_PTR(a_src[i] + (int64_t)kb * KB), LDS_PTR(sa + (wave + 8 * i) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < TN / 64; ++i)
+            __builtin_amdgcn_global_load_lds(GLB_PTR(b_src[i] + (int64_t)kb * KB), LDS_PTR(sb + (wave + 8 * i) * 1024), 16, 0, 0);
+    };
+
+    // ---- scales: activation rows of this lane (4 block rows), weight scale blocks of this wave
+    int64_t arow[4];
+    bool arow_ok[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        arow[mb] = m0 + wm * 64 + mb * 16 + l16;
+        arow_ok[mb] = arow[mb] < M;
+    }
+    const int64_t wcol0 = n0 + wn * (TN / 2);                  // first weight row of this wave
+    const int64_t sblk0 = wcol0 >> 7;                           // its scale block
+    const int64_t sblk1 = (wcol0 + TN / 2 - 1) >> 7;            // scale block of the wave's last row
+    const int64_t sblk_max = (N >> 7) - 1;
+    const int split_nb = (int)((((sblk0 + 1) << 7) - wcol0) >> 4);   // first 16-col block that uses sblk1
+
+    auto load_scales = [&](int kb, float sa[4], float sb[2]) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) sa[mb] = arow_ok[mb] ? gemm::scale_at<SDT>(As, arow[mb] * kblocks + kb) : 0.0f;
+        sb[0] = gemm::scale_at<SDT>(Bs, (sblk0 < sblk_max ? sblk0 : sblk_max) * kblocks + kb);
+        sb[1] = gemm::scale_at<SDT>(Bs, (sblk1 < sblk_max ? sblk1 : sblk_max) * kblocks + kb);
+    };
+
+    f32x4v acc[4][NB];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    float sa_next[4], sb_next[2];
+    issue_stage(0, 0);
+    load_scales(0, sa_next, sb_next);
+    __syncthreads();
+
+    const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int kb = 0; kb < kblocks; ++kb) {
+        const int stage = kb & 1;
+        float sc[4][2];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) { sc[mb][0] = sa_next[mb] * sb_next[0]; sc[mb][1] = sa_next[mb] * sb_next[1]; }
+        if (kb + 1 < kblocks) {
+            issue_stage(kb + 1, stage ^ 1);
+            load_scales(kb + 1, sa_next, sb_next);
+        }
+        const uint8_t *sa = smem + stage * STAGE, *sb = sa + A_BYTES;
+
+        // activation fragments of the wave's 4 block rows: lane reads 32 bytes (chunks 2*lq, 2*lq+1) of its row
+        i32x8 af[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+            const int row = wm * 64 + mb * 16 + l16;
+            const u32x4 x0 = *(const u32x4 *)(sa + row * KB + swz(row, 2 * lq) * 16);
+            const u32x4 x1 = *(const u32x4 *)(sa + row * KB + swz(row, 2 * lq + 1) * 16);
+            af[mb] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int row = wn * (TN / 2) + nb * 16 + l16;
+            const u32x4 y0 = *(const u32x4 *)(sb + row * KB + swz(row, 2 * lq) * 16);
+            const u32x4 y1 = *(const u32x4 *)(sb + row * KB + swz(row, 2 * lq + 1) * 16);
+            const i32x8 wf = i32x8{(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+            const int which = nb >= split_nb ? 1 : 0;
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) {
+                const f32x4v p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af[mb], zero, 0, 0, 0, 0, 0, 0);
+                const float s = which ? sc[mb][1] : sc[mb][0];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[mb][nb][r] = __builtin_fmaf(p[r], s, acc[mb][nb][r]);
+            }
+        }
+        __syncthreads();      // waits for the DMA of the next stage and for every wave to leave this one
+    }
+
+    // ---- epilogue: lane owns row m = .. + l16 and, per block, columns 4*lq .. 4*lq+3
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        if (!arow_ok[mb]) continue;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int64_t n = wcol0 + nb * 16 + 4 * lq;
+            if (n >= N) continue;
+            const f32x4v v = acc[mb][nb];
+            if (out_dtype == LP_BF16) {
+                u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+                *(u32x2 *)((uint16_t *)C + arow[mb] * N + n) = o;
+            } else {
+                u32x4 o = {f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])};
+                *(u32x4 *)((float *)C + arow[mb] * N + n) = o;
+            }
+        }
+    }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Hand-scheduled variant: 256 x 256 tile, fp32 scales.  Set-up and epilogue are C++, the K loop
+// is the generated assembly in gemm_big_loop.inc (see gen_gemm_loop.py for the register plan).
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                        const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                        int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                        void *__restrict__ C, int out_dtype)
+{
+    constexpr int TN = 256, A_BYTES = BM * KB, STAGE = 2 * A_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * STAGE];
+
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    const int64_t m0 = tm * BM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const uint32_t kblocks = (uint32_t)(K / KB);
+
+    // DMA source offsets (bytes from the matrix base; the host guarantees they fit 32 bits)
+    const int ld_row = lane >> 3, ld_slot = lane & 7;
+    uint32_t aoff[4], boff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 8 * (wave + 8 * i) + ld_row;
+        const int64_t m = m0 + row < M ? m0 + row : M - 1;
+        const int64_t n = n0 + row < N ? n0 + row : N - 1;
+        aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
+        boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
+    }
+    // activation scale offsets of the lane's four block rows
+    int64_t arow[4];
+    uint32_t soff[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        arow[mb] = m0 + wm * 64 + mb * 16 + l16;
+        soff[mb] = (uint32_t)((arow[mb] < M ? arow[mb] : M - 1) * kblocks * 4);
+    }
+    // weight scale row of this wave (its 128 columns lie in one scale block)
+    const int64_t wcol0 = n0 + wn * 128;
+    int64_t sblk = wcol0 >> 7;
+    if (sblk > (N >> 7) - 1) sblk = (N >> 7) - 1;
+    const float *bs_ptr = Bs + sblk * kblocks;
+    const uint32_t bs_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)bs_ptr);
+    const uint32_t bs_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)bs_ptr >> 32));
+    const uint64_t bs_u = ((uint64_t)bs_hi << 32) | bs_lo;
+
+    // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
+    const uint32_t m0base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    const int arow_l = wm * 64 + l16, brow_l = wn * 128 + l16;
+    const uint32_t ard0 = lds0 + arow_l * KB + swz(arow_l, 2 * lq) * 16;
+    const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
+    const uint32_t brd0 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq) * 16;
+    const uint32_t brd1 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
+
+    f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
+    asm volatile(
+#include "gemm_big_loop.inc"
+        : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
+          "={v[192:207]}"(acc4), "={v[208:223]}"(acc5), "={v[224:239]}"(acc6), "={v[240:255]}"(acc7)
+        : [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]),
+          [boff0] "v"(boff[0]), [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]),
+          [soff0] "v"(soff[0]), [soff1] "v"(soff[1]), [soff2] "v"(soff[2]), [soff3] "v"(soff[3]),
+          [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),
+          [abase] "s"(Aq), [bbase] "s"(Bq), [sbase] "s"(As), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [ksteps] "s"(kblocks)
+        : "memory", "scc",
+          "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45",
+          "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61",
+          "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77",
+          "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93",
+          "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107",
+          "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120",
+          "v121", "v122", "v123", "v124", "v125", "v126", "v127",
+          "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55");
+
+    const f32x16v accs[8] = {acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7};
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+        if (arow[mb] >= M) continue;
+#pragma unroll
+        for (int nb = 0; nb < 8; ++nb) {
+            const int64_t n = wcol0 + nb * 16 + 4 * lq;
+            if (n >= N) continue;
+            const float v0 = accs[nb][mb * 4], v1 = accs[nb][mb * 4 + 1], v2 = accs[nb][mb * 4 + 2], v3 = accs[nb][mb * 4 + 3];
+            if (out_dtype == LP_BF16) {
+                u32x2 o = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
+                *(u32x2 *)((uint16_t *)C + arow[mb] * N + n) = o;
+            } else {
+                u32x4 o = {f2u(v0), f2u(v1), f2u(v2), f2u(v3)};
+                *(u32x4 *)((float *)C + arow[mb] * N + n) = o;
+            }
+        }
+    }
+}
+
+template <int SDT, int NB>
+int launch_nb(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
+              int out_dtype, hipStream_t st)
+{
+    const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 32 * NB - 1) / (32 * NB);
+    const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+    hipLaunchKernelGGL((gemm_big<SDT, NB>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, As,
+                       (const uint8_t *)Bq, Bs, M, N, K, tiles_m, tiles_n, C, out_dtype);
+    return check_launch("lp_gemm_fp8_block(big)");
+}
+
+}  // namespace
+
+namespace lowp {
+namespace gemm {
+
+// Picks the tile width whose last round of tiles wastes the fewest CU slots.
+int choose_big_tn(int64_t M, int64_t N)
+{
+    const int64_t tiles_m = (M + BM - 1) / BM;
+    int best = 256;
+    double best_cost = 1e30;
+    for (int tn : {256, 192, 128}) {
+        const int64_t tiles = tiles_m * ((N + tn - 1) / tn);
+        const int64_t rounds = (tiles + 255) / 256;
+        // time ~ rounds * (work per tile); narrower tiles pay more operand traffic per flop
+        const double cost = (double)rounds * tn * (tn == 256 ? 1.0 : tn == 192 ? 1.04 : 1.10);
+        if (cost < best_cost) { best_cost = cost; best = tn; }
+    }
+    return best;
+}
+
+int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
+               int64_t K, void *C, int out_dtype, int tn, hipStream_t st)
+{
+#define GO(SDT)                                                                                         \
+    do {                                                                                                \
+        if (tn == 256) return launch_nb<SDT, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);             \
+        if (tn == 192) return launch_nb<SDT, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);             \
+        return launch_nb<SDT, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);                            \
+    } while (0)
+    static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;       // tuning / test aid
+    if (!no_asm && scale_dtype == LP_F32 && tn == 256 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
+        M * (K / 128) * 4 < 0xFFFFFFFFll) {
+        const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
+        const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
+        if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+        hipLaunchKernelGGL(gemm_big_asm, dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, (const float *)As,
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, out_dtype);
+        return check_launch("lp_gemm_fp8_block(asm)");
+    }
+    if (scale_dtype == LP_F32) GO(LP_F32);
+    GO(LP_E8M0);
+#undef GO
+}
+
+}  // namespace gemm
+}  // namespace lowp

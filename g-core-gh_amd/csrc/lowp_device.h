@@ -72,6 +72,23 @@ __device__ __forceinline__ uint8_t quant_slow(float v, const BlockScale &b)
     return sw_f32_to_e4m3fn(y);
 }
 
+// Slow-path worker, deliberately out of line and not unrolled so that it adds
+// neither instructions nor registers to the hot kernels: quantises `n`
+// consecutive elements starting at element `off` of x into q with the literal
+// arithmetic.  `mul` is the factor of the MUL mode, `div` the divisor otherwise.
+template <int MODE>
+__device__ __noinline__ void quant_slow_span(const void *x, int is_bf16, int64_t off, int n, float div_or_mul,
+                                             uint8_t *q)
+{
+    BlockScale b;
+    b.stored = div_or_mul; b.div = div_or_mul; b.recip = 0.0f; b.exp2 = 0; b.fast = false;
+#pragma unroll 1
+    for (int j = 0; j < n; ++j) {
+        float v = is_bf16 ? u2f((uint32_t)((const uint16_t *)x)[off + j] << 16) : ((const float *)x)[off + j];
+        q[off + j] = quant_slow<MODE>(v, b);
+    }
+}
+
 __device__ __forceinline__ float clamp448(float y) { return __builtin_amdgcn_fmed3f(y, -kE4M3Max, kE4M3Max); }
 
 // four floats -> four e4m3fn bytes (element 0 in the low byte)

@@ -89,24 +89,23 @@ __global__ __launch_bounds__(256) void quant_tile128(const void *__restrict__ xi
     }
 
     const bool slow = special || (MODE == LP_SCALE_DIV && !bs.fast);
+    if (slow) {
+        // rare: NaN/inf in the block or a scale outside 2^+-60; literal arithmetic, inputs re-read
+        const float d = MODE == LP_SCALE_POW2 ? bs.stored : bs.div;
+#pragma unroll 1
+        for (int i = 0; i < NV; ++i)
+            quant_slow_span<MODE>(xin, IS_BF16, (row0 + (int64_t)i * row_step) * cols + col0, IS_BF16 ? 8 : 4, d, q);
+        return;
+    }
     if (IS_BF16) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             float v[8];
 #pragma unroll
             for (int j = 0; j < 4; ++j) { v[2 * j] = u2f(w[i][j] << 16); v[2 * j + 1] = u2f(w[i][j] & 0xFFFF0000u); }
-            u32x2 out;
-            if (!slow) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
-                out.x = cvt4(v[0], v[1], v[2], v[3]);
-                out.y = cvt4(v[4], v[5], v[6], v[7]);
-            } else {
-                uint32_t o[2] = {0, 0};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) o[j >> 2] |= (uint32_t)quant_slow<MODE>(v[j], bs) << (8 * (j & 3));
-                out.x = o[0]; out.y = o[1];
-            }
+            for (int j = 0; j < 8; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
+            u32x2 out = {cvt4(v[0], v[1], v[2], v[3]), cvt4(v[4], v[5], v[6], v[7])};
             __builtin_nontemporal_store(out, (u32x2 *)(q + (row0 + (int64_t)i * row_step) * cols + col0));
         }
     } else {
@@ -114,18 +113,9 @@ __global__ __launch_bounds__(256) void quant_tile128(const void *__restrict__ xi
         for (int i = 0; i < NV; ++i) {
             float v[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = u2f(w[i][j]);
-            uint32_t out;
-            if (!slow) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
-                out = cvt4(v[0], v[1], v[2], v[3]);
-            } else {
-                out = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) out |= (uint32_t)quant_slow<MODE>(v[j], bs) << (8 * j);
-            }
-            __builtin_nontemporal_store(out, (uint32_t *)(q + (row0 + (int64_t)i * row_step) * cols + col0));
+            for (int j = 0; j < 4; ++j) v[j] = clamp448(scale_fast<MODE>(u2f(w[i][j]), bs));
+            __builtin_nontemporal_store(cvt4(v[0], v[1], v[2], v[3]),
+                                        (uint32_t *)(q + (row0 + (int64_t)i * row_step) * cols + col0));
         }
     }
 }
@@ -191,20 +181,16 @@ __global__ __launch_bounds__(256) void quant_group128(const void *__restrict__ x
         BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
         if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
         const bool slow = special || (MODE == LP_SCALE_DIV && !bs.fast);
-        u32x2 out;
-        if (!slow) {
+        if (slow) {
+            if (g < n_groups)
+                quant_slow_span<MODE>(xin, IS_BF16, g * 128 + lane16 * 8, 8, MODE == LP_SCALE_POW2 ? bs.stored : bs.div, q);
+        } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
-            out.x = cvt4(v[0], v[1], v[2], v[3]);
-            out.y = cvt4(v[4], v[5], v[6], v[7]);
-        } else {
-            uint32_t o[2] = {0, 0};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o[j >> 2] |= (uint32_t)quant_slow<MODE>(v[j], bs) << (8 * (j & 3));
-            out.x = o[0]; out.y = o[1];
+            u32x2 out = {cvt4(v[0], v[1], v[2], v[3]), cvt4(v[4], v[5], v[6], v[7])};
+            if (g < n_groups) __builtin_nontemporal_store(out, (u32x2 *)(q + g * 128 + lane16 * 8));
         }
         if (g < n_groups) {
-            __builtin_nontemporal_store(out, (u32x2 *)(q + g * 128 + lane16 * 8));
             if (lane16 == 0) {
                 store_scale(scale_out, scale_dtype, g, bs.stored);
                 if (has_nan && nan_count) atomicAdd(nan_count, 1);

@@ -12,7 +12,8 @@ __device__ __forceinline__ void count(uint64_t *out, bool bad)
     if ((threadIdx.x & 63) == 0 && b) atomicAdd((unsigned long long *)out, (unsigned long long)__popcll(b));
 }
 
-// which 0: every fp32 pattern; patterns with |x| > 448 (or NaN) are skipped
+// which 0: every fp32 pattern; patterns with |x| > 464 (or NaN) are skipped
+// (448 < |x| <= 464 must round down to 448, which is what lets kernels skip a clamp)
 __global__ __launch_bounds__(256) void st_cvt_fp8(uint64_t *out)
 {
     const uint32_t base = (blockIdx.x * 256u + threadIdx.x) * 16u;
@@ -20,7 +21,7 @@ __global__ __launch_bounds__(256) void st_cvt_fp8(uint64_t *out)
     for (uint32_t i = 0; i < 16u; i += 2) {
         uint32_t u0 = base + i, u1 = base + i + 1;
         float a = u2f(u0), b = u2f(u1);
-        bool ok0 = (u0 & 0x7FFFFFFFu) <= 0x43E00000u, ok1 = (u1 & 0x7FFFFFFFu) <= 0x43E00000u;
+        bool ok0 = (u0 & 0x7FFFFFFFu) <= 0x43E80000u, ok1 = (u1 & 0x7FFFFFFFu) <= 0x43E80000u;
         int w = __builtin_amdgcn_cvt_pk_fp8_f32(ok0 ? a : 0.0f, ok1 ? b : 0.0f, 0, false);
         int w2 = __builtin_amdgcn_cvt_pk_fp8_f32(ok1 ? b : 0.0f, ok0 ? a : 0.0f, 0, true);
         if (ok0) bad |= (uint8_t)w != sw_f32_to_e4m3fn(a) || (uint8_t)(w2 >> 24) != sw_f32_to_e4m3fn(a);

@@ -11,7 +11,7 @@ import os
 import torch  # noqa: F401  (must be imported first: it loads the HIP runtime the library binds to)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "_lib", "liblowp.so")
+LIB_PATH = os.environ.get("LOWP_LIB") or os.path.join(_HERE, "_lib", "liblowp.so")
 
 # enum lp_dtype
 F32, BF16, E8M0, E4M3 = 0, 1, 2, 3

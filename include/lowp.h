@@ -178,7 +178,7 @@ int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const vo
  * On-device self tests of the gfx950 conversion instructions against the
  * library's software casts.  Each writes the number of mismatching inputs to
  * *mismatches (device uint64, zeroed by the call).  No reference counterpart.
- *   which = 0: v_cvt_pk_fp8_f32 over every fp32 with |x| <= 448 (and +-0)
+ *   which = 0: v_cvt_pk_fp8_f32 over every fp32 with |x| <= 464 (and +-0)
  *   which = 1: v_cvt_pk_f32_fp8 over all 256 codes except the two NaNs
  *   which = 2: fp32 -> bf16 conversion over every non-NaN fp32
  *   which = 3: v_cvt_scalef32_pk_f32_fp4 over 256 bytes x the scale exponents used
