@@ -32,7 +32,7 @@ def sources():
 
 
 def _headers_mtime():
-    paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".inc"))]
     paths.append(os.path.join(HERE, "..", "include", "lowp.h"))
     return max(os.path.getmtime(p) for p in paths)
 
@@ -53,7 +53,16 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
+def _generate():
+    """Regenerate the hand-scheduled GEMM loop when its generator is newer than the output."""
+    gen = os.path.join(CSRC, "gen_gemm_loop.py")
+    out = os.path.join(CSRC, "gemm_big_loop.inc")
+    if not os.path.exists(out) or os.path.getmtime(out) < os.path.getmtime(gen):
+        subprocess.check_call([sys.executable, gen])
+
+
 def build(force: bool = False) -> str:
+    _generate()
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(sources()))) as ex:
