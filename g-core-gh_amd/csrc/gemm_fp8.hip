@@ -171,17 +171,17 @@ __device__ __forceinline__ void for_each_quad(const Acc &acc, int64_t m0, int64_
     }
 }
 
-__device__ __forceinline__ void store_tile(const Acc &acc, int64_t m0, int64_t m_end, int64_t n0, int64_t N, void *C,
+__device__ __forceinline__ void store_tile(const Acc &acc, int64_t m0, int64_t m_end, int64_t n0, int64_t ldc, void *C,
                                            int out_dtype)
 {
     for_each_quad(acc, m0, n0, [&](int64_t m, int64_t n, float a, float b, float c, float d) {
         if (m >= m_end) return;
         if (out_dtype == LP_BF16) {
             u32x2 o = {pack_bf16(a, b), pack_bf16(c, d)};
-            *(u32x2 *)((uint16_t *)C + m * N + n) = o;
+            *(u32x2 *)((uint16_t *)C + m * ldc + n) = o;
         } else {
             u32x4 o = {f2u(a), f2u(b), f2u(c), f2u(d)};
-            *(u32x4 *)((float *)C + m * N + n) = o;
+            *(u32x4 *)((float *)C + m * ldc + n) = o;
         }
     });
 }
@@ -190,7 +190,7 @@ template <int SDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_dense(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                   int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
-                                                  int64_t tiles_n, void *__restrict__ C, int out_dtype)
+                                                  int64_t tiles_n, void *__restrict__ C, int64_t ldc, int out_dtype)
 {
     __shared__ Smem sm;
     int64_t tm, tn;
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     ta.kb_begin = 0; ta.kb_end = (int)(K / TK);
     Acc acc;
     gemm_tile<SDT>(ta, sm, acc);
-    store_tile(acc, ta.m0, M, ta.n0, N, C, out_dtype);
+    store_tile(acc, ta.m0, M, ta.n0, ldc, C, out_dtype);
 }
 
 // ------------------------------------------------------------------ split-K
@@ -349,6 +349,22 @@ static int check_gemm_args(const char *name, const void *Aq, const void *As, con
     return LP_OK;
 }
 
+// One launch of the 128 x 128 kernel on columns [0, N) of a problem whose C has row stride ldc.
+static int launch_small(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M,
+                        int64_t N, int64_t K, void *C, int64_t ldc, int out_dtype, hipStream_t st)
+{
+    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
+    const int64_t grid = padded_grid(tiles_m, tiles_n);
+    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");
+    if (scale_dtype == LP_F32)
+        hipLaunchKernelGGL(gemm_dense<LP_F32>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
+    else
+        hipLaunchKernelGGL(gemm_dense<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
+    return check_launch("lp_gemm_fp8_block");
+}
+
 extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
                                  int64_t M, int64_t N, int64_t K, void *C, int out_dtype, void *workspace,
                                  int64_t workspace_bytes, lp_stream_t stream)
@@ -376,23 +392,30 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
                            splits, mn, C, out_dtype);
         return check_launch("lp_gemm_fp8_block(reduce)");
     }
-    // prefill-sized problems go to the 256-row kernel; LP_GEMM_FORCE_SMALL=1 keeps the 128 x 128 kernel (tests)
+    // Prefill-sized problems go to the 256-row kernel.  Its 256 x 256 tiles are dealt to the 256 CUs in
+    // rounds; when the last round would be mostly empty, the columns it would cover are given to the
+    // 128 x 128 kernel instead, whose smaller tiles fill the machine.
+    // LP_GEMM_FORCE_SMALL=1 keeps the 128 x 128 kernel, LP_GEMM_TN forces the big kernel's tile width (tuning aids).
     static const bool force_small = getenv("LP_GEMM_FORCE_SMALL") != nullptr;
-    if (!force_small && M >= 192 && tiles_m * tiles_n >= 512)
-    {
-        const char *force_tn = getenv("LP_GEMM_TN");      // tuning aid: 128 / 192 / 256
-        const int tn = force_tn ? atoi(force_tn) : gemm::choose_big_tn(M, N);
-        return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, tn, st);
+    static const char *force_tn = getenv("LP_GEMM_TN");
+    const int esz = out_dtype == LP_BF16 ? 2 : 4, ssz = scale_dtype == LP_F32 ? 4 : 1;
+    if (!force_small && M >= 192 && tiles_m * tiles_n >= 800) {
+        if (force_tn) return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, atoi(force_tn), st);
+        const int64_t bm = (M + 255) / 256, bn = (N + 255) / 256, tiles = bm * bn;
+        const int64_t full = tiles / 256, rem = tiles % 256;
+        int64_t n_big = N;                                   // columns given to the big kernel
+        if (full >= 1 && rem > 0 && rem < 160) n_big = (full * 256 / bm) * 256;
+        if (n_big > N) n_big = N;
+        if (n_big > 0) {
+            rc = gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, n_big, K, C, N, out_dtype, 256, st);
+            if (rc) return rc;
+        }
+        if (n_big < N)
+            return launch_small(Aq, As, (const uint8_t *)Bq + n_big * K, (const char *)Bs + (n_big / 128) * (K / 128) * ssz,
+                                scale_dtype, M, N - n_big, K, (char *)C + n_big * esz, N, out_dtype, st);
+        return LP_OK;
     }
-    const int64_t grid = padded_grid(tiles_m, tiles_n);
-    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");
-    if (scale_dtype == LP_F32)
-        hipLaunchKernelGGL(gemm_dense<LP_F32>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
-    else
-        hipLaunchKernelGGL(gemm_dense<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, out_dtype);
-    return check_launch("lp_gemm_fp8_block");
+    return launch_small(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, st);
 }
 
 extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
@@ -404,6 +427,9 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
     if (rc) return rc > 0 ? LP_OK : rc;
     if (E == 0) return LP_OK;
     LP_REQUIRE(m_offsets, "lp_gemm_fp8_grouped: null m_offsets");
+    // many rows per expert on average: 256-row tiles on the hand-scheduled kernel
+    if (M_total >= (int64_t)E * 96 && M_total >= 2048 && gemm::big_grouped_ok(scale_dtype, M_total, N, K))
+        return gemm::launch_big_grouped(Aq, As, Bq, Bs, m_offsets, E, M_total, N, K, C, out_dtype, (hipStream_t)stream);
     const int64_t max_mtiles = M_total / TM + E, tiles_n = N / TN;
     const int64_t grid = padded_grid(max_mtiles, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_grouped: problem too large");

@@ -56,7 +56,7 @@ template <int SDT, int NB>
 __global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                     const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                     int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
-                                                    void *__restrict__ C, int out_dtype)
+                                                    void *__restrict__ C, int64_t ldc, int out_dtype)
 {
     constexpr int TN = 32 * NB;
     constexpr int A_BYTES = BM * KB, B_BYTES = TN * KB, STAGE = A_BYTES + B_BYTES;
@@ -180,10 +180,10 @@ __global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ 
             const f32x4v v = acc[mb][nb];
             if (out_dtype == LP_BF16) {
                 u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-                *(u32x2 *)((uint16_t *)C + arow[mb] * N + n) = o;
+                *(u32x2 *)((uint16_t *)C + arow[mb] * ldc + n) = o;
             } else {
                 u32x4 o = {f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3])};
-                *(u32x4 *)((float *)C + arow[mb] * N + n) = o;
+                *(u32x4 *)((float *)C + arow[mb] * ldc + n) = o;
             }
         }
     }
@@ -195,21 +195,26 @@ __global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ 
 // is the generated assembly in gemm_big_loop.inc (see gen_gemm_loop.py for the register plan).
 typedef float f32x16v __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
-                                                        const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                                        int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
-                                                        void *__restrict__ C, int out_dtype)
+// One 256 x 256 tile: activation rows m0 .. min(m0 + 256, M) - 1 (rows at or past M are clamped on the
+// way in and masked on the way out, so M may be the end of an expert's row range), weight rows
+// n0 .. n0 + 255 of the matrix at Bq / Bs.
+__device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                             const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0,
+                                             int64_t M, int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc,
+                                             int out_dtype)
 {
-    constexpr int TN = 256, A_BYTES = BM * KB, STAGE = 2 * A_BYTES;
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * STAGE];
-
-    int64_t tm, tn;
-    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    const int64_t m0 = tm * BM, n0 = tn * TN;
+    constexpr int A_BYTES = BM * KB;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, lq = lane >> 4;
     const uint32_t kblocks = (uint32_t)(K / KB);
+    // the bases go into scalar registers: tell the compiler they are wave-uniform
+    auto uniform = [](const void *p) -> uint64_t {
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)p);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)p >> 32));
+        return ((uint64_t)hi << 32) | lo;
+    };
+    const uint64_t a_u = uniform(Aq), b_u = uniform(Bq), s_u = uniform(As);
 
     // DMA source offsets (bytes from the matrix base; the host guarantees they fit 32 bits)
     const int ld_row = lane >> 3, ld_slot = lane & 7;
@@ -235,9 +240,7 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restric
     int64_t sblk = wcol0 >> 7;
     if (sblk > (N >> 7) - 1) sblk = (N >> 7) - 1;
     const float *bs_ptr = Bs + sblk * kblocks;
-    const uint32_t bs_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)bs_ptr);
-    const uint32_t bs_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)bs_ptr >> 32));
-    const uint64_t bs_u = ((uint64_t)bs_hi << 32) | bs_lo;
+    const uint64_t bs_u = uniform(bs_ptr);
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0)
     const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restric
           [boff0] "v"(boff[0]), [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]),
           [soff0] "v"(soff[0]), [soff1] "v"(soff[1]), [soff2] "v"(soff[2]), [soff3] "v"(soff[3]),
           [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),
-          [abase] "s"(Aq), [bbase] "s"(Bq), [sbase] "s"(As), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [ksteps] "s"(kblocks)
+          [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [ksteps] "s"(kblocks)
         : "memory", "scc",
           "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45",
           "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61",
@@ -279,24 +282,79 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restric
             const float v0 = accs[nb][mb * 4], v1 = accs[nb][mb * 4 + 1], v2 = accs[nb][mb * 4 + 2], v3 = accs[nb][mb * 4 + 3];
             if (out_dtype == LP_BF16) {
                 u32x2 o = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
-                *(u32x2 *)((uint16_t *)C + arow[mb] * N + n) = o;
+                *(u32x2 *)((uint16_t *)C + arow[mb] * ldc + n) = o;
             } else {
                 u32x4 o = {f2u(v0), f2u(v1), f2u(v2), f2u(v3)};
-                *(u32x4 *)((float *)C + arow[mb] * N + n) = o;
+                *(u32x4 *)((float *)C + arow[mb] * ldc + n) = o;
             }
         }
     }
 }
 
+
+__global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                        const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                        int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                        void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    big_tile_asm(smem, Aq, As, Bq, Bs, tm * BM, M, tn * 256, N, K, C, ldc, out_dtype);
+}
+
+// Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
+// The grid is sized from an upper bound on the number of 256-row tiles; each workgroup finds its expert
+// with a block-wide scan over the per-expert tile counts.
+__global__ __launch_bounds__(THREADS) void gemm_big_asm_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                                const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                                const int32_t *__restrict__ m_offsets, int E, int64_t N,
+                                                                int64_t K, int64_t max_mtiles, int64_t tiles_n,
+                                                                void *__restrict__ C, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB];
+    __shared__ int scan[THREADS];
+    __shared__ int found_e, found_first;
+    int64_t gmt, tn;
+    const bool in_range = gemm::tile_coords(blockIdx.x, max_mtiles, tiles_n, gmt, tn);
+    const int t = threadIdx.x;
+    if (t == 0) found_e = -1;
+    __syncthreads();
+    int base = 0;
+    for (int e0 = 0; e0 < E; e0 += THREADS) {
+        const int e = e0 + t;
+        int cnt = 0;
+        if (e < E) cnt = (m_offsets[e + 1] - m_offsets[e] + BM - 1) / BM;
+        scan[t] = cnt;
+        __syncthreads();
+        for (int off = 1; off < THREADS; off <<= 1) {
+            int v = t >= off ? scan[t - off] : 0;
+            __syncthreads();
+            scan[t] += v;
+            __syncthreads();
+        }
+        const int incl = base + scan[t], excl = incl - cnt;
+        if (in_range && e < E && gmt >= excl && gmt < incl) { found_e = e; found_first = excl; }
+        base += scan[THREADS - 1];
+        __syncthreads();
+    }
+    if (!in_range || found_e < 0) return;
+    const int e = found_e;
+    const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
+    const int64_t kblocks = K / KB;
+    big_tile_asm(smem, Aq, As, Bq + (int64_t)e * N * K, Bs + (int64_t)e * (N / 128) * kblocks,
+                 row_begin + (gmt - found_first) * BM, row_end, tn * 256, N, K, C, N, out_dtype);
+}
+
 template <int SDT, int NB>
 int launch_nb(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-              int out_dtype, hipStream_t st)
+              int64_t ldc, int out_dtype, hipStream_t st)
 {
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 32 * NB - 1) / (32 * NB);
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
     hipLaunchKernelGGL((gemm_big<SDT, NB>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, As,
-                       (const uint8_t *)Bq, Bs, M, N, K, tiles_m, tiles_n, C, out_dtype);
+                       (const uint8_t *)Bq, Bs, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
     return check_launch("lp_gemm_fp8_block(big)");
 }
 
@@ -322,13 +380,13 @@ int choose_big_tn(int64_t M, int64_t N)
 }
 
 int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
-               int64_t K, void *C, int out_dtype, int tn, hipStream_t st)
+               int64_t K, void *C, int64_t ldc, int out_dtype, int tn, hipStream_t st)
 {
 #define GO(SDT)                                                                                         \
     do {                                                                                                \
-        if (tn == 256) return launch_nb<SDT, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);             \
-        if (tn == 192) return launch_nb<SDT, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);             \
-        return launch_nb<SDT, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);                            \
+        if (tn == 256) return launch_nb<SDT, 8>(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);             \
+        if (tn == 192) return launch_nb<SDT, 6>(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);             \
+        return launch_nb<SDT, 4>(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);                            \
     } while (0)
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;       // tuning / test aid
     if (!no_asm && scale_dtype == LP_F32 && tn == 256 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
@@ -337,12 +395,31 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
         const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
         hipLaunchKernelGGL(gemm_big_asm, dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, (const float *)As,
-                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, out_dtype);
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
         return check_launch("lp_gemm_fp8_block(asm)");
     }
     if (scale_dtype == LP_F32) GO(LP_F32);
     GO(LP_E8M0);
 #undef GO
+}
+
+// Grouped problems on the hand-scheduled kernel: fp32 scales, N a multiple of 256, offsets that fit 32 bits.
+bool big_grouped_ok(int scale_dtype, int64_t M_total, int64_t N, int64_t K)
+{
+    static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;
+    return !no_asm && scale_dtype == LP_F32 && N % 256 == 0 && M_total * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
+           M_total * (K / 128) * 4 < 0xFFFFFFFFll;
+}
+
+int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,
+                       int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype, hipStream_t st)
+{
+    const int64_t max_mtiles = M_total / BM + E, tiles_n = N / 256;
+    const int64_t grid = padded_grid(max_mtiles, tiles_n);
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
+    hipLaunchKernelGGL(gemm_big_asm_grouped, dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, (const float *)As,
+                       (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+    return check_launch("lp_gemm_fp8_grouped(asm)");
 }
 
 }  // namespace gemm

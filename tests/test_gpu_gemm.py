@@ -67,6 +67,10 @@ DENSE_SHAPES = [
     (128, 128, 128), (128, 256, 256), (256, 128, 512), (64, 4096, 7168), (1, 128, 128), (7, 256, 384),
     (200, 384, 1024), (512, 1024, 2048), (2048, 4096, 7168), (128, 4096, 4096), (1024, 4096, 1024),
     (333, 640, 896),
+    # prefill-sized: 256-row kernel (hand-scheduled loop), ragged M / N tails, and the column split
+    # between the 256 x 256 and the 128 x 128 kernel (576 tiles on 256 CUs)
+    (333, 8320, 512), (200, 16384, 256), (2048, 4224, 384), (256, 32768, 128), (1000, 9216, 640),
+    (2048, 18432, 512), (4096, 4096, 1024),
 ]
 
 
@@ -124,6 +128,10 @@ GROUPED = [
     (5, 128, 384, [0, 0, 0, 0, 0]),
     (3, 384, 512, [300, 0, 77]),
     (300, 128, 128, [i % 7 for i in range(300)]),
+    # many rows per expert: 256-row tiles on the hand-scheduled kernel (ragged experts, empty experts)
+    (8, 512, 512, [700, 0, 300, 1, 255, 256, 257, 600]),
+    (16, 768, 1024, [513, 0, 0, 90, 1024, 17, 256, 300, 2, 511, 128, 129, 64, 1, 700, 333]),
+    (3, 256, 384, [2048, 1, 515]),
 ]
 
 
