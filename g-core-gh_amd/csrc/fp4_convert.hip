@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void fp4_rebase(const uint8_t *__restrict__ pa
 
 // ---------------------------------------------------------------- fused amax
 
-template <int MODE>
+template <int MODE, bool WRITE_BF16>
 __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scale,
                                                 int64_t cols, int64_t supers_c, int64_t n_supers, int64_t per_xcd,
                                                 float amax_floor, int zero_rule, uint8_t *__restrict__ q,
@@ -139,17 +139,16 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
     const Geometry g = geometry(super, supers_c, cols, t);
     const int64_t pcols = cols >> 1, scols = cols >> 5;
 
+    // Lanes of a half that lies past the last tile (odd tile count per row) read the left half's
+    // columns instead, so the loads need no branches; their results are never stored.
+    const int64_t ld_colb = g.active ? g.colb : g.colb - 64, ld_scol = g.active ? g.scol : g.scol - 4;
     uint32_t w[kPasses];
     uint32_t sb[kPasses];
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
         const int64_t r = g.row0 + p * kRowsPerPass;
-        if (g.active) {
-            w[p] = fp4_pos_zero(__builtin_nontemporal_load((const uint32_t *)(packed + r * pcols + g.colb)));
-            sb[p] = scale[r * scols + g.scol];
-        } else {
-            w[p] = 0; sb[p] = 127;
-        }
+        w[p] = fp4_pos_zero(__builtin_nontemporal_load((const uint32_t *)(packed + r * pcols + ld_colb)));
+        sb[p] = scale[r * scols + ld_scol];
     }
 
     // amax of |table(code)| * 2^(sb-127).  The product is exact in fp32 (and
@@ -167,47 +166,70 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
         mbits = prod > mbits ? prod : mbits;
         edge |= (sb[p] < 2u || sb[p] > 252u) ? 1u : 0u;
     }
-    // every thread of the workgroup must take the same number of barriers, so
-    // the slow decision is made for the super tile as a whole
-    const bool slow_tile = __syncthreads_or((int)edge) != 0;
-    const uint32_t key = slow_tile ? 0u : tile_max_u32(mbits, lds, t);
+    // Every thread of the workgroup must take the same number of barriers, so both slow
+    // decisions (edge scale bytes, tile scale outside the fast range) are made for the
+    // super tile as a whole.
+    bool slow_tile = __syncthreads_or((int)edge) != 0;
+    BlockScale bs;
+    // Each element is +-{0, .5, 1, 2, 4} * 2^e (even codes and 0.5) or +-{1, 2, 4} * 1.5 * 2^e (codes
+    // 1.5, 3, 6), so its quotient by the tile scale is a power-of-two multiple of one of two numbers,
+    // c1 = RN(1/s) and c3 = RN(1.5/s) (resp. f and RN(1.5 f) in the multiply form): two correctly
+    // rounded constants per tile replace one division per element, and power-of-two scaling keeps
+    // them correctly rounded.
+    float c1 = 1.0f, c3 = 1.5f;
+    if (!slow_tile) {
+        const uint32_t key = tile_max_u32(mbits, lds, t);
+        bs = derive_scale<MODE>(u2f(key), amax_floor, zero_rule);
+        bool bad;
+        if (MODE == LP_SCALE_POW2) {
+            bad = bs.exp2 < -100 || bs.exp2 > 100;
+            c1 = ldexpf(1.0f, -bs.exp2);
+            c3 = ldexpf(1.5f, -bs.exp2);
+        } else if (MODE == LP_SCALE_DIV) {
+            bad = !bs.fast;
+            c1 = bs.recip;
+            c3 = 1.5f / bs.div;
+        } else {
+            bad = !(bs.div >= 0x1p-100f && bs.div <= 0x1p100f);
+            c1 = bs.div;
+            c3 = 1.5f * bs.div;
+        }
+        slow_tile = __syncthreads_or((int)bad) != 0;
+    }
 
     if (!slow_tile) {
-        const float amax = u2f(key);
-        BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
-        const bool slow = (MODE == LP_SCALE_DIV && !bs.fast);
         if (g.active && (t & 15) == 0 && (t >> 5) == 0) store_scale(scale_out, scale_dtype, g.tile, bs.stored);
         if (!g.active) return;
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int64_t r = g.row0 + p * kRowsPerPass;
-            const float s = u2f(sb[p] << 23);            // sb in 2..252: a normal power of two
-            // decode again rather than keep 128 decoded values alive across the
-            // reduction: the empty asm hides the value from common-subexpression
-            // elimination so the register footprint stays small
+            const int e = (int)sb[p] - 127;
+            // an all-zero block may carry any exponent: keep the factors finite so that 0 * t stays 0
+            const float t1 = fminf(ldexpf(c1, e), 3.0e38f), t3 = fminf(ldexpf(c3, e), 3.0e38f);
+            // decode again rather than keep decoded values alive across the reduction: the empty asm
+            // hides the value from common-subexpression elimination so the register footprint stays small
             uint32_t wp = w[p];
             asm volatile("" : "+v"(wp));
+            const uint32_t mant = wp & 0x11111111u;
+            const uint32_t expnz = ((wp >> 1) | (wp >> 2)) & 0x11111111u;
+            const uint32_t odd = mant & expnz;                  // nibbles holding 1.5, 3 or 6
+            const uint32_t oddmask = (odd << 4) - odd;          // 0xF on those nibbles
+            float fe[8], fo[8];
+            fp4_decode8(wp & ~oddmask, fe);                     // the other elements, as they are
+            fp4_decode8((wp & oddmask) ^ odd, fo);              // 1.5, 3, 6 with the mantissa bit cleared: 1, 2, 4
             float v[8];
-            fp4_decode8(wp, v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] *= s;
-            if (bf16_out) {
-                u32x4 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_fmaf(fo[j], t3, fe[j] * t1);
+            u32x2 out = {cvt4(v[0], v[1], v[2], v[3]), cvt4(v[4], v[5], v[6], v[7])};
+            __builtin_nontemporal_store(out, (u32x2 *)(q + r * cols + (g.colb << 1)));
+            if (WRITE_BF16) {
+                const float s = u2f(sb[p] << 23);            // sb in 2..252: a normal power of two
+                float b[8];
+                fp4_decode8(wp, b);
+                u32x4 o = {pack_bf16(b[0] * s, b[1] * s), pack_bf16(b[2] * s, b[3] * s), pack_bf16(b[4] * s, b[5] * s),
+                           pack_bf16(b[6] * s, b[7] * s)};
                 __builtin_nontemporal_store(o, (u32x4 *)(bf16_out + r * cols + (g.colb << 1)));
             }
-            u32x2 out;
-            if (!slow) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = __builtin_amdgcn_fmed3f(scale_fast<MODE>(v[j], bs), -kE4M3Max, kE4M3Max);
-                out.x = cvt4(v[0], v[1], v[2], v[3]);
-                out.y = cvt4(v[4], v[5], v[6], v[7]);
-            } else {
-                uint32_t o[2] = {0, 0};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) o[j >> 2] |= (uint32_t)quant_slow<MODE>(v[j], bs) << (8 * (j & 3));
-                out.x = o[0]; out.y = o[1];
-            }
-            __builtin_nontemporal_store(out, (u32x2 *)(q + r * cols + (g.colb << 1)));
         }
         return;
     }
@@ -231,7 +253,7 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
     m2 = tile_max_u32(m2, lds, t);
     const bool has_nan = m2 > 0x7F800000u;
     const float amax = u2f(has_nan ? 0x7FC00000u : m2);
-    BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
+    bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
     if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
     if (g.active && (t & 15) == 0 && (t >> 5) == 0) store_scale(scale_out, scale_dtype, g.tile, bs.stored);
     if (!g.active) return;
@@ -301,8 +323,16 @@ extern "C" int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t
     dim3 grid((unsigned)(per_xcd * 8)), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(MODE)                                                                                                   \
-    hipLaunchKernelGGL(fp4_amax<MODE>, grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, cols, supers_c, \
-                       n_supers, per_xcd, amax_floor, zero_rule, (uint8_t *)q_out, scale_out, scale_dtype, (uint16_t *)bf16_out)
+    do {                                                                                                               \
+        if (bf16_out)                                                                                                  \
+            hipLaunchKernelGGL((fp4_amax<MODE, true>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
+                               cols, supers_c, n_supers, per_xcd, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,   \
+                               scale_dtype, (uint16_t *)bf16_out);                                                      \
+        else                                                                                                           \
+            hipLaunchKernelGGL((fp4_amax<MODE, false>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
+                               cols, supers_c, n_supers, per_xcd, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,   \
+                               scale_dtype, (uint16_t *)bf16_out);                                                      \
+    } while (0)
     if (scale_mode == LP_SCALE_POW2) LAUNCH(LP_SCALE_POW2);
     else if (scale_mode == LP_SCALE_DIV) LAUNCH(LP_SCALE_DIV);
     else LAUNCH(LP_SCALE_MUL);
