@@ -57,24 +57,35 @@ __device__ __forceinline__ void decode_fp8x4(uint32_t w, float v[4])
 
 constexpr int kPasses = 8;
 
+// Scale index of chunk c (8 consecutive elements of one row).  With one-row blocks (bm == 1) and
+// cols % bn == 0 the scale grid is just the element index divided by bn: no row / column split.
+template <bool ROWSCALE>
+__device__ __forceinline__ int64_t scale_index(uint32_t c, uint32_t chunks_per_row, int bm_shift, int bn_shift,
+                                               uint32_t scale_cols)
+{
+    if (ROWSCALE) return (int64_t)(((uint64_t)c * 8u) >> bn_shift);
+    const uint32_t row = c / chunks_per_row, cc = c - row * chunks_per_row;
+    return (int64_t)(row >> bm_shift) * scale_cols + ((cc * 8u) >> bn_shift);
+}
+
 // FP8: each lane owns 8 consecutive codes of one row per pass.
 // chunks_per_row = cols / 8; bm, bn powers of two given as shifts; bn >= 8.
-template <bool OUT_BF16>
+// CHECKED = false: every chunk of the workgroup exists (no bounds tests at all).
+template <bool OUT_BF16, bool CHECKED, bool ROWSCALE>
 __global__ __launch_bounds__(256) void dequant_fp8_fast(const uint8_t *__restrict__ q, const void *__restrict__ scale,
-                                                        int scale_dtype, uint32_t n_chunks, uint32_t chunks_per_row,
-                                                        int bm_shift, int bn_shift, uint32_t scale_cols,
-                                                        void *__restrict__ out)
+                                                        int scale_dtype, uint32_t chunk0, uint32_t n_chunks,
+                                                        uint32_t chunks_per_row, int bm_shift, int bn_shift,
+                                                        uint32_t scale_cols, void *__restrict__ out)
 {
-    const uint32_t base = blockIdx.x * (256u * kPasses) + threadIdx.x;
+    const uint32_t base = chunk0 + blockIdx.x * (256u * kPasses) + threadIdx.x;
     u32x2 w[kPasses];
     float s[kPasses];
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-        uint32_t c = base + p * 256u;
-        if (c < n_chunks) {
-            uint32_t row = c / chunks_per_row, cc = c - row * chunks_per_row;
+        const uint32_t c = base + p * 256u;
+        if (!CHECKED || c < n_chunks) {
             w[p] = __builtin_nontemporal_load((const u32x2 *)(q + (int64_t)c * 8));
-            s[p] = load_scale(scale, scale_dtype, (int64_t)(row >> bm_shift) * scale_cols + ((cc * 8u) >> bn_shift));
+            s[p] = load_scale(scale, scale_dtype, scale_index<ROWSCALE>(c, chunks_per_row, bm_shift, bn_shift, scale_cols));
         } else {
             w[p] = u32x2{0, 0};
             s[p] = 0.0f;
@@ -82,34 +93,33 @@ __global__ __launch_bounds__(256) void dequant_fp8_fast(const uint8_t *__restric
     }
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-        uint32_t c = base + p * 256u;
+        const uint32_t c = base + p * 256u;
         float v[8];
         decode_fp8x4(w[p].x, v);
         decode_fp8x4(w[p].y, v + 4);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = v[j] * s[p];
-        if (c < n_chunks) store8<OUT_BF16>(out, (int64_t)c * 8, v);
+        if (!CHECKED || c < n_chunks) store8<OUT_BF16>(out, (int64_t)c * 8, v);
     }
 }
 
 // FP4: each lane owns 4 packed bytes = 8 consecutive elements of one row.
 // chunks_per_row = cols / 8 (logical columns); bn >= 8.
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool CHECKED, bool ROWSCALE>
 __global__ __launch_bounds__(256) void dequant_fp4_fast(const uint8_t *__restrict__ packed, const void *__restrict__ scale,
-                                                        int scale_dtype, uint32_t n_chunks, uint32_t chunks_per_row,
-                                                        int bm_shift, int bn_shift, uint32_t scale_cols, int neg_zero,
-                                                        void *__restrict__ out)
+                                                        int scale_dtype, uint32_t chunk0, uint32_t n_chunks,
+                                                        uint32_t chunks_per_row, int bm_shift, int bn_shift,
+                                                        uint32_t scale_cols, int neg_zero, void *__restrict__ out)
 {
-    const uint32_t base = blockIdx.x * (256u * kPasses) + threadIdx.x;
+    const uint32_t base = chunk0 + blockIdx.x * (256u * kPasses) + threadIdx.x;
     uint32_t w[kPasses];
     float s[kPasses];
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-        uint32_t c = base + p * 256u;
-        if (c < n_chunks) {
-            uint32_t row = c / chunks_per_row, cc = c - row * chunks_per_row;
+        const uint32_t c = base + p * 256u;
+        if (!CHECKED || c < n_chunks) {
             w[p] = __builtin_nontemporal_load((const uint32_t *)(packed + (int64_t)c * 4));
-            s[p] = load_scale(scale, scale_dtype, (int64_t)(row >> bm_shift) * scale_cols + ((cc * 8u) >> bn_shift));
+            s[p] = load_scale(scale, scale_dtype, scale_index<ROWSCALE>(c, chunks_per_row, bm_shift, bn_shift, scale_cols));
         } else {
             w[p] = 0;
             s[p] = 0.0f;
@@ -117,13 +127,13 @@ __global__ __launch_bounds__(256) void dequant_fp4_fast(const uint8_t *__restric
     }
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) {
-        uint32_t c = base + p * 256u;
-        uint32_t x = neg_zero ? w[p] : fp4_pos_zero(w[p]);
+        const uint32_t c = base + p * 256u;
+        const uint32_t x = neg_zero ? w[p] : fp4_pos_zero(w[p]);
         float v[8];
         fp4_decode8(x, v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = v[j] * s[p];
-        if (c < n_chunks) store8<OUT_BF16>(out, (int64_t)c * 8, v);
+        if (!CHECKED || c < n_chunks) store8<OUT_BF16>(out, (int64_t)c * 8, v);
     }
 }
 
@@ -175,19 +185,34 @@ int dequant_common(const char *name, bool is_fp4, const void *codes, const void 
                       (uintptr_t)codes % 8 == 0 && (uintptr_t)out % 16 == 0;
     const bool bf = out_dtype == LP_BF16;
     if (fast) {
-        unsigned wgs = (unsigned)((n_chunks + 256 * kPasses - 1) / (256 * kPasses));
-        uint32_t cpr = (uint32_t)(cols / 8), sc = (uint32_t)(cols / bn);
-        if (is_fp4) {
-            if (bf) hipLaunchKernelGGL(dequant_fp4_fast<true>, dim3(wgs), dim3(256), 0, st, (const uint8_t *)codes, scale,
-                                       scale_dtype, (uint32_t)n_chunks, cpr, bm_shift, bn_shift, sc, neg_zero, out);
-            else hipLaunchKernelGGL(dequant_fp4_fast<false>, dim3(wgs), dim3(256), 0, st, (const uint8_t *)codes, scale,
-                                    scale_dtype, (uint32_t)n_chunks, cpr, bm_shift, bn_shift, sc, neg_zero, out);
-        } else {
-            if (bf) hipLaunchKernelGGL(dequant_fp8_fast<true>, dim3(wgs), dim3(256), 0, st, (const uint8_t *)codes, scale,
-                                       scale_dtype, (uint32_t)n_chunks, cpr, bm_shift, bn_shift, sc, out);
-            else hipLaunchKernelGGL(dequant_fp8_fast<false>, dim3(wgs), dim3(256), 0, st, (const uint8_t *)codes, scale,
-                                    scale_dtype, (uint32_t)n_chunks, cpr, bm_shift, bn_shift, sc, out);
-        }
+        // full workgroups run without bounds tests; the ragged end (< one workgroup of chunks) is a second launch
+        const uint32_t per_wg = 256 * kPasses;
+        const uint32_t full_wgs = (uint32_t)(n_chunks / per_wg), tail0 = full_wgs * per_wg;
+        const uint32_t cpr = (uint32_t)(cols / 8), sc = (uint32_t)(cols / bn);
+        const bool rowscale = bm == 1;
+#define LP_DQ(KERNEL, BF, CHK, RS, GRID, C0, ...)                                                                     \
+    hipLaunchKernelGGL((KERNEL<BF, CHK, RS>), dim3(GRID), dim3(256), 0, st, (const uint8_t *)codes, scale, scale_dtype, \
+                       (uint32_t)(C0), (uint32_t)n_chunks, cpr, bm_shift, bn_shift, sc, ##__VA_ARGS__, out)
+#define LP_DQ_ALL(KERNEL, ...)                                                                                        \
+    do {                                                                                                              \
+        for (int part = 0; part < 2; ++part) {                                                                        \
+            const bool chk = part == 1;                                                                               \
+            const uint32_t grid = chk ? (tail0 < n_chunks ? 1u : 0u) : full_wgs, c0 = chk ? tail0 : 0u;               \
+            if (!grid) continue;                                                                                      \
+            if (bf && !chk && rowscale) LP_DQ(KERNEL, true, false, true, grid, c0, ##__VA_ARGS__);                    \
+            else if (bf && !chk) LP_DQ(KERNEL, true, false, false, grid, c0, ##__VA_ARGS__);                          \
+            else if (bf && rowscale) LP_DQ(KERNEL, true, true, true, grid, c0, ##__VA_ARGS__);                        \
+            else if (bf) LP_DQ(KERNEL, true, true, false, grid, c0, ##__VA_ARGS__);                                   \
+            else if (!chk && rowscale) LP_DQ(KERNEL, false, false, true, grid, c0, ##__VA_ARGS__);                    \
+            else if (!chk) LP_DQ(KERNEL, false, false, false, grid, c0, ##__VA_ARGS__);                               \
+            else if (rowscale) LP_DQ(KERNEL, false, true, true, grid, c0, ##__VA_ARGS__);                             \
+            else LP_DQ(KERNEL, false, true, false, grid, c0, ##__VA_ARGS__);                                          \
+        }                                                                                                             \
+    } while (0)
+        if (is_fp4) LP_DQ_ALL(dequant_fp4_fast, neg_zero);
+        else LP_DQ_ALL(dequant_fp8_fast);
+#undef LP_DQ_ALL
+#undef LP_DQ
     } else {
         int64_t n = rows * cols;
         unsigned wgs = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);

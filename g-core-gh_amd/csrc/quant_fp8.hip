@@ -124,21 +124,22 @@ __global__ __launch_bounds__(256) void quant_tile128(const void *__restrict__ xi
 
 // One group = 128 consecutive elements of a row = 16 lanes x 8 elements.
 // A 256-thread workgroup owns 16 groups per pass and PASSES passes.
-template <bool IS_BF16, int MODE, int PASSES>
-__global__ __launch_bounds__(256) void quant_group128(const void *__restrict__ xin, int64_t n_groups,
+// CHECKED = false: every group of the workgroup exists (no bounds tests).
+template <bool IS_BF16, int MODE, int PASSES, bool CHECKED>
+__global__ __launch_bounds__(256) void quant_group128(const void *__restrict__ xin, int64_t group0, int64_t n_groups,
                                                       uint8_t *__restrict__ q, void *__restrict__ scale_out,
                                                       int scale_dtype, float amax_floor, int zero_rule,
                                                       int32_t *nan_count)
 {
     const int t = threadIdx.x;
-    const int64_t g0 = (int64_t)blockIdx.x * (16 * PASSES) + (t >> 4);
+    const int64_t g0 = group0 + (int64_t)blockIdx.x * (16 * PASSES) + (t >> 4);
     const int lane16 = t & 15;
 
     u32x4 w[PASSES][IS_BF16 ? 1 : 2];
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
         int64_t g = g0 + p * 16;
-        if (g < n_groups) {
+        if (!CHECKED || g < n_groups) {
             if (IS_BF16) {
                 w[p][0] = __builtin_nontemporal_load((const u32x4 *)((const char *)xin + (g * 128 + lane16 * 8) * 2));
             } else {
@@ -182,15 +183,15 @@ __global__ __launch_bounds__(256) void quant_group128(const void *__restrict__ x
         if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
         const bool slow = special || (MODE == LP_SCALE_DIV && !bs.fast);
         if (slow) {
-            if (g < n_groups)
+            if (!CHECKED || g < n_groups)
                 quant_slow_span<MODE>(xin, IS_BF16, g * 128 + lane16 * 8, 8, MODE == LP_SCALE_POW2 ? bs.stored : bs.div, q);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
             u32x2 out = {cvt4(v[0], v[1], v[2], v[3]), cvt4(v[4], v[5], v[6], v[7])};
-            if (g < n_groups) __builtin_nontemporal_store(out, (u32x2 *)(q + g * 128 + lane16 * 8));
+            if (!CHECKED || g < n_groups) __builtin_nontemporal_store(out, (u32x2 *)(q + g * 128 + lane16 * 8));
         }
-        if (g < n_groups) {
+        if (!CHECKED || g < n_groups) {
             if (lane16 == 0) {
                 store_scale(scale_out, scale_dtype, g, bs.stored);
                 if (has_nan && nan_count) atomicAdd(nan_count, 1);
@@ -261,15 +262,26 @@ int launch_mode(const void *x, bool is_bf16, int64_t rows, int64_t cols, int bm,
                                q, scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
     } else if (bm == 1 && bn == 128 && aligned16) {
         constexpr int PASSES = 4;
-        int64_t groups = rows * (cols / 128);
-        int64_t wgs = (groups + 16 * PASSES - 1) / (16 * PASSES);
-        if (wgs > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_quant_fp8_block: too many groups");
-        if (is_bf16)
-            hipLaunchKernelGGL((quant_group128<true, MODE, PASSES>), dim3((unsigned)wgs), dim3(256), 0, st, x, groups,
-                               q, scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
-        else
-            hipLaunchKernelGGL((quant_group128<false, MODE, PASSES>), dim3((unsigned)wgs), dim3(256), 0, st, x, groups,
-                               q, scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
+        const int64_t groups = rows * (cols / 128), per_wg = 16 * PASSES;
+        const int64_t full = groups / per_wg, tail0 = full * per_wg;
+        if (full > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_quant_fp8_block: too many groups");
+        // full workgroups run without bounds tests; the ragged end is a one-workgroup launch
+        if (full > 0) {
+            if (is_bf16)
+                hipLaunchKernelGGL((quant_group128<true, MODE, PASSES, false>), dim3((unsigned)full), dim3(256), 0, st, x,
+                                   (int64_t)0, groups, q, scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
+            else
+                hipLaunchKernelGGL((quant_group128<false, MODE, PASSES, false>), dim3((unsigned)full), dim3(256), 0, st, x,
+                                   (int64_t)0, groups, q, scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
+        }
+        if (tail0 < groups) {
+            if (is_bf16)
+                hipLaunchKernelGGL((quant_group128<true, MODE, PASSES, true>), dim3(1), dim3(256), 0, st, x, tail0, groups, q,
+                                   scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
+            else
+                hipLaunchKernelGGL((quant_group128<false, MODE, PASSES, true>), dim3(1), dim3(256), 0, st, x, tail0, groups, q,
+                                   scale_out, scale_dtype, amax_floor, zero_rule, nan_count);
+        }
     } else {
         int64_t blocks_c = cols / bn, blocks = (rows / bm) * blocks_c;
         if (blocks > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_quant_fp8_block: too many blocks");
