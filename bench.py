@@ -146,6 +146,28 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_extras:
+        # -------------------------------------------------------------- calibration: a plain device copy of known size
+        # (what a streaming read+write kernel reaches on this box; also the reference kernel for scaling the
+        # FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this script)
+        for mib in (32, 256):
+            n = mib * 1024 * 1024 // 2
+            sets = max(2, 768 // mib)
+            src = [torch.empty(n, dtype=torch.bfloat16, device=dev).normal_() for _ in range(sets)]
+            dst = [torch.empty(n, dtype=torch.bfloat16, device=dev) for _ in range(sets)]
+            ms_c, _ = time_launches([(lambda i=i: dst[i].copy_(src[i])) for i in range(sets)], 24, 6)
+            extras[f"copy_{mib}MiB_calibration"] = {"ms": ms_c, "GB/s": 4.0 * n / ms_c / 1e6, "hbm_frac": 4.0 * n / ms_c / 1e6 / HBM_PEAK_GBS,
+                                                   "bytes": 4 * n, "kernel": "torch elementwise copy (bf16)"}
+            del src, dst
+            torch.cuda.empty_cache()
+        # -------------------------------------------------------------- config 2 operand: weight quantisation at full size
+        w_big = randn(N, K, std=0.02)
+        wq_big = torch.empty(N, K, dtype=torch.uint8, device=dev)
+        ws_big = torch.empty(N // 128, K // 128, dtype=torch.float32, device=dev)
+        ms_wq, _ = time_launches([lambda: quant_into(w_big, 128, 128, wq_big, ws_big)], 10, 3)
+        extras["c2_weight_quant_128x128"] = {"ms": ms_wq, "GB/s": N * K * 3 / ms_wq / 1e6, "hbm_frac": N * K * 3 / ms_wq / 1e6 / HBM_PEAK_GBS,
+                                             "bytes": N * K * 3}
+        del w_big, wq_big, ws_big
+        torch.cuda.empty_cache()
         # -------------------------------------------------------------- config 1: 128x128 quant / dequant
         R = C = 4096
         sets = 12                                   # 12 x (32 + 16 MiB) > 256 MB
