@@ -227,14 +227,13 @@ __device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__res
         aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
         boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
     }
-    // activation scale offsets of the lane's four block rows
+    // activation scales travel in groups of four K steps through LDS: waves 0..3 copy one row per lane
     int64_t arow[4];
-    uint32_t soff[4];
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-        arow[mb] = m0 + wm * 64 + mb * 16 + l16;
-        soff[mb] = (uint32_t)((arow[mb] < M ? arow[mb] : M - 1) * kblocks * 4);
-    }
+    for (int mb = 0; mb < 4; ++mb) arow[mb] = m0 + wm * 64 + mb * 16 + l16;
+    const int64_t srow = m0 + (wave & 3) * 64 + lane;
+    const uint32_t soff = (uint32_t)((srow < M ? srow : M - 1) * kblocks * 4);
+    const uint32_t copies = __builtin_amdgcn_readfirstlane(wave < 4 ? 1u : 0u);
     // weight scale row of this wave (its 128 columns lie in one scale block)
     const int64_t wcol0 = n0 + wn * 128;
     int64_t sblk = wcol0 >> 7;
@@ -250,6 +249,7 @@ __device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__res
     const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
     const uint32_t brd0 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq) * 16;
     const uint32_t brd1 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
+    const uint32_t srd = lds0 + 4 * A_BYTES + arow_l * 16;
 
     f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
     asm volatile(
@@ -258,9 +258,9 @@ __device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__res
           "={v[192:207]}"(acc4), "={v[208:223]}"(acc5), "={v[224:239]}"(acc6), "={v[240:255]}"(acc7)
         : [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]),
           [boff0] "v"(boff[0]), [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]),
-          [soff0] "v"(soff[0]), [soff1] "v"(soff[1]), [soff2] "v"(soff[2]), [soff3] "v"(soff[3]),
-          [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),
-          [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [ksteps] "s"(kblocks)
+          [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),
+          [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base),
+          [trips] "s"(kblocks / 4), [copies] "s"(copies)
         : "memory", "scc",
           "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45",
           "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61",
@@ -269,7 +269,8 @@ __device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__res
           "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107",
           "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120",
           "v121", "v122", "v123", "v124", "v125", "v126", "v127",
-          "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55");
+          "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55",
+          "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63");
 
     const f32x16v accs[8] = {acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7};
 #pragma unroll
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm(const uint8_t *__restric
                                                         int64_t M, int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
                                                         void *__restrict__ C, int64_t ldc, int out_dtype)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB + 8192];   // two operand stages + scale groups
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
     big_tile_asm(smem, Aq, As, Bq, Bs, tm * BM, M, tn * 256, N, K, C, ldc, out_dtype);
@@ -312,7 +313,7 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm_grouped(const uint8_t *_
                                                                 int64_t K, int64_t max_mtiles, int64_t tiles_n,
                                                                 void *__restrict__ C, int out_dtype)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * BM * KB + 8192];   // two operand stages + scale groups
     __shared__ int scan[THREADS];
     __shared__ int found_e, found_first;
     int64_t gmt, tn;
@@ -363,6 +364,14 @@ int launch_nb(const void *Aq, const void *As, const void *Bq, const void *Bs, in
 namespace lowp {
 namespace gemm {
 
+// The hand-scheduled loop addresses operands with 32-bit offsets and moves scales in 16-byte groups
+// of four K steps.
+static bool asm_shape_ok(const void *As, const void *Bs, int64_t M, int64_t N, int64_t K)
+{
+    return K % 512 == 0 && (((uintptr_t)As | (uintptr_t)Bs) & 15) == 0 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
+           M * (K / 128) * 4 < 0xFFFFFFFFll;
+}
+
 // Picks the tile width whose last round of tiles wastes the fewest CU slots.
 int choose_big_tn(int64_t M, int64_t N)
 {
@@ -389,8 +398,7 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
         return launch_nb<SDT, 4>(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);                            \
     } while (0)
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;       // tuning / test aid
-    if (!no_asm && scale_dtype == LP_F32 && tn == 256 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
-        M * (K / 128) * 4 < 0xFFFFFFFFll) {
+    if (!no_asm && scale_dtype == LP_F32 && tn == 256 && asm_shape_ok(As, Bs, M, N, K)) {
         const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
         const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
@@ -404,11 +412,10 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
 }
 
 // Grouped problems on the hand-scheduled kernel: fp32 scales, N a multiple of 256, offsets that fit 32 bits.
-bool big_grouped_ok(int scale_dtype, int64_t M_total, int64_t N, int64_t K)
+bool big_grouped_ok(const void *As, const void *Bs, int scale_dtype, int64_t M_total, int64_t N, int64_t K)
 {
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;
-    return !no_asm && scale_dtype == LP_F32 && N % 256 == 0 && M_total * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
-           M_total * (K / 128) * 4 < 0xFFFFFFFFll;
+    return !no_asm && scale_dtype == LP_F32 && N % 256 == 0 && asm_shape_ok(As, Bs, M_total, N, K);
 }
 
 int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,

@@ -14,10 +14,18 @@ Register plan (per lane, all physical):
   v[48:63]   wf[buf]        = v[48 + 8*buf : 55 + 8*buf]      weight fragment of block nb
   v[44:47]   sc[mb]         = As[m, kb] * Bs[n/128, kb]
   v[40:43]   raw As of the next step
+  v38, v39   LDS address of the lane's activation scales: buffer half 0, half in use
   v[30:37]   LDS read addresses: stage 0 (a0, a1, b0, b1) and stage 1
-  s[40:55]   bases, counters, M0 base, weight scale of this / the next step
+  s[40:55]   bases, counters, M0 base, buffer toggles
+  s[56:59], s[60:63]  weight scales of this / the next group of four steps
 One K step = 128 bytes of K = one scale block: 8 DMA instructions for the next stage, 10 + 14
 LDS fragment reads, 32 MFMA 16x16x128 (zero C), 128 FMA folds.
+
+Scales: a gather of one activation scale per lane per step costs the texture path about as much as
+the operand copies themselves (16 distinct cache lines per instruction), so the scales move in groups
+of four K steps: waves 0..3 copy 16 bytes per activation row (256 rows) straight into a small LDS
+buffer with one global_load_lds_dwordx4 each, the four weight scales come with one s_load_dwordx4,
+and each step reads its four activation scales from LDS.  Hence K must be a multiple of 512 here.
 """
 import os
 
@@ -27,6 +35,7 @@ NB, MB = 8, 4
 
 ACC, P, AF, WF, SC, SAN = 128, 96, 64, 48, 44, 40
 RD = {0: (30, 31, 32, 33), 1: (34, 35, 36, 37)}     # a0, a1, b0, b1 per stage
+SCL_LDS = 2 * STAGE          # activation-scale buffer: 2 halves x 256 rows x 16 bytes, after the operand stages
 
 lines = []
 
@@ -55,14 +64,27 @@ def dma(stage):
     emit("s_addc_u32 s43, s43, 0")
 
 
-def load_scales():
-    for mb in range(MB):
-        emit(f"global_load_dword v{SAN + mb}, %[soff{mb}], s[44:45]")
-    emit("s_load_dword s51, s[46:47], 0x0")
-    emit("s_add_u32 s44, s44, 4")
+def scale_group_copy_body(tag):
+    """Copy the activation scales of the next group of four K steps into LDS (waves 0..3, one row per lane,
+    16 bytes each) and load the four weight scales of that group into s[60:63]."""
+    emit("s_cmp_eq_u32 s53, 0")
+    emit(f"s_cbranch_scc1 Lnosc{tag}%=")
+    emit("s_add_u32 m0, s48, s54")
+    emit(f"s_add_u32 m0, m0, {SCL_LDS}")
+    emit("s_nop 0")
+    emit("global_load_lds_dwordx4 %[soff], s[44:45]")
+    emit(f"Lnosc{tag}%=:")
+    emit("s_load_dwordx4 s[60:63], s[46:47], 0x0")
+    emit("s_add_u32 s44, s44, 16")
     emit("s_addc_u32 s45, s45, 0")
-    emit("s_add_u32 s46, s46, 4")
+    emit("s_add_u32 s46, s46, 16")
     emit("s_addc_u32 s47, s47, 0")
+
+
+def read_scales(col):
+    """Activation scales of the lane's four block rows for one K step (column col of the group buffer v39)."""
+    for mb in range(MB):
+        emit(f"ds_read_b32 v{SAN + mb}, v39 offset:{mb * 256 + col * 4}")
 
 
 def compute(stage):
@@ -92,16 +114,29 @@ def compute(stage):
             emit(f"v_fmac_f32 v{ACC + 16 * (NB - 1) + 4 * mb + r}, v{P + 16 * last + 4 * mb + r}, v{SC + mb}")
 
 
-def step(stage, label):
-    # scales of this step were loaded one step ahead
+def step(stage, c):
+    """K step c (0..3) of a trip.  s50 = 1 on the last trip."""
     for mb in range(MB):
-        emit(f"v_mul_f32 v{SC + mb}, s51, v{SAN + mb}")
-    emit("s_sub_u32 s49, s49, 1")
-    emit("s_cmp_eq_u32 s49, 0")
-    emit(f"s_cbranch_scc1 {label}_nodma%=")
-    dma(stage ^ 1)
-    load_scales()
-    emit(f"{label}_nodma%=:")
+        emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
+    if c == 0:
+        # next group of scales: into the other half of the scale buffer
+        emit("s_cmp_eq_u32 s50, 1")
+        emit("s_cbranch_scc1 Lnogrp%=")
+        emit("s_xor_b32 s54, s54, 4096")
+        scale_group_copy_body("b")
+        emit("Lnogrp%=:")
+    if c == 3:
+        emit("s_cmp_eq_u32 s50, 1")
+        emit("s_cbranch_scc1 Lnodma%=")
+        dma(stage ^ 1)
+        emit("Lnodma%=:")
+        # the next step belongs to the next group
+        emit("s_xor_b32 s55, s55, 4096")
+        emit("v_add_u32 v39, s55, v38")
+        read_scales(0)
+    else:
+        dma(stage ^ 1)
+        read_scales(c + 1)
     compute(stage)
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     emit("s_barrier")
@@ -114,25 +149,34 @@ def main():
     emit("s_mov_b64 s[44:45], %[sbase]")
     emit("s_mov_b64 s[46:47], %[bsptr]")
     emit("s_mov_b32 s48, %[m0base]")
-    emit("s_mov_b32 s49, %[ksteps]")
+    emit("s_mov_b32 s49, %[trips]")
+    emit("s_mov_b32 s53, %[copies]")
+    emit("s_mov_b32 s54, 0")
+    emit("s_mov_b32 s55, 0")
     for i, name in enumerate(("ard0", "ard1", "brd0", "brd1")):
         emit(f"v_mov_b32 v{RD[0][i]}, %[{name}]")
         emit(f"v_add_u32 v{RD[1][i]}, {STAGE}, %[{name}]")
+    emit("v_mov_b32 v38, %[srd]")
+    emit("v_mov_b32 v39, %[srd]")
     for r in range(128):
         emit(f"v_mov_b32 v{ACC + r}, 0")
+    scale_group_copy_body("a")
     dma(0)
-    load_scales()
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     emit("s_barrier")
-    # ---- main loop, two K steps per trip (one per LDS stage)
+    read_scales(0)
+    emit("s_waitcnt lgkmcnt(0)")
+    # ---- main loop: one trip = four K steps = one group of scales
     emit("Lloop%=:")
-    step(0, "Ls0")
+    emit("s_mov_b64 s[56:57], s[60:61]")
+    emit("s_mov_b64 s[58:59], s[62:63]")
+    emit("s_sub_u32 s49, s49, 1")
     emit("s_cmp_eq_u32 s49, 0")
-    emit("s_cbranch_scc1 Lend%=")
-    step(1, "Ls1")
-    emit("s_cmp_lg_u32 s49, 0")
+    emit("s_cselect_b32 s50, 1, 0")
+    for c in range(4):
+        step(c & 1, c)
+    emit("s_cmp_lg_u32 s50, 1")
     emit("s_cbranch_scc1 Lloop%=")
-    emit("Lend%=:")
 
     here = os.path.dirname(os.path.abspath(__file__))
     with open(os.path.join(here, "gemm_big_loop.inc"), "w") as f:
