@@ -241,14 +241,15 @@ __device__ __forceinline__ void big_tile_asm(uint8_t *smem, const uint8_t *__res
     const float *bs_ptr = Bs + sblk * kblocks;
     const uint64_t bs_u = uniform(bs_ptr);
 
-    // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0)
+    // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
+    // Layout: activation stages at 0 / 32 KB, weight stages at 64 / 96 KB, scale groups at 128 KB.
     const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
     const uint32_t m0base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const int arow_l = wm * 64 + l16, brow_l = wn * 128 + l16;
     const uint32_t ard0 = lds0 + arow_l * KB + swz(arow_l, 2 * lq) * 16;
     const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
-    const uint32_t brd0 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq) * 16;
-    const uint32_t brd1 = lds0 + A_BYTES + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
+    const uint32_t brd0 = lds0 + 2 * A_BYTES + brow_l * KB + swz(brow_l, 2 * lq) * 16;
+    const uint32_t brd1 = lds0 + 2 * A_BYTES + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
     const uint32_t srd = lds0 + 4 * A_BYTES + arow_l * 16;
 
     f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;

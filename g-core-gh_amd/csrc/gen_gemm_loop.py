@@ -3,39 +3,45 @@
 FP8 GEMM (fp32 scales) as one inline-asm string for gfx950.
 
 Why generated assembly: the loop must keep eight MFMA results in flight while the VALU folds
-the previous block into the fp32 accumulators and the LDS streams the next weight fragment.
-With 128 accumulator registers per lane the compiler serialises MFMA -> fold -> MFMA instead;
-fixing the register plan by hand removes that.
+the previous block into the fp32 accumulators and the LDS streams the weight fragments two
+blocks ahead.  With 128 accumulator registers per lane the compiler serialises
+MFMA -> fold -> MFMA instead; fixing the register plan by hand removes that.
 
 Register plan (per lane, all physical):
   v[128:255] acc[nb][mb][r] = v[128 + 16*nb + 4*mb + r]      (outputs of the asm statement)
   v[96:127]  p[buf][mb][r]  = v[96 + 16*buf + 4*mb + r]       MFMA results of block nb (buf = nb & 1)
   v[64:95]   af[mb]         = v[64 + 8*mb : 71 + 8*mb]        activation fragments of this K step
-  v[48:63]   wf[buf]        = v[48 + 8*buf : 55 + 8*buf]      weight fragment of block nb
-  v[44:47]   sc[mb]         = As[m, kb] * Bs[n/128, kb]
-  v[40:43]   raw As of the next step
-  v38, v39   LDS address of the lane's activation scales: buffer half 0, half in use
-  v[30:37]   LDS read addresses: stage 0 (a0, a1, b0, b1) and stage 1
+  v[48:63], v[36:43]  wf[nb % 3]                              weight fragment of block nb (three buffers)
+  v[44:47]   sc[mb]         = As[m, kb] * Bs[n/128, kb]       (raw As of the next step from the end of a step on)
+  v34, v35   LDS address of the lane's activation scales: buffer half 0, half in use
+  v[30:33]   LDS fragment read addresses a0, a1, b0, b1 (stage and block go into the offset field)
   s[40:55]   bases, counters, M0 base, buffer toggles
   s[56:59], s[60:63]  weight scales of this / the next group of four steps
-One K step = 128 bytes of K = one scale block: 8 DMA instructions for the next stage, 10 + 14
-LDS fragment reads, 32 MFMA 16x16x128 (zero C), 128 FMA folds.
+LDS: activation stages at 0 and 32 KB, weight stages at 64 and 96 KB, scale groups at 128 KB.
+One K step = 128 bytes of K = one scale block: 8 DMA instructions for the next stage, 8 + 16
+LDS fragment reads, 32 MFMA 16x16x128 (zero C), 128 FMA folds.  Fragment reads are waited for
+one at a time (counted lgkmcnt), so the first MFMA of a step starts after 4 of the 14 reads.
 
 Scales: a gather of one activation scale per lane per step costs the texture path about as much as
 the operand copies themselves (16 distinct cache lines per instruction), so the scales move in groups
 of four K steps: waves 0..3 copy 16 bytes per activation row (256 rows) straight into a small LDS
 buffer with one global_load_lds_dwordx4 each, the four weight scales come with one s_load_dwordx4,
 and each step reads its four activation scales from LDS.  Hence K must be a multiple of 512 here.
+The scalar load shares lgkmcnt with the LDS reads and returns out of order, so it is only issued
+where no counted wait follows before the next full wait.
 """
 import os
 
 A_BYTES = 256 * 128
-STAGE = 2 * A_BYTES          # 256 activation rows + 256 weight rows, 128 bytes each
+A_LDS = (0, A_BYTES)                       # activation stages
+B_LDS = (2 * A_BYTES, 3 * A_BYTES)         # weight stages
+SCL_LDS = 4 * A_BYTES                      # activation-scale buffer: 2 halves x 256 rows x 16 bytes
 NB, MB = 8, 4
 
-ACC, P, AF, WF, SC, SAN = 128, 96, 64, 48, 44, 40
-RD = {0: (30, 31, 32, 33), 1: (34, 35, 36, 37)}     # a0, a1, b0, b1 per stage
-SCL_LDS = 2 * STAGE          # activation-scale buffer: 2 halves x 256 rows x 16 bytes, after the operand stages
+ACC, P, AF, SC, SAN = 128, 96, 64, 44, 40
+WFB = (48, 56)
+RA0, RA1, RB0, RB1 = 30, 31, 32, 33
+SRD0, SRD = 34, 35
 
 lines = []
 
@@ -51,11 +57,11 @@ def vr(base, n):
 def dma(stage):
     """Issue the 8 global->LDS copies of one stage and advance the operand bases by one K step."""
     for i in range(4):
-        emit(f"s_add_u32 m0, s48, {stage * STAGE + i * 8192}")
+        emit(f"s_add_u32 m0, s48, {A_LDS[stage] + i * 8192}")
         emit("s_nop 0")
         emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
     for i in range(4):
-        emit(f"s_add_u32 m0, s48, {stage * STAGE + A_BYTES + i * 8192}")
+        emit(f"s_add_u32 m0, s48, {B_LDS[stage] + i * 8192}")
         emit("s_nop 0")
         emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
     emit("s_add_u32 s40, s40, 128")
@@ -64,9 +70,9 @@ def dma(stage):
     emit("s_addc_u32 s43, s43, 0")
 
 
-def scale_group_copy_body(tag):
-    """Copy the activation scales of the next group of four K steps into LDS (waves 0..3, one row per lane,
-    16 bytes each) and load the four weight scales of that group into s[60:63]."""
+def scale_group_copy(tag):
+    """Copy the activation scales of the next group of four K steps into LDS (waves 0..3, one row per
+    lane, 16 bytes each)."""
     emit("s_cmp_eq_u32 s53, 0")
     emit(f"s_cbranch_scc1 Lnosc{tag}%=")
     emit("s_add_u32 m0, s48, s54")
@@ -74,48 +80,46 @@ def scale_group_copy_body(tag):
     emit("s_nop 0")
     emit("global_load_lds_dwordx4 %[soff], s[44:45]")
     emit(f"Lnosc{tag}%=:")
-    emit("s_load_dwordx4 s[60:63], s[46:47], 0x0")
     emit("s_add_u32 s44, s44, 16")
     emit("s_addc_u32 s45, s45, 0")
+
+
+def weight_scale_load():
+    """The four weight scales of the next group into s[60:63]."""
+    emit("s_load_dwordx4 s[60:63], s[46:47], 0x0")
     emit("s_add_u32 s46, s46, 16")
     emit("s_addc_u32 s47, s47, 0")
 
 
+def read_frag(dst, addr0, addr1, off):
+    emit(f"ds_read_b128 {vr(dst, 4)}, v{addr0} offset:{off}")
+    emit(f"ds_read_b128 {vr(dst + 4, 4)}, v{addr1} offset:{off}")
+
+
 def read_scales(col):
-    """Activation scales of the lane's four block rows for one K step (column col of the group buffer v39)."""
+    """Raw activation scales of the lane's four block rows for one K step (column col of the group half at v35)."""
     for mb in range(MB):
-        emit(f"ds_read_b32 v{SAN + mb}, v39 offset:{mb * 256 + col * 4}")
+        emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256 + col * 4}")
 
 
-def compute(stage):
-    a0, a1, b0, b1 = RD[stage]
-    for mb in range(MB):
-        emit(f"ds_read_b128 {vr(AF + 8 * mb, 4)}, v{a0} offset:{mb * 2048}")
-        emit(f"ds_read_b128 {vr(AF + 8 * mb + 4, 4)}, v{a1} offset:{mb * 2048}")
-    emit(f"ds_read_b128 {vr(WF, 4)}, v{b0}")
-    emit(f"ds_read_b128 {vr(WF + 4, 4)}, v{b1}")
-    emit("s_waitcnt lgkmcnt(0)")
-    for nb in range(NB):
-        cur, nxt = nb & 1, (nb & 1) ^ 1
-        if nb + 1 < NB:
-            emit(f"ds_read_b128 {vr(WF + 8 * nxt, 4)}, v{b0} offset:{(nb + 1) * 2048}")
-            emit(f"ds_read_b128 {vr(WF + 8 * nxt + 4, 4)}, v{b1} offset:{(nb + 1) * 2048}")
-        for mb in range(MB):
-            emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * cur + 4 * mb, 4)}, {vr(WF + 8 * cur, 8)}, {vr(AF + 8 * mb, 8)}, 0")
-            if nb > 0:
-                for r in range(4):
-                    emit(f"v_fmac_f32 v{ACC + 16 * (nb - 1) + 4 * mb + r}, v{P + 16 * nxt + 4 * mb + r}, v{SC + mb}")
-        if nb + 1 < NB:
-            emit("s_waitcnt lgkmcnt(0)")
-    # fold of the last block: the 12 folds of mb 0..2 separate the last MFMA from the read of its result
-    last = (NB - 1) & 1
-    for mb in range(MB):
-        for r in range(4):
-            emit(f"v_fmac_f32 v{ACC + 16 * (NB - 1) + 4 * mb + r}, v{P + 16 * last + 4 * mb + r}, v{SC + mb}")
+def mfma(nb, mb):
+    emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * (nb & 1) + 4 * mb, 4)}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, 0")
+
+
+def fold(nb, mb):
+    for r in range(4):
+        emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * (nb & 1) + 4 * mb + r}, v{SC + mb}")
 
 
 def step(stage, c):
-    """K step c (0..3) of a trip.  s50 = 1 on the last trip."""
+    """K step c (0..3) of a trip; s50 = 1 on the last trip.
+
+    On entry the fragments wf0 and af0..3 of this step are already on their way (10 LDS reads issued in the
+    previous step's last block).  The stage flip (wait for the copies of the next stage, barrier, issue the
+    copies of the stage after it, first fragment reads of the next step) happens inside the last block, so the
+    matrix pipe keeps working across it."""
+    aoff, boff = A_LDS[stage], B_LDS[stage] - B_LDS[0]
+    naoff, nboff = A_LDS[stage ^ 1], B_LDS[stage ^ 1] - B_LDS[0]
     for mb in range(MB):
         emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
     if c == 0:
@@ -123,23 +127,47 @@ def step(stage, c):
         emit("s_cmp_eq_u32 s50, 1")
         emit("s_cbranch_scc1 Lnogrp%=")
         emit("s_xor_b32 s54, s54, 4096")
-        scale_group_copy_body("b")
+        scale_group_copy("b")
+        weight_scale_load()
         emit("Lnogrp%=:")
     if c == 3:
-        emit("s_cmp_eq_u32 s50, 1")
-        emit("s_cbranch_scc1 Lnodma%=")
-        dma(stage ^ 1)
-        emit("Lnodma%=:")
         # the next step belongs to the next group
         emit("s_xor_b32 s55, s55, 4096")
-        emit("v_add_u32 v39, s55, v38")
-        read_scales(0)
-    else:
-        dma(stage ^ 1)
-        read_scales(c + 1)
-    compute(stage)
-    emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
-    emit("s_barrier")
+        emit(f"v_add_u32 v{SRD}, s55, v{SRD0}")
+    read_frag(WFB[1], RB0, RB1, boff + 2048)
+    # LDS queue now: wf0, af0..3, wf1 = 12 reads
+    for mb in range(MB):
+        emit(f"s_waitcnt lgkmcnt({8 - 2 * mb})")
+        mfma(0, mb)
+    read_scales((c + 1) & 3)
+    for nb in range(1, NB):
+        if nb + 1 < NB:
+            read_frag(WFB[(nb + 1) & 1], RB0, RB1, boff + (nb + 1) * 2048)
+        if nb == 1:
+            emit("s_waitcnt lgkmcnt(6)")        # 4 scales and wf2 may still be outstanding
+        elif nb + 1 < NB:
+            emit("s_waitcnt lgkmcnt(2)")
+        else:
+            # stage flip: every wave has read all of this stage and its share of the next stage has landed
+            emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+            emit("s_barrier")
+            read_frag(WFB[0], RB0, RB1, nboff)
+        for mb in range(MB):
+            mfma(nb, mb)
+            fold(nb - 1, mb)
+            if nb + 1 == NB:
+                read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
+                if mb == 0:
+                    # copies of the stage after the next one overwrite the stage just finished
+                    if c >= 2:
+                        emit("s_cmp_eq_u32 s50, 1")
+                        emit(f"s_cbranch_scc1 Lnodma{c}%=")
+                    dma(stage)
+                    if c >= 2:
+                        emit(f"Lnodma{c}%=:")
+    # fold of the last block: the 12 folds of mb 0..2 separate the last MFMA from the read of its result
+    for mb in range(MB):
+        fold(NB - 1, mb)
 
 
 def main():
@@ -153,19 +181,22 @@ def main():
     emit("s_mov_b32 s53, %[copies]")
     emit("s_mov_b32 s54, 0")
     emit("s_mov_b32 s55, 0")
-    for i, name in enumerate(("ard0", "ard1", "brd0", "brd1")):
-        emit(f"v_mov_b32 v{RD[0][i]}, %[{name}]")
-        emit(f"v_add_u32 v{RD[1][i]}, {STAGE}, %[{name}]")
-    emit("v_mov_b32 v38, %[srd]")
-    emit("v_mov_b32 v39, %[srd]")
+    for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
+        emit(f"v_mov_b32 v{reg}, %[{name}]")
     for r in range(128):
         emit(f"v_mov_b32 v{ACC + r}, 0")
-    scale_group_copy_body("a")
+    scale_group_copy("a")
+    weight_scale_load()
     dma(0)
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     emit("s_barrier")
-    read_scales(0)
+    dma(1)                                   # K >= 512: there are at least four steps
+    for mb in range(MB):
+        emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256}")
     emit("s_waitcnt lgkmcnt(0)")
+    read_frag(WFB[0], RB0, RB1, 0)
+    for mb in range(MB):
+        read_frag(AF + 8 * mb, RA0, RA1, mb * 2048)
     # ---- main loop: one trip = four K steps = one group of scales
     emit("Lloop%=:")
     emit("s_mov_b64 s[56:57], s[60:61]")
@@ -177,6 +208,7 @@ def main():
         step(c & 1, c)
     emit("s_cmp_lg_u32 s50, 1")
     emit("s_cbranch_scc1 Lloop%=")
+    emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
     here = os.path.dirname(os.path.abspath(__file__))
     with open(os.path.join(here, "gemm_big_loop.inc"), "w") as f:
