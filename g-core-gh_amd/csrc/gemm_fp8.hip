@@ -353,6 +353,9 @@ static int check_gemm_args(const char *name, const void *Aq, const void *As, con
 static int launch_small(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M,
                         int64_t N, int64_t K, void *C, int64_t ldc, int out_dtype, hipStream_t st)
 {
+    static const char *mid_min = getenv("LP_GEMM_MID_MIN_M");       // tuning aid
+    if (M >= (mid_min ? atoi(mid_min) : 64) && gemm::mid_asm_ok(As, Bs, scale_dtype, M, N, K))
+        return gemm::launch_mid_asm(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);
     const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
     const int64_t grid = padded_grid(tiles_m, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");

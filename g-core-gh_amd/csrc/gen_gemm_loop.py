@@ -32,19 +32,37 @@ where no counted wait follows before the next full wait.
 """
 import os
 
-A_BYTES = 256 * 128
-A_LDS = (0, A_BYTES)                       # activation stages
-B_LDS = (2 * A_BYTES, 3 * A_BYTES)         # weight stages
-SCL_LDS = 4 * A_BYTES                      # activation-scale buffer: 2 halves x 256 rows x 16 bytes
-NB, MB = 8, 4
+MB = 4                                     # 16-row blocks per wave (64 activation rows)
+
+
+def configure(tm, tn, waves_m, waves_n, ksub):
+    """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128."""
+    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, lines
+    assert tm == 64 * waves_m
+    WAVES = waves_m * waves_n
+    KSUB = ksub
+    A_BYTES, B_BYTES = tm * 128, tn * 128
+    SCL_LDS = 2 * ksub * (A_BYTES + B_BYTES)               # activation-scale buffer: 2 halves x tm rows x 16 bytes
+    SCL_HALF = tm * 16
+    NB = tn // waves_n // 16
+    assert (tm // 8) % WAVES == 0 and (tn // 8) % WAVES == 0
+    lines = []
+
+
+def a_lds(stage, sub):
+    """LDS offset of the activation rows of K block sub of a stage (all activation blocks come first)."""
+    return (stage * KSUB + sub) * A_BYTES
+
+
+def b_lds(stage, sub):
+    """Same for the weight rows, relative to the first weight block (at 2 * KSUB * A_BYTES)."""
+    return (stage * KSUB + sub) * B_BYTES
+
 
 ACC, P, AF, SC, SAN = 128, 96, 64, 44, 40
 WFB = (48, 56)
 RA0, RA1, RB0, RB1 = 30, 31, 32, 33
 SRD0, SRD = 34, 35
-
-lines = []
-
 
 def emit(s):
     lines.append(s)
@@ -55,19 +73,21 @@ def vr(base, n):
 
 
 def dma(stage):
-    """Issue the 8 global->LDS copies of one stage and advance the operand bases by one K step."""
-    for i in range(4):
-        emit(f"s_add_u32 m0, s48, {A_LDS[stage] + i * 8192}")
-        emit("s_nop 0")
-        emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
-    for i in range(4):
-        emit(f"s_add_u32 m0, s48, {B_LDS[stage] + i * 8192}")
-        emit("s_nop 0")
-        emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
-    emit("s_add_u32 s40, s40, 128")
-    emit("s_addc_u32 s41, s41, 0")
-    emit("s_add_u32 s42, s42, 128")
-    emit("s_addc_u32 s43, s43, 0")
+    """Issue the global->LDS copies of one stage; the operand bases advance by one K block after each."""
+    bbase = 2 * KSUB * A_BYTES
+    for sub in range(KSUB):
+        for i in range(A_BYTES // 1024 // WAVES):
+            emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
+            emit("s_nop 0")
+            emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
+        for i in range(B_BYTES // 1024 // WAVES):
+            emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + i * WAVES * 1024}")
+            emit("s_nop 0")
+            emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
+        emit("s_add_u32 s40, s40, 128")
+        emit("s_addc_u32 s41, s41, 0")
+        emit("s_add_u32 s42, s42, 128")
+        emit("s_addc_u32 s43, s43, 0")
 
 
 def scale_group_copy(tag):
@@ -111,28 +131,31 @@ def fold(nb, mb):
         emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * (nb & 1) + 4 * mb + r}, v{SC + mb}")
 
 
-def step(stage, c):
+def step(c):
     """K step c (0..3) of a trip; s50 = 1 on the last trip.
 
     On entry the fragments wf0 and af0..3 of this step are already on their way (10 LDS reads issued in the
-    previous step's last block).  The stage flip (wait for the copies of the next stage, barrier, issue the
-    copies of the stage after it, first fragment reads of the next step) happens inside the last block, so the
-    matrix pipe keeps working across it."""
-    aoff, boff = A_LDS[stage], B_LDS[stage] - B_LDS[0]
-    naoff, nboff = A_LDS[stage ^ 1], B_LDS[stage ^ 1] - B_LDS[0]
+    previous step's last block).  After the last K block of a stage comes the stage flip (wait for the copies
+    of the next stage, barrier, issue the copies that overwrite the stage just finished); it and the first
+    fragment reads of the next step happen inside the last block, so the matrix pipe keeps working across it."""
+    stage, sub = (c // KSUB) & 1, c % KSUB
+    flip = sub == KSUB - 1
+    nstage, nsub = (stage ^ 1, 0) if flip else (stage, sub + 1)
+    aoff, boff = a_lds(stage, sub), b_lds(stage, sub)
+    naoff, nboff = a_lds(nstage, nsub), b_lds(nstage, nsub)
     for mb in range(MB):
         emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
     if c == 0:
         # next group of scales: into the other half of the scale buffer
         emit("s_cmp_eq_u32 s50, 1")
         emit("s_cbranch_scc1 Lnogrp%=")
-        emit("s_xor_b32 s54, s54, 4096")
+        emit(f"s_xor_b32 s54, s54, {SCL_HALF}")
         scale_group_copy("b")
         weight_scale_load()
         emit("Lnogrp%=:")
     if c == 3:
         # the next step belongs to the next group
-        emit("s_xor_b32 s55, s55, 4096")
+        emit(f"s_xor_b32 s55, s55, {SCL_HALF}")
         emit(f"v_add_u32 v{SRD}, s55, v{SRD0}")
     read_frag(WFB[1], RB0, RB1, boff + 2048)
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
@@ -144,33 +167,37 @@ def step(stage, c):
         if nb + 1 < NB:
             read_frag(WFB[(nb + 1) & 1], RB0, RB1, boff + (nb + 1) * 2048)
         if nb == 1:
-            emit("s_waitcnt lgkmcnt(6)")        # 4 scales and wf2 may still be outstanding
+            emit(f"s_waitcnt lgkmcnt({6 if NB > 2 else 4})")        # 4 scales and wf2 may still be outstanding
         elif nb + 1 < NB:
             emit("s_waitcnt lgkmcnt(2)")
-        else:
-            # stage flip: every wave has read all of this stage and its share of the next stage has landed
-            emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
-            emit("s_barrier")
+        if nb + 1 == NB:
+            if flip:
+                # every wave has read all of this stage and its share of the next stage has landed
+                emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+                emit("s_barrier")
+            else:
+                emit("s_waitcnt lgkmcnt(0)")
             read_frag(WFB[0], RB0, RB1, nboff)
         for mb in range(MB):
             mfma(nb, mb)
             fold(nb - 1, mb)
             if nb + 1 == NB:
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
-                if mb == 0:
-                    # copies of the stage after the next one overwrite the stage just finished
-                    if c >= 2:
+                if mb == 0 and flip:
+                    # copies for the K blocks after the next stage overwrite the stage just finished
+                    cond = c + 1 + KSUB >= 4
+                    if cond:
                         emit("s_cmp_eq_u32 s50, 1")
                         emit(f"s_cbranch_scc1 Lnodma{c}%=")
                     dma(stage)
-                    if c >= 2:
+                    if cond:
                         emit(f"Lnodma{c}%=:")
     # fold of the last block: the 12 folds of mb 0..2 separate the last MFMA from the read of its result
     for mb in range(MB):
         fold(NB - 1, mb)
 
 
-def main():
+def generate():
     # ---- prologue
     emit("s_mov_b64 s[40:41], %[abase]")
     emit("s_mov_b64 s[42:43], %[bbase]")
@@ -190,7 +217,7 @@ def main():
     dma(0)
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     emit("s_barrier")
-    dma(1)                                   # K >= 512: there are at least four steps
+    dma(1)                                   # K >= 512: there are at least four steps, which two stages hold at most
     for mb in range(MB):
         emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256}")
     emit("s_waitcnt lgkmcnt(0)")
@@ -205,16 +232,23 @@ def main():
     emit("s_cmp_eq_u32 s49, 0")
     emit("s_cselect_b32 s50, 1, 0")
     for c in range(4):
-        step(c & 1, c)
+        step(c)
     emit("s_cmp_lg_u32 s50, 1")
     emit("s_cbranch_scc1 Lloop%=")
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
+
+
+def main():
     here = os.path.dirname(os.path.abspath(__file__))
-    with open(os.path.join(here, "gemm_big_loop.inc"), "w") as f:
-        f.write("// Generated by gen_gemm_loop.py -- do not edit.\n")
-        for ln in lines:
-            f.write('"' + ln + '\\n"\n')
+    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)),
+                      ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2))):
+        configure(*cfg)
+        generate()
+        with open(os.path.join(here, name), "w") as f:
+            f.write("// Generated by gen_gemm_loop.py -- do not edit.\n")
+            for ln in lines:
+                f.write('"' + ln + '\\n"\n')
 
 
 if __name__ == "__main__":
