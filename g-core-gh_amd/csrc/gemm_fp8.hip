@@ -444,10 +444,3 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
                            (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
     return check_launch("lp_gemm_fp8_grouped");
 }
-
-extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M, int64_t N, int64_t K, void *C,
-                          int out_dtype, lp_stream_t stream)
-{
-    (void)A; (void)B; (void)in_dtype; (void)M; (void)N; (void)K; (void)C; (void)out_dtype; (void)stream;
-    return lowp::fail(LP_ERR_UNSUPPORTED, "lp_gemm_nt: not built yet");
-}

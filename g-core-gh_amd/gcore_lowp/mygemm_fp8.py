@@ -70,7 +70,29 @@ def gemm_fp8_block_scaling_impl(Aq, As, Bq, Bs, BLK_M=64, BLK_N=128, BLK_K=128, 
     return C.to(home)
 
 
+_NT_CODES = {torch.float8_e4m3fn: A.E4M3, torch.bfloat16: A.BF16, torch.float32: A.F32}
+
+
 def gemm_impl(A_, B_, block_M=128, block_N=128, block_K=64, dtype=torch.bfloat16, out_dtype=torch.bfloat16,
               accum_dtype=torch.float32):
-    """gfused/mygemm_fp8.py:12-41: C = A B^T, fp8 or bf16 operands, fp32 accumulation."""
-    raise A.LowpError("gemm_impl: the unscaled GEMM is not built yet")
+    """gfused/mygemm_fp8.py:12-41: C[M,N] = A[M,K] B[N,K]^T, operands of `dtype` (e4m3fn or bf16),
+    fp32 accumulation, result cast to `out_dtype` (an e4m3fn result saturates at +-448, as the tile
+    compiler's fp8 conversion does)."""
+    assert accum_dtype == torch.float32
+    if dtype not in (torch.float8_e4m3fn, torch.bfloat16):
+        raise TypeError(f"gemm_impl: operands must be float8_e4m3fn or bfloat16, got {dtype}")
+    if out_dtype not in _NT_CODES:
+        raise TypeError(f"gemm_impl: unsupported out_dtype {out_dtype}")
+    assert A_.dtype == dtype and B_.dtype == dtype, (A_.dtype, B_.dtype, dtype)
+    assert A_.ndim == 2 and B_.ndim == 2 and A_.shape[1] == B_.shape[1]
+    M, K = A_.shape
+    N = B_.shape[0]
+    a, home = A.to_device(A_)
+    dev = a.device
+    a = a.contiguous()
+    b = B_.to(dev).contiguous()
+    C = torch.empty((M, N), dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        A.check(A.lib().lp_gemm_nt(a.data_ptr(), b.data_ptr(), _NT_CODES[dtype], M, N, K, C.data_ptr(),
+                                   _NT_CODES[out_dtype], A.stream_ptr()))
+    return C.to(home)

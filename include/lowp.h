@@ -155,6 +155,9 @@ int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /*
  * Unscaled C = A B^T with fp32 accumulation.  A [M,K], B [N,K], both of
  * in_dtype (LP_E4M3 or LP_BF16); C [M,N] of out_dtype (LP_E4M3, LP_BF16, LP_F32).
+ * K must be a multiple of 128 (LP_E4M3) or 64 (LP_BF16), N a multiple of 16; M is free.
+ * An LP_E4M3 result saturates at +-448 (NaN stays NaN), like the fp8 conversion
+ * of the tile compiler the reference uses.
  * Replaces gemm_impl (gfused/mygemm_fp8.py:12-41).
  */
 int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M, int64_t N, int64_t K,

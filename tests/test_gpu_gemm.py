@@ -172,3 +172,45 @@ def test_grouped_linear_module(G):
     wq, ws = G.quant_fp8_e4m3_scale_e8m0(w)
     out2 = lin(x, (wq, ws), m_splits)
     assert torch.equal(out2, out)
+
+
+# ---------------------------------------------------------------------------------------------
+# unscaled NT GEMM (gemm_impl): shapes and tolerance of the reference's test_gemm_fp8
+NT_SHAPES = [(128, 4096, 2048), (512, 1024, 4096), (2048, 4096, 1024), (4096, 4096, 4096), (200, 1280, 4096),
+             (1000, 16384, 512), (1, 16, 128), (77, 4112, 256)]
+
+
+@pytest.mark.parametrize("shape", NT_SHAPES, ids=lambda s: "M%d_N%d_K%d" % s)
+@pytest.mark.parametrize("kind", ["fp8", "bf16"])
+def test_gemm_impl(G, shape, kind):
+    say("gemm_impl", shape, kind)
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + N + K)
+    dt = torch.float8_e4m3fn if kind == "fp8" else torch.bfloat16
+    a = torch.randn(M, K, generator=g).to(dt)
+    b = torch.randn(N, K, generator=g).to(dt)
+    ref = a.float().cuda() @ b.float().cuda().T
+    for out_dtype in ([torch.float8_e4m3fn, torch.bfloat16] if kind == "fp8" else [torch.bfloat16, torch.float32]):
+        c = G.gemm_impl(a.cuda(), b.cuda(), 128, 128, 64, dtype=dt, out_dtype=out_dtype)
+        assert c.dtype == out_dtype and tuple(c.shape) == (M, N)
+        want = ref.clamp(-448, 448).to(out_dtype) if out_dtype == torch.float8_e4m3fn else ref.to(out_dtype)
+        assert calc_diff(c.float(), want.float()) < 1e-3       # the reference's own bar (test_my_gemm_fp8.py:131)
+        if out_dtype != torch.float8_e4m3fn:
+            err = (c.float() - ref).abs().max() / ref.abs().max()
+            assert err < (1e-2 if out_dtype == torch.bfloat16 else 1e-5), err
+        else:
+            # fp32 accumulation order differs from the library matmul: allow results one code apart
+            ci, wi = c.view(torch.uint8).int(), want.view(torch.uint8).int()
+            assert ((ci - wi).abs() <= 1).float().mean() > 0.9999
+
+
+def test_gemm_impl_errors_and_cpu_inputs(G):
+    a = torch.randn(64, 256).to(torch.bfloat16)
+    b = torch.randn(32, 256).to(torch.bfloat16)
+    c = G.gemm_impl(a, b)                     # CPU in -> CPU out, like every wrapper
+    assert c.device.type == "cpu"
+    assert calc_diff(c.float(), a.float() @ b.float().T) < 1e-4
+    with pytest.raises(TypeError):
+        G.gemm_impl(a.half(), b.half(), dtype=torch.float16)
+    with pytest.raises(Exception):
+        G.gemm_impl(a[:, :100].contiguous(), b[:, :100].contiguous())      # K not a multiple of 64
