@@ -48,6 +48,13 @@ int choose_big_tn(int64_t M, int64_t N);
 int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                int64_t K, void *C, int64_t ldc, int out_dtype, int tn, hipStream_t st);
 
+// gemm_skinny.hip: at most 64 activation rows
+constexpr int kSkinnyBlocks = 7;          // K blocks one workgroup handles
+void skinny_plan(int64_t N, int64_t K, int &splits, int &per);
+int64_t skinny_workspace_bytes(int64_t N, int splits);
+int launch_skinny(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
+                  int64_t K, void *C, int out_dtype, float *ws, int splits, int per, hipStream_t st);
+
 bool mid_asm_ok(const void *As, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K);
 int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
                    int64_t ldc, int out_dtype, hipStream_t st);

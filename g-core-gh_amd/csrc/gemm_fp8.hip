@@ -328,6 +328,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 extern "C" int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+    if (M <= 64) {
+        int sp, per;
+        gemm::skinny_plan(N, K, sp, per);
+        if (per <= gemm::kSkinnyBlocks) return gemm::skinny_workspace_bytes(N, sp);
+    }
     const int64_t tiles = ((M + TM - 1) / TM) * (N / TN);
     const int splits = choose_splits(tiles, K / TK);
     return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
@@ -375,6 +380,17 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     int rc = check_gemm_args("lp_gemm_fp8_block", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
     if (rc) return rc > 0 ? LP_OK : rc;
     hipStream_t st = (hipStream_t)stream;
+    static const bool no_skinny = getenv("LP_GEMM_NO_SKINNY") != nullptr;       // tuning aid
+    if (M <= 64 && !no_skinny) {
+        // decode-sized: the weight-streaming kernel, when the caller gave scratch for its K ranges and one range
+        // fits its window of K blocks (longer ranges are better served by the tiled kernels below)
+        int sp, per;
+        gemm::skinny_plan(N, K, sp, per);
+        const bool ws_ok = sp == 1 || (workspace && workspace_bytes >= gemm::skinny_workspace_bytes(N, sp) &&
+                                       (uintptr_t)workspace % 16 == 0);
+        if (per <= gemm::kSkinnyBlocks && ws_ok)
+            return gemm::launch_skinny(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, (float *)workspace, sp, per, st);
+    }
     const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
     int splits = choose_splits(tiles_m * tiles_n, K / TK);
     if (splits > 1 && (!workspace || workspace_bytes < (int64_t)splits * M * N * 4 || (uintptr_t)workspace % 16)) splits = 1;

@@ -70,7 +70,7 @@ DENSE_SHAPES = [
     # prefill-sized: 256-row kernel (hand-scheduled loop), ragged M / N tails, and the column split
     # between the 256 x 256 and the 128 x 128 kernel (576 tiles on 256 CUs)
     (333, 8320, 512), (200, 16384, 256), (2048, 4224, 384), (256, 32768, 128), (1000, 9216, 640),
-    (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536),
+    (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536), (32, 128, 7168), (48, 16384, 2048), (64, 2048, 7168),
 ]
 
 
