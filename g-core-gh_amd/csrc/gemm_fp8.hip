@@ -325,9 +325,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 }  // namespace
 
+// e8m0 scale bytes -> fp32, for the kernels that only read fp32 scales
+__global__ __launch_bounds__(256) void scales_to_f32(const uint8_t *__restrict__ a, int64_t na, const uint8_t *__restrict__ b,
+                                                     int64_t nb, float *__restrict__ out_a, float *__restrict__ out_b)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < na) out_a[i] = gemm::scale_at<LP_E8M0>(a, i);
+    else if (i < na + nb) out_b[i - na] = gemm::scale_at<LP_E8M0>(b, i - na);
+}
+
+static int64_t round_up(int64_t x, int64_t a) { return (x + a - 1) / a * a; }
+
+// fp32 copies of e8m0 scales sit at the start of the workspace (activation scales, then weight scales)
+static int64_t scale_copy_bytes(int64_t M, int64_t N, int64_t K)
+{
+    return M > 64 && K % 512 == 0 ? round_up(M * (K / 128) * 4, 256) + round_up((N / 128) * (K / 128) * 4, 256) : 0;
+}
+
+static int64_t split_bytes(int64_t M, int64_t N, int64_t K);
+
 extern "C" int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 {
     if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+    return scale_copy_bytes(M, N, K) + split_bytes(M, N, K);
+}
+
+static int64_t split_bytes(int64_t M, int64_t N, int64_t K)
+{
     if (M <= 64) {
         int sp, per;
         gemm::skinny_plan(N, K, sp, per);
@@ -380,6 +404,18 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     int rc = check_gemm_args("lp_gemm_fp8_block", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
     if (rc) return rc > 0 ? LP_OK : rc;
     hipStream_t st = (hipStream_t)stream;
+    // The hand-scheduled kernels read fp32 scales: with scratch, e8m0 scales are expanded first (one small launch).
+    const int64_t sc_bytes = scale_copy_bytes(M, N, K);
+    if (scale_dtype == LP_E8M0 && sc_bytes > 0 && workspace && workspace_bytes >= sc_bytes && (uintptr_t)workspace % 256 == 0) {
+        const int64_t na = M * (K / 128), nb = (N / 128) * (K / 128);
+        float *fa = (float *)workspace, *fb = (float *)((char *)workspace + round_up(na * 4, 256));
+        hipLaunchKernelGGL(scales_to_f32, dim3((unsigned)((na + nb + 255) / 256)), dim3(256), 0, st, (const uint8_t *)As, na,
+                           (const uint8_t *)Bs, nb, fa, fb);
+        rc = check_launch("lp_gemm_fp8_block(scales)");
+        if (rc) return rc;
+        return lp_gemm_fp8_block(Aq, fa, Bq, fb, LP_F32, M, N, K, C, out_dtype, (char *)workspace + sc_bytes,
+                                 workspace_bytes - sc_bytes, stream);
+    }
     static const bool no_skinny = getenv("LP_GEMM_NO_SKINNY") != nullptr;       // tuning aid
     if (M <= 64 && !no_skinny) {
         // decode-sized: the weight-streaming kernel, when the caller gave scratch for its K ranges and one range

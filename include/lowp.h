@@ -141,8 +141,9 @@ int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t rows, int6
  * Bs: device [N/128,K/128]; scales of scale_dtype (LP_F32 or LP_E8M0);
  * C: device [M,N] LP_BF16 or LP_F32.  K % 128 == 0, N % 128 == 0, any M.
  * workspace: optional device scratch of at least lp_gemm_workspace_bytes(M,N,K)
- * bytes (16-byte aligned); with it, problems with few output tiles split K
- * across workgroups (fixed summation order).  NULL / too small = no split.
+ * bytes (256-byte aligned); with it, problems with few output tiles split K
+ * across workgroups (fixed summation order) and LP_E8M0 scales are expanded to
+ * fp32 for the fastest kernels.  NULL / too small = slower paths, same results.
  * Replaces gemm_fp8_block_scaling_impl (gfused/mygemm_fp8.py:44-97).
  */
 int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
