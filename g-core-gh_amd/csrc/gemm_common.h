@@ -19,10 +19,20 @@ __device__ __forceinline__ float scale_at(const void *s, int64_t idx)
 // modulo 8) is handed whole blocks, so panels are re-used out of one L2.
 constexpr int GROUP_M = 8, GROUP_N = 4, CHUNK = GROUP_M * GROUP_N;
 
-__device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t tiles_n, int64_t &tm, int64_t &tn)
+// ends_first: the chunks an XCD works through come alternately from the front and the back of the tile
+// list (grid = number of workgroups launched, a multiple of 8 * CHUNK).  Grouped problems list experts in
+// caller order; when the heavy experts sit at one end, this keeps compute-bound tiles and tiles that only
+// stream weights on the machine at the same time.
+__device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t tiles_n, int64_t &tm, int64_t &tn,
+                                            bool ends_first = false, int64_t grid = 0)
 {
     const int64_t xcd = b & 7, s = b >> 3;
-    const int64_t lin = ((s / CHUNK) * 8 + xcd) * CHUNK + s % CHUNK;
+    int64_t q = s / CHUNK;
+    if (ends_first) {
+        const int64_t Q = grid / (8 * CHUNK);
+        q = (q & 1) ? Q - 1 - (q >> 1) : (q >> 1);
+    }
+    const int64_t lin = (q * 8 + xcd) * CHUNK + s % CHUNK;
     if (lin >= tiles_m * tiles_n) return false;
     // groups of GROUP_M m-tiles (the last may be short); inside a group, blocks of
     // GROUP_N n-tiles (the last may be narrow); inside a block m runs fastest

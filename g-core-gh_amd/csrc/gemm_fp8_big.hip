@@ -340,30 +340,42 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
 }
 
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
-// The grid is sized from an upper bound on the number of 256-row tiles; each workgroup finds its expert
-// with a block-wide scan over the per-expert tile counts.
-__global__ __launch_bounds__(THREADS) void gemm_big_asm_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
-                                                                const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                                                const int32_t *__restrict__ m_offsets, int E, int64_t N,
-                                                                int64_t K, int64_t max_mtiles, int64_t tiles_n,
-                                                                void *__restrict__ C, int out_dtype)
+// The grid is sized from an upper bound on the number of row tiles; each workgroup finds its expert with a
+// block-wide scan over the per-expert tile counts.  PART selects which rows of every expert a launch covers:
+//   0  all rows, in tiles of TM (the last tile of an expert may be partly empty)
+//   1  only the full 256-row tiles (TM = 256)
+//   2  what PART 1 leaves, i.e. the last M_e % 256 rows, in tiles of TM
+// Launching 1 with 256 x 256 tiles and then 2 with 128 x 128 tiles keeps the large tiles full and bounds the
+// padding of an expert by 127 rows.
+template <int TM, int TN, int KSUB, int PART>
+__global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                           const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                           const int32_t *__restrict__ m_offsets, int E, int64_t N,
+                                                           int64_t K, int64_t max_mtiles, int64_t tiles_n,
+                                                           void *__restrict__ C, int out_dtype)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<256, 256, 1>::LDS_BYTES];
-    __shared__ int scan[THREADS];
+    constexpr int NT = TM * 2;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB>::LDS_BYTES];
+    __shared__ int scan[NT];
     __shared__ int found_e, found_first;
     int64_t gmt, tn;
-    const bool in_range = gemm::tile_coords(blockIdx.x, max_mtiles, tiles_n, gmt, tn);
+    const bool in_range = gemm::tile_coords(blockIdx.x, max_mtiles, tiles_n, gmt, tn, true, gridDim.x);
     const int t = threadIdx.x;
     if (t == 0) found_e = -1;
     __syncthreads();
+    auto tiles_of = [](int rows) -> int {
+        if (PART == 1) return rows / TM;
+        if (PART == 2) rows %= 256;
+        return (rows + TM - 1) / TM;
+    };
     int base = 0;
-    for (int e0 = 0; e0 < E; e0 += THREADS) {
+    for (int e0 = 0; e0 < E; e0 += NT) {
         const int e = e0 + t;
         int cnt = 0;
-        if (e < E) cnt = (m_offsets[e + 1] - m_offsets[e] + BM - 1) / BM;
+        if (e < E) cnt = tiles_of(m_offsets[e + 1] - m_offsets[e]);
         scan[t] = cnt;
         __syncthreads();
-        for (int off = 1; off < THREADS; off <<= 1) {
+        for (int off = 1; off < NT; off <<= 1) {
             int v = t >= off ? scan[t - off] : 0;
             __syncthreads();
             scan[t] += v;
@@ -371,15 +383,16 @@ __global__ __launch_bounds__(THREADS) void gemm_big_asm_grouped(const uint8_t *_
         }
         const int incl = base + scan[t], excl = incl - cnt;
         if (in_range && e < E && gmt >= excl && gmt < incl) { found_e = e; found_first = excl; }
-        base += scan[THREADS - 1];
+        base += scan[NT - 1];
         __syncthreads();
     }
     if (!in_range || found_e < 0) return;
     const int e = found_e;
     const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
+    const int64_t first = PART == 2 ? row_begin + (row_end - row_begin) / 256 * 256 : row_begin;
     const int64_t kblocks = K / KB;
-    tile_asm<256, 256, 1>(smem, Aq, As, Bq + (int64_t)e * N * K, Bs + (int64_t)e * (N / 128) * kblocks,
-                 row_begin + (gmt - found_first) * BM, row_end, tn * 256, N, K, C, N, out_dtype);
+    tile_asm<TM, TN, KSUB>(smem, Aq, As, Bq + (int64_t)e * N * K, Bs + (int64_t)e * (N / 128) * kblocks,
+                           first + (gmt - found_first) * TM, row_end, tn * TN, N, K, C, N, out_dtype);
 }
 
 template <int SDT, int NB>
@@ -484,12 +497,38 @@ bool big_grouped_ok(const void *As, const void *Bs, int scale_dtype, int64_t M_t
 int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,
                        int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype, hipStream_t st)
 {
-    const int64_t max_mtiles = M_total / BM + E, tiles_n = N / 256;
-    const int64_t grid = padded_grid(max_mtiles, tiles_n);
+    // Few rows per expert on average: the weights of most experts are read for one or two row tiles, so the launch
+    // is as much a weight stream as a GEMM.  128 x 128 tiles (two workgroups per CU, tiles taken from both ends
+    // of the expert list) let streaming tiles and compute-bound tiles overlap and bound the padding per expert
+    // by 127 rows.  With many rows per expert the 256 x 256 kernel takes the full 256-row tiles and the
+    // 128 x 128 kernel what is left.
+    static const char *force = getenv("LP_GEMM_GROUPED_MODE");          // tuning aid: 0 = 128 tiles, 1 = 256 + 128
+    const bool split = force ? atoi(force) == 1 : M_total >= (int64_t)E * 1024;
+    if (split) {
+        const int64_t big_mtiles = M_total / 256;
+        const int64_t grid = padded_grid(big_mtiles, N / 256);
+        if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
+        hipLaunchKernelGGL((gemm_asm_grouped<256, 256, 1, 1>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, big_mtiles, N / 256,
+                           C, out_dtype);
+        const int rc = check_launch("lp_gemm_fp8_grouped(asm 256)");
+        if (rc) return rc;
+        int64_t rest_mtiles = 2 * (int64_t)E;
+        if (rest_mtiles > M_total / 128 + E) rest_mtiles = M_total / 128 + E;
+        const int64_t grid2 = padded_grid(rest_mtiles, N / 128);
+        if (grid2 > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
+        hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 2>), dim3((unsigned)grid2), dim3(256), 0, st, (const uint8_t *)Aq,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, rest_mtiles, N / 128,
+                           C, out_dtype);
+        return check_launch("lp_gemm_fp8_grouped(asm 128)");
+    }
+    const int64_t mtiles = M_total / 128 + E;
+    const int64_t grid = padded_grid(mtiles, N / 128);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
-    hipLaunchKernelGGL(gemm_big_asm_grouped, dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, (const float *)As,
-                       (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
-    return check_launch("lp_gemm_fp8_grouped(asm)");
+    hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 0>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
+                       (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, mtiles, N / 128, C,
+                       out_dtype);
+    return check_launch("lp_gemm_fp8_grouped(asm 128)");
 }
 
 }  // namespace gemm

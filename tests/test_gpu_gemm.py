@@ -132,6 +132,9 @@ GROUPED = [
     (8, 512, 512, [700, 0, 300, 1, 255, 256, 257, 600]),
     (16, 768, 1024, [513, 0, 0, 90, 1024, 17, 256, 300, 2, 511, 128, 129, 64, 1, 700, 333]),
     (3, 256, 384, [2048, 1, 515]),
+    (4, 256, 512, [300, 0, 255, 513]),
+    (6, 512, 1024, [128, 129, 256, 257, 1, 640]),
+    (5, 256, 1536, [0, 0, 7, 0, 0]),
 ]
 
 
