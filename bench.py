@@ -291,6 +291,15 @@ def main():
         e1 = bufs[0][0][4] * bufs[0][0][5]
         b1 = e1 // 2 + e1 // 32 + e1 * 2
         extras["c5_fp4_to_bf16"] = {"ms": ms5b, "GB/s": b1 / ms5b / 1e6, "hbm_frac": b1 / ms5b / 1e6 / HBM_PEAK_GBS, "bytes": b1}
+        # the way back: bf16 -> packed FP4 with 1 x 32 e8m0 scales (quant_fp4_e2m1_scale_e8m0_packed), on the tensors
+        # the previous step wrote
+        def c5_fp4q(i):
+            packed, sc, q, so, rows, cc = bufs[i][0]
+            return lambda: chk(L.lp_quant_fp4_block(bouts[i].data_ptr(), A.BF16, rows, cc, 1, 32, packed.data_ptr(),
+                                                    sc.data_ptr(), None, stream()))
+
+        ms5q, _ = time_launches([c5_fp4q(i) for i in range(n_chunksets)], 16, 4)
+        extras["c5_bf16_to_fp4"] = {"ms": ms5q, "GB/s": b1 / ms5q / 1e6, "hbm_frac": b1 / ms5q / 1e6 / HBM_PEAK_GBS, "bytes": b1}
         del bufs, bouts
         torch.cuda.empty_cache()
 

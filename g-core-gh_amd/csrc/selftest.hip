@@ -4,6 +4,10 @@
 
 using namespace lowp;
 
+namespace lowp {
+int selftest_cvt_to_fp4(uint64_t *mismatches, hipStream_t st);      // quant_fp4.hip
+}
+
 namespace {
 
 __device__ __forceinline__ void count(uint64_t *out, bool bad)
@@ -89,7 +93,9 @@ __global__ __launch_bounds__(256) void debug_cast(int kind, const float *__restr
         if (kind == 0) ((uint8_t *)out)[i] = sw_f32_to_e4m3fn(v);
         else if (kind == 1) ((uint8_t *)out)[i] = (uint8_t)__builtin_amdgcn_cvt_pk_fp8_f32(clamp448(v), 0.0f, 0, false);
         else if (kind == 2) ((uint8_t *)out)[i] = f32_to_e8m0(v);
-        else ((uint16_t *)out)[i] = sw_f32_to_bf16(v);
+        else if (kind == 3) ((uint16_t *)out)[i] = sw_f32_to_bf16(v);
+        else if (kind == 4) ((uint8_t *)out)[i] = (uint8_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, v, 1.0f, 0);
+        else ((uint8_t *)out)[i] = (uint8_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, v, 4.0f, 0);
     }
 }
 
@@ -98,7 +104,7 @@ __global__ __launch_bounds__(256) void debug_cast(int kind, const float *__restr
 extern "C" int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream)
 {
     LP_REQUIRE(mismatches, "lp_selftest: null pointer");
-    LP_REQUIRE(which >= 0 && which <= 3, "lp_selftest: which must be 0..3");
+    LP_REQUIRE(which >= 0 && which <= 4, "lp_selftest: which must be 0..4");
     hipStream_t st = (hipStream_t)stream;
     hipError_t e = hipMemsetAsync(mismatches, 0, sizeof(uint64_t), st);
     if (e != hipSuccess) return fail(LP_ERR_HIP, "lp_selftest: %s", hipGetErrorString(e));
@@ -106,13 +112,14 @@ extern "C" int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream)
     if (which == 0) hipLaunchKernelGGL(st_cvt_fp8, dim3(all), dim3(256), 0, st, mismatches);
     else if (which == 1) hipLaunchKernelGGL(st_cvt_from_fp8, dim3(1), dim3(256), 0, st, mismatches);
     else if (which == 2) hipLaunchKernelGGL(st_cvt_bf16, dim3(all), dim3(256), 0, st, mismatches);
-    else hipLaunchKernelGGL(st_cvt_fp4, dim3(1), dim3(256), 0, st, mismatches);
+    else if (which == 3) hipLaunchKernelGGL(st_cvt_fp4, dim3(1), dim3(256), 0, st, mismatches);
+    else return selftest_cvt_to_fp4(mismatches, st);
     return check_launch("lp_selftest");
 }
 
 extern "C" int lp_debug_cast(int kind, const float *x, void *out, int64_t n, lp_stream_t stream)
 {
-    LP_REQUIRE(kind >= 0 && kind <= 3, "lp_debug_cast: kind must be 0..3");
+    LP_REQUIRE(kind >= 0 && kind <= 5, "lp_debug_cast: kind must be 0..5");
     LP_REQUIRE(n >= 0, "lp_debug_cast: negative length");
     if (n == 0) return LP_OK;
     LP_REQUIRE(x && out, "lp_debug_cast: null pointer");

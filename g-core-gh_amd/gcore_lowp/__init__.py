@@ -4,7 +4,8 @@ Python call signatures follow the reference functions they replace; the work is
 done by hand-written gfx950 HIP kernels behind a C ABI (include/lowp.h).
 """
 from . import _abi  # noqa: F401
-from .eager_quant_kernels import dequant_fp4_e2m1_fp8_scale_e8m0_packed, quant_fp8_e4m3_scale_e8m0  # noqa: F401
+from .eager_quant_kernels import (  # noqa: F401
+    dequant_fp4_e2m1_fp8_scale_e8m0_packed, quant_fp4_e2m1_scale_e8m0_packed, quant_fp8_e4m3_scale_e8m0)
 from .fp8_blockwise import quant_1d, quant_2d, quant_act, quant_weight, quantize_fp8_blockwise  # noqa: F401
 from .convert_deepseek_v4_fp4_to_bf16 import cast_e2m1fn_to_bf16, cast_e4m3fn_to_bf16  # noqa: F401
 from .dsv4_kernels import (  # noqa: F401

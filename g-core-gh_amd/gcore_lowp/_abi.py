@@ -29,6 +29,7 @@ PROTOTYPES = {
     "lp_version": (_i32, []),
     "lp_last_error": (ctypes.c_char_p, []),
     "lp_quant_fp8_block": (_i32, [_p, _i32, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _p, _p, _i32, _p, _p]),
+    "lp_quant_fp4_block": (_i32, [_p, _i32, _i64, _i64, _i32, _i32, _p, _p, _p, _p]),
     "lp_dequant_fp8_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _p, _i32, _p]),
     "lp_dequant_fp4_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _p, _i32, _p]),
     "lp_fp4_to_fp8_rebase": (_i32, [_p, _p, _i64, _i64, _p, _p, _i32, _p]),

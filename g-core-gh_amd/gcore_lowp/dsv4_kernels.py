@@ -5,12 +5,34 @@ from __future__ import annotations
 import torch
 
 from . import ops
-from .eager_quant_kernels import dequant_fp4_e2m1_fp8_scale_e8m0_packed, quant_fp8_e4m3_scale_e8m0
+import re
+
+from .eager_quant_kernels import (dequant_fp4_e2m1_fp8_scale_e8m0_packed, quant_fp4_e2m1_scale_e8m0_packed,
+                                  quant_fp8_e4m3_scale_e8m0)
 
 __all__ = [
     "dequant_fp8_block", "cast_e2m1fn_to_e4m3fn", "official_expert_to_sgl", "official_dense_to_sgl",
-    "sgl_dense_to_official", "official_wo_a_to_sgl", "sgl_wo_a_to_official", "fp4_to_fp8_blockwise",
+    "sgl_dense_to_official", "official_wo_a_to_sgl", "sgl_wo_a_to_official", "sgl_expert_to_official",
+    "fp4_to_fp8_blockwise", "is_expert_weight", "is_wo_a_weight", "scale_key",
 ]
+
+# weight roles by checkpoint key (kernels.py:68-83)
+_EXPERT_WEIGHT_RE = re.compile(r"(?:^|\.)experts\.\d+\.w[123]\.weight$")
+_SHARED_EXPERT_RE = re.compile(r"shared_experts")
+_WO_A_WEIGHT_RE = re.compile(r"(?:^|\.)attn\.wo_a\.weight$")
+
+
+def is_expert_weight(name: str) -> bool:
+    return _EXPERT_WEIGHT_RE.search(name) is not None and _SHARED_EXPERT_RE.search(name) is None
+
+
+def is_wo_a_weight(name: str) -> bool:
+    return _WO_A_WEIGHT_RE.search(name) is not None
+
+
+def scale_key(weight_key: str) -> str:
+    assert weight_key.endswith(".weight"), weight_key
+    return weight_key[:-len(".weight")] + ".scale"
 
 
 def dequant_fp8_block(weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
@@ -60,6 +82,16 @@ def official_wo_a_to_sgl(weight: torch.Tensor, scale: torch.Tensor) -> torch.Ten
 def sgl_wo_a_to_official(weight: torch.Tensor):
     """kernels.py:160-162."""
     return quant_fp8_e4m3_scale_e8m0(weight.float(), block_size=(128, 128))
+
+
+def sgl_expert_to_official(weight: torch.Tensor, scale: torch.Tensor):
+    """kernels.py:136-140: FP8 expert (fp32 128 x 128 scales) -> packed FP4 + e8m0 1 x 32 scales.  The
+    intermediate is the bf16 dequantised weight, as in the reference; it stays on the GPU."""
+    dev = ops.A.require_gpu()
+    home = weight.device
+    full = dequant_fp8_block(weight.to(dev), scale.to(dev))
+    q, s = quant_fp4_e2m1_scale_e8m0_packed(full, block_size=(1, 32))
+    return q.to(home), s.to(home)
 
 
 def fp4_to_fp8_blockwise(x: torch.Tensor, scale: torch.Tensor, *, return_bf16: bool = False):

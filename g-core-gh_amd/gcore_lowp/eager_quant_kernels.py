@@ -1,4 +1,4 @@
-"""MI355X drop-in for gpatch_v4/kernel/quantize/eager_quant_kernels.py (FP8 rows).
+"""MI355X drop-in for gpatch_v4/kernel/quantize/eager_quant_kernels.py.
 
 Same names, arguments, return dtypes/shapes and exceptions as the reference
 functions; the arithmetic runs in hand-written HIP kernels.
@@ -10,7 +10,20 @@ import torch
 from . import _abi as A
 from . import ops
 
-__all__ = ["quant_fp8_e4m3_scale_e8m0", "dequant_fp4_e2m1_fp8_scale_e8m0_packed"]
+__all__ = ["quant_fp4_e2m1_scale_e8m0_packed", "quant_fp8_e4m3_scale_e8m0", "dequant_fp4_e2m1_fp8_scale_e8m0_packed"]
+
+
+def quant_fp4_e2m1_scale_e8m0_packed(value: torch.Tensor, block_size: tuple[int, int] = (1, 32)):
+    """eager_quant_kernels.py:63-129: packed e2m1 codes (int8 [..., M, N/2], low nibble = even column) + one
+    power-of-two (e8m0) scale per block, s = 2^ceil(log2(amax/6)), all-zero block -> s = 1; a value half way
+    between two code points takes the one of smaller magnitude; -0.0 keeps its sign (code 8)."""
+    m, n = value.shape[-2:]
+    bm, bn = block_size
+    assert m % bm == 0 and n % bn == 0, f"value shape ({m}, {n}) not divisible by block ({bm}, {bn})"
+    assert n % 2 == 0, f"FP4 packing requires N (={n}) to be even (two nibbles per byte)"
+    packed, scale, n_nan = ops.quant_fp4_block(value, (bm, bn), count_nan=True)
+    assert n_nan == 0, "quant_fp4_e2m1_scale_e8m0_packed: input contains NaN"
+    return packed, scale
 
 
 def quant_fp8_e4m3_scale_e8m0(value: torch.Tensor, block_size: tuple[int, int] = (128, 128)):

@@ -44,6 +44,27 @@ def quant_fp8_block(x: torch.Tensor, block_size, *, scale_mode: int, scale_dtype
     return q.view(E4M3).to(home), scale.to(home), n_nan
 
 
+def quant_fp4_block(x: torch.Tensor, block_size=(1, 32), *, count_nan: bool = False):
+    """[..., M, N] -> (packed e2m1 int8 [..., M, N/2], e8m0 scales [..., M/bm, N/bn]) and, when count_nan,
+    the number of NaN inputs (forces a sync)."""
+    bm, bn = int(block_size[0]), int(block_size[1])
+    m, n = x.shape[-2:]
+    xg, home = A.to_device(x)
+    xg, code = _as_input(xg)
+    lead = tuple(x.shape[:-2])
+    rows = m
+    for d in lead:
+        rows *= d
+    packed = torch.empty(lead + (m, n // 2), dtype=torch.int8, device=xg.device)
+    scale = torch.empty(lead + (m // max(bm, 1), n // max(bn, 1)), dtype=E8M0, device=xg.device)
+    nan = torch.zeros(1, dtype=torch.int32, device=xg.device) if count_nan else None
+    with torch.cuda.device(xg.device):
+        A.check(A.lib().lp_quant_fp4_block(xg.data_ptr(), code, rows, n, bm, bn, packed.data_ptr(), scale.data_ptr(),
+                                           nan.data_ptr() if count_nan else None, A.stream_ptr()))
+    n_nan = int(nan.item()) if count_nan else 0
+    return packed.to(home), scale.to(home), n_nan
+
+
 def _block_from_shapes(rows, cols, scales, what):
     sr, sc = scales.shape[-2:]
     if sr == 0 or sc == 0 or rows % sr or cols % sc:

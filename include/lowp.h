@@ -136,6 +136,24 @@ int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t rows, int6
                        lp_stream_t stream);
 
 /*
+ * Block quantisation to packed FP4 (e2m1) with e8m0 block scales.
+ * x: device [rows, cols] of x_dtype (LP_F32 or LP_BF16); packed_out: device
+ * [rows, cols/2] bytes, low nibble = even column; scale_out: device
+ * [rows/bm, cols/bn] e8m0 bytes.  scale = 2^ceil(log2(amax/6)) (1 for an all-zero
+ * block), code = nearest e2m1 value of x/scale with ties to the smaller
+ * magnitude, sign bit kept (also for -0).  cols even; the fast path is
+ * bm = 1, bn = 32, other shapes need an even bn.  nan_count: optional device
+ * int32 that is incremented by the number of NaN inputs (caller zeroes it; the
+ * reference asserts the input holds none).
+ * Replaces quant_fp4_e2m1_scale_e8m0_packed
+ * (gpatch_v4/kernel/quantize/eager_quant_kernels.py:63-129); with
+ * lp_dequant_fp8_block in front it is sgl_expert_to_official
+ * (tools/dsv4_quant_and_dequant/kernels.py:136-140).
+ */
+int lp_quant_fp4_block(const void *x, int x_dtype, int64_t rows, int64_t cols, int bm, int bn,
+                       void *packed_out, void *scale_out, int32_t *nan_count, lp_stream_t stream);
+
+/*
  * Block-scaled FP8 GEMM: C[i,j] = cast(sum_kb (sum_{k in kb} Aq[i,k] Bq[j,k]) * As[i,kb] * Bs[j/128,kb]).
  * Aq: device e4m3fn [M,K]; As: device [M,K/128]; Bq: device e4m3fn [N,K];
  * Bs: device [N/128,K/128]; scales of scale_dtype (LP_F32 or LP_E8M0);
@@ -186,6 +204,8 @@ int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const vo
  *   which = 1: v_cvt_pk_f32_fp8 over all 256 codes except the two NaNs
  *   which = 2: fp32 -> bf16 conversion over every non-NaN fp32
  *   which = 3: v_cvt_scalef32_pk_f32_fp4 over 256 bytes x the scale exponents used
+ *   which = 4: v_cvt_scalef32_pk_fp4_f32 with the tie adjustment of lp_quant_fp4_block
+ *              over every finite fp32 at three scales
  */
 int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream);
 

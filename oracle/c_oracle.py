@@ -48,6 +48,8 @@ def lib() -> ctypes.CDLL:
         L.orc_e2m1_value.restype = f32
         L.orc_quant_fp8_block.argtypes = [p, i64, i64, i32, i32, i32, f32, i32, i32, p, p, p]
         L.orc_quant_fp8_block.restype = i64
+        L.orc_quant_fp4_block.argtypes = [p, i64, i64, i32, i32, i32, p, p]
+        L.orc_quant_fp4_block.restype = i64
         L.orc_dequant_fp8_block.argtypes = [p, p, i64, i64, i32, i32, p, p]
         L.orc_dequant_fp8_block.restype = None
         L.orc_fp4_dequant.argtypes = [p, p, i64, i64, i32, i32, i32, p, p]
@@ -112,6 +114,17 @@ def quant_fp8_block(x, bm, bn, mode, amax_floor=0.0, zero_rule=ZERO_NONE, log2_k
     nan = lib().orc_quant_fp8_block(_ptr(x), rows, cols, bm, bn, mode, ctypes.c_float(amax_floor),
                                     zero_rule, log2_kind, _ptr(q), _ptr(s), _ptr(sb))
     return q, s, sb, nan
+
+
+def quant_fp4_block(x, bm=1, bn=32, log2_kind=LOG2_LIBM):
+    """x fp32 [rows, cols] -> (packed u8 [rows, cols/2], scale e8m0 bytes [rows/bm, cols/bn], NaN count)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, cols = x.shape
+    assert rows % bm == 0 and cols % bn == 0 and cols % 2 == 0
+    packed = np.empty((rows, cols // 2), np.uint8)
+    sb = np.empty((rows // bm, cols // bn), np.uint8)
+    nan = lib().orc_quant_fp4_block(_ptr(x), rows, cols, bm, bn, log2_kind, _ptr(packed), _ptr(sb))
+    return packed, sb, nan
 
 
 def dequant_fp8_block(codes, scale_f32, want_bf16=True):

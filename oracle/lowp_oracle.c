@@ -21,6 +21,10 @@
  *   block quant / dequant / FP4 converts : hand-derived vectors from the
  *       reference's CPU tests, grid round-trip invariants, and equality with an
  *       independent eager-torch restatement (oracle/torch_ref.py).
+ *   orc_quant_fp4_block                  : the reference's known answers
+ *       (tests/test_gfused/test_eager_quantize_kernels.py:54-150), hand-made tie vectors at
+ *       three scales, the closed form "smallest 2^e with 6 * 2^e >= amax", equality
+ *       with the eager-torch restatement; blocks holding NaN / inf: parity unpinned.
  *   orc_pow2_exponent (libm flavour)     : equals the exact flavour for every
  *       bf16-grid amax (exhaustive test); for raw fp32 amax within a few ulp
  *       above a power of two the reference itself depends on the log2
@@ -237,6 +241,57 @@ int64_t orc_quant_fp8_block(const float *x, int64_t rows, int64_t cols, int bm, 
                     if (y > 448.0f) y = 448.0f;                      /* clamp keeps NaN */
                     if (y < -448.0f) y = -448.0f;
                     q[idx] = orc_f32_to_e4m3fn(y);
+                }
+        }
+    }
+    return nan_count;
+}
+
+/*
+ * Block quantiser to packed FP4 e2m1 + e8m0 scales (eager_quant_kernels.py:63-129).
+ * x is fp32 [rows, cols]; packed is [rows, cols/2] (low nibble = even column); scale_e8m0 is
+ * [rows/bm, cols/bn].  Per block: r = max(amax, FLT_MIN) / 6 (an fp32 division, :105-106),
+ * s = 2^ceil(log2 r) (:106-107), all-zero block -> s = 1 (:108); y = x / s (:111); the code is
+ * the number of midpoints {0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0} strictly below |y| -- ties go
+ * to the smaller magnitude, what torch.bucketize(right=False) does (:116-121) -- plus 8 when the
+ * sign bit of y is set (-0.0 keeps its sign, :112,121).  The stored scale is the e8m0 cast of s
+ * (:128); the division uses s itself.  Returns the number of NaN inputs (the reference asserts
+ * there are none, :97); what a block holding NaN or inf yields is not pinned by anything.
+ * Pinned by: the reference's known answers (tests/test_gfused/test_eager_quantize_kernels.py:
+ * 54-150: grid round trip with +6 planted per block, zero block, signed extremes, first byte 0xE6),
+ * hand-made tie vectors, and equality with the eager-torch restatement.
+ */
+int64_t orc_quant_fp4_block(const float *x, int64_t rows, int64_t cols, int bm, int bn, int log2_kind,
+                            uint8_t *packed, uint8_t *scale_e8m0)
+{
+    static const float mid[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
+    int64_t nbr = rows / bm, nbc = cols / bn, nan_count = 0;
+    for (int64_t i = 0; i < rows * (cols / 2); ++i) packed[i] = 0;
+    for (int64_t br = 0; br < nbr; ++br) {
+        for (int64_t bc = 0; bc < nbc; ++bc) {
+            float amax = 0.0f;
+            for (int i = 0; i < bm; ++i)
+                for (int j = 0; j < bn; ++j) {
+                    float v = x[(br * bm + i) * cols + bc * bn + j];
+                    if (v != v) ++nan_count;
+                    float a = fabsf(v);
+                    if (a > amax) amax = a;
+                }
+            float safe = amax < FLT_MIN ? FLT_MIN : amax;
+            float r = safe / 6.0f;
+            float s = ldexpf(1.0f, orc_pow2_exponent(r, log2_kind));
+            if (!(amax > 0.0f)) s = 1.0f;
+            scale_e8m0[br * nbc + bc] = orc_f32_to_e8m0(s);
+            for (int i = 0; i < bm; ++i)
+                for (int j = 0; j < bn; ++j) {
+                    int64_t row = br * bm + i, col = bc * bn + j;
+                    float y = x[row * cols + col] / s;
+                    float a = fabsf(y);
+                    int code = 0;
+                    for (int k = 0; k < 7; ++k)
+                        if (a > mid[k]) ++code;
+                    if (f2u(y) >> 31) code += 8;
+                    packed[row * (cols / 2) + col / 2] |= (uint8_t)(code << (4 * (col & 1)));
                 }
         }
     }

@@ -60,6 +60,36 @@ def quant_fp8_e4m3_scale_e8m0(value: torch.Tensor, block_size=(128, 128)):
     return q, s.to(_E8M0)
 
 
+def quant_fp4_e2m1_scale_e8m0_packed(value: torch.Tensor, block_size=(1, 32)):
+    """gpatch_v4/kernel/quantize/eager_quant_kernels.py:63-129: packed e2m1 codes (int8, low nibble = even
+    column) + e8m0 block scales; ties between two code points go to the smaller magnitude (bucketize)."""
+    m, n = value.shape[-2:]
+    bm, bn = block_size
+    assert m % bm == 0 and n % bn == 0, f"value shape ({m}, {n}) not divisible by block ({bm}, {bn})"
+    assert n % 2 == 0, f"FP4 packing requires N (={n}) to be even (two nibbles per byte)"
+    assert not torch.isnan(value).any(), "quant_fp4_e2m1_scale_e8m0_packed: input contains NaN"
+    lead = value.shape[:-2]
+    t = _tiles(value.float(), bm, bn)
+    amax = _tile_amax(t)
+    r = amax.clamp(min=torch.finfo(torch.float32).tiny) / 6.0
+    s = torch.pow(2.0, torch.ceil(torch.log2(r)))
+    s = torch.where(amax > 0, s, torch.ones_like(s))
+    y = t / _bcast(s)
+    pos = torch.tensor(_MAG, dtype=torch.float32)
+    mid = (pos[1:] + pos[:-1]) / 2.0
+    idx = torch.bucketize(y.abs().contiguous(), mid)
+    code = (idx + torch.signbit(y).to(torch.int64) * 8).to(torch.uint8).reshape(*lead, m, n)
+    pair = code.reshape(*lead, m, n // 2, 2)
+    packed = (pair[..., 0] | (pair[..., 1] << 4)).view(torch.int8).contiguous()
+    return packed, s.to(_E8M0)
+
+
+def sgl_expert_to_official(weight: torch.Tensor, scale: torch.Tensor):
+    """tools/dsv4_quant_and_dequant/kernels.py:136-140: FP8 expert (fp32 128x128 scales) -> packed FP4 + e8m0 1x32."""
+    full = dequant_fp4_e2m1_fp8_scale_e8m0_packed(weight, scale).float()
+    return quant_fp4_e2m1_scale_e8m0_packed(full, (1, 32))
+
+
 # --------------------------------------------------------------------- a2
 
 def quantize_fp8_blockwise(weight: torch.Tensor, block_size, *, device=None, scale_dtype=torch.bfloat16):
