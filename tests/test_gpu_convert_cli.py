@@ -1,0 +1,170 @@
+"""The checkpoint converters (tools/convert_deepseek_v4_fp4_to_bf16.py, tools/dsv4_quant_and_dequant/convert.py
+drop-ins) on a tiny synthetic DeepSeek-V4-style checkpoint: every written tensor equals the CPU oracle's,
+key / shard / index / aux-file conventions follow the reference."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+from oracle import torch_ref as T
+
+pytestmark = pytest.mark.gpu
+
+E4M3, E8M0 = torch.float8_e4m3fn, torch.float8_e8m0fnu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8)
+
+
+def same(a, b):
+    return a.dtype == b.dtype and a.shape == b.shape and torch.equal(u8(a), u8(b))
+
+
+def make_official(root):
+    """Two shards; the scale of expert 0 / w1 lives in the other shard than its weight."""
+    g = torch.Generator().manual_seed(1)
+    t = {}
+    for layer in (0, 1):
+        for e in (0, 1):
+            for w, (o, i) in (("w1", (128, 256)), ("w2", (256, 128))):
+                name = f"layers.{layer}.ffn.experts.{e}.{w}"
+                t[name + ".weight"] = torch.randint(0, 256, (o, i // 2), generator=g, dtype=torch.int32).to(torch.uint8).view(torch.int8)
+                t[name + ".scale"] = torch.randint(117, 128, (o, i // 32), generator=g, dtype=torch.int32).to(torch.uint8).view(E8M0)
+        for nm, (o, i) in (("attn.wo_a", (128, 128)), ("attn.wq_a", (256, 128)), ("ffn.shared_experts.w1", (128, 256))):
+            name = f"layers.{layer}.{nm}"
+            t[name + ".weight"] = torch.randint(0, 0x7E, (o, i), generator=g, dtype=torch.int32).to(torch.uint8).view(E4M3)
+            t[name + ".scale"] = torch.randint(115, 125, (o // 128, i // 128), generator=g, dtype=torch.int32).to(torch.uint8).view(E8M0)
+        t[f"layers.{layer}.attn_norm.weight"] = torch.randn(128, generator=g).to(torch.bfloat16)
+        t[f"layers.{layer}.ffn.gate.bias"] = torch.randn(4, generator=g)
+    t["embed.weight"] = torch.randn(64, 128, generator=g).to(torch.bfloat16)
+    shard_of = {k: ("model-00001-of-00002.safetensors" if (".experts.0." in k or "attn" in k or k == "embed.weight")
+                    else "model-00002-of-00002.safetensors") for k in t}
+    shard_of["layers.0.ffn.experts.0.w1.scale"] = "model-00002-of-00002.safetensors"
+    os.makedirs(root, exist_ok=True)
+    for shard in sorted(set(shard_of.values())):
+        save_file({k: v for k, v in t.items() if shard_of[k] == shard}, os.path.join(root, shard))
+    with open(os.path.join(root, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {"total_size": 0}, "weight_map": shard_of}, f)
+    with open(os.path.join(root, "config.json"), "w") as f:
+        json.dump({"model_type": "deepseek_v4", "expert_dtype": "fp4"}, f)
+    with open(os.path.join(root, "tokenizer.json"), "w") as f:
+        f.write("{}")
+    return t, shard_of
+
+
+def load_dir(root):
+    out, where = {}, {}
+    for fn in sorted(os.listdir(root)):
+        if fn.endswith(".safetensors"):
+            with safe_open(os.path.join(root, fn), framework="pt", device="cpu") as f:
+                for k in f.keys():
+                    out[k] = f.get_tensor(k)
+                    where[k] = fn
+    return out, where
+
+
+def test_fp4_checkpoint_to_bf16(tmp_path):
+    from gcore_lowp import convert_deepseek_v4_fp4_to_bf16 as C
+    say("convert_deepseek_v4_fp4_to_bf16.main")
+    src, dst = str(tmp_path / "official"), str(tmp_path / "bf16")
+    t, shard_of = make_official(src)
+    C.main(src, dst)
+    out, where = load_dir(dst)
+    assert not any(k.endswith(".scale") for k in out)
+    assert set(out) == {k for k in t if not k.endswith(".scale")}
+    for k, v in out.items():
+        assert where[k] == shard_of[k], k                         # same file names as the source
+        if t[k].dtype == torch.int8:
+            assert same(v, T.cast_e2m1fn_to_bf16(t[k], t[k.replace(".weight", ".scale")])), k
+        elif t[k].dtype == E4M3:
+            assert same(v, T.cast_e4m3fn_to_bf16(t[k], t[k.replace(".weight", ".scale")])), k
+        else:
+            assert same(v, t[k]), k
+    idx = json.load(open(os.path.join(dst, "model.safetensors.index.json")))
+    assert idx["weight_map"] == where
+    assert idx["metadata"]["total_size"] == sum(v.numel() * v.element_size() for v in out.values())
+    assert os.path.isfile(os.path.join(dst, "tokenizer.json")) and os.path.isfile(os.path.join(dst, "config.json"))
+    # --layers keeps layer-agnostic keys and the chosen layers only
+    dst1 = str(tmp_path / "bf16_l1")
+    C.main(src, dst1, layers=C._parse_layers("1"))
+    out1, _ = load_dir(dst1)
+    assert "embed.weight" in out1 and all(not k.startswith("layers.0.") for k in out1)
+    assert any(k.startswith("layers.1.") for k in out1)
+    assert C._parse_layers("0,1,3-5") == {0, 1, 3, 4, 5} and C._parse_layers(None) is None
+
+
+def expected_official2sgl(t):
+    want = {}
+    for k, v in t.items():
+        if k.endswith(".scale"):
+            continue
+        sk = k[:-len(".weight")] + ".scale" if k.endswith(".weight") else None
+        s = t.get(sk) if sk else None
+        if ".experts." in k and "shared_experts" not in k and k.endswith(".weight"):
+            want[k], want[sk] = T.official_expert_to_sgl(v, s)
+        elif k.endswith("attn.wo_a.weight"):
+            want[k] = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(v, s).to(torch.bfloat16)
+        elif s is not None and v.dtype == E4M3:
+            want[k], want[sk] = v, s.float()
+        else:
+            want[k] = v
+    return want
+
+
+def test_official_to_sgl_and_back(tmp_path):
+    from gcore_lowp import dsv4_convert as D
+    say("dsv4_convert official2sgl")
+    src, mid, back = str(tmp_path / "official"), str(tmp_path / "sgl"), str(tmp_path / "official2")
+    t, shard_of = make_official(src)
+    D.convert_checkpoint(src, mid, "official2sgl")
+    out, where = load_dir(mid)
+    want = expected_official2sgl(t)
+    assert set(out) == set(want)
+    for k in want:
+        assert same(out[k], want[k]), k
+        assert where[k] == shard_of[k[:-len(".scale")] + ".weight" if k.endswith(".scale") else k], k
+    cfg = json.load(open(os.path.join(mid, "config.json")))
+    assert "expert_dtype" not in cfg and cfg["model_type"] == "deepseek_v4"
+    idx = json.load(open(os.path.join(mid, "model.safetensors.index.json")))
+    assert idx["weight_map"] == where
+    assert idx["metadata"]["total_size"] == sum(v.numel() * v.element_size() for v in out.values())
+
+    say("dsv4_convert sgl2official (module CLI in a child process)")
+    env = dict(os.environ)
+    env["PYTHONPATH"] = os.pathsep.join(p for p in sys.path if p)
+    r = subprocess.run([sys.executable, "-m", "gcore_lowp.dsv4_convert", "--direction", "sgl2official", "--src", mid,
+                        "--dst", back], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    out2, _ = load_dir(back)
+    for k, v in out.items():
+        if k.endswith(".scale"):
+            continue
+        sk = k[:-len(".weight")] + ".scale" if k.endswith(".weight") else None
+        s = out.get(sk) if sk else None
+        if ".experts." in k and "shared_experts" not in k and k.endswith(".weight"):
+            wq, ws = T.sgl_expert_to_official(v, s)
+            assert same(out2[k], wq) and same(out2[sk], ws), k
+        elif k.endswith("attn.wo_a.weight"):
+            wq, ws = T.quant_fp8_e4m3_scale_e8m0(v.float(), (128, 128))
+            assert same(out2[k], wq) and same(out2[sk], ws), k
+        elif s is not None and v.dtype == E4M3:
+            assert same(out2[k], v) and same(out2[sk], s.to(E8M0)), k
+        else:
+            assert same(out2[k], v), k
+    assert json.load(open(os.path.join(back, "config.json")))["expert_dtype"] == "fp4"
+    # dense weights and scales are back to the official bytes
+    for k in t:
+        if "wq_a" in k or "shared_experts" in k:
+            assert same(out2[k], t[k]), k
+    with pytest.raises(RuntimeError):
+        D.convert_checkpoint(src, str(tmp_path / "x"), "official2sgl", device="cpu")
