@@ -300,6 +300,23 @@ def main():
 
         ms5q, _ = time_launches([c5_fp4q(i) for i in range(n_chunksets)], 16, 4)
         extras["c5_bf16_to_fp4"] = {"ms": ms5q, "GB/s": b1 / ms5q / 1e6, "hbm_frac": b1 / ms5q / 1e6 / HBM_PEAK_GBS, "bytes": b1}
+        # fused QAT conversions of the weight-export path on one expert-sized tensor set (rotating, > 256 MB)
+        qs = 6
+        wq32 = [torch.randn(2048, 7168, generator=gen, device=dev) * 0.02 for _ in range(qs)]
+        wqb = [w.to(torch.bfloat16) for w in wq32]
+        q8o = torch.empty(2048, 7168, dtype=torch.uint8, device=dev)
+        s8o = torch.empty(16, 56, dtype=torch.uint8, device=dev)
+        bo = torch.empty(2048, 7168, dtype=torch.bfloat16, device=dev)
+        eq = 2048 * 7168
+        msq, _ = time_launches([(lambda i=i: chk(L.lp_fp4_qat_to_fp8(wq32[i].data_ptr(), 2048, 7168, q8o.data_ptr(),
+                                                                       s8o.data_ptr(), stream()))) for i in range(qs)], 18, 6)
+        extras["fp4_qat_then_to_fp8_2048x7168"] = {"ms": msq, "GB/s": eq * 5 / msq / 1e6, "hbm_frac": eq * 5 / msq / 1e6 / HBM_PEAK_GBS,
+                                                   "bytes": eq * 5}
+        msq, _ = time_launches([(lambda i=i: chk(L.lp_qdq_fp8_tile128(wqb[i].data_ptr(), 2048, 7168, bo.data_ptr(), stream())))
+                                for i in range(qs)], 18, 6)
+        extras["fp_qat_128x128_2048x7168"] = {"ms": msq, "GB/s": eq * 4 / msq / 1e6, "hbm_frac": eq * 4 / msq / 1e6 / HBM_PEAK_GBS,
+                                              "bytes": eq * 4}
+        del wq32, wqb, q8o, s8o, bo
         del bufs, bouts
         torch.cuda.empty_cache()
 

@@ -20,6 +20,11 @@ struct BlockScale {
     bool fast;      // DIV: reciprocal path is safe
 };
 
+// scale modes that divide by a general divisor / by a power of two
+constexpr bool div_like(int mode) { return mode == LP_SCALE_DIV || mode == LP_SCALE_RCP; }
+constexpr bool pow2_like(int mode) { return mode == LP_SCALE_POW2 || mode == LP_SCALE_RCP_POW2; }
+constexpr float kInv448 = 0.002232142857142857f;      // fl32(1 / 448)
+
 template <int MODE>
 __device__ __forceinline__ BlockScale derive_scale(float amax, float amax_floor, int zero_rule)
 {
@@ -32,9 +37,16 @@ __device__ __forceinline__ BlockScale derive_scale(float amax, float amax_floor,
         if (!(amax > 0.0f)) e = 0;
         b.exp2 = e;
         b.stored = ldexpf(1.0f, e);
-    } else if (MODE == LP_SCALE_DIV) {
+    } else if (MODE == LP_SCALE_RCP_POW2) {
+        // bit-defined: exponent field - 127, + 1 when any mantissa bit is set; 2^e rebuilt from bits
+        const float a = amax < amax_floor ? amax_floor : amax;
+        const uint32_t rb = f2u(a * kInv448);
+        const int e = (int)((rb >> 23) & 0xFFu) - 127 + ((rb & 0x7FFFFFu) ? 1 : 0);
+        b.exp2 = e;
+        b.stored = u2f((uint32_t)(e + 127) << 23);
+    } else if (div_like(MODE)) {
         float a = amax < amax_floor ? amax_floor : amax;
-        float s = a / kE4M3Max;
+        float s = MODE == LP_SCALE_RCP ? a * kInv448 : a / kE4M3Max;
         if (zero_rule == LP_ZERO_SCALE_TO_ONE && s == 0.0f) s = 1.0f;
         if (zero_rule == LP_ZERO_AMAX_TO_ONE && amax == 0.0f) s = 1.0f;
         b.div = s;
@@ -54,8 +66,8 @@ __device__ __forceinline__ BlockScale derive_scale(float amax, float amax_floor,
 template <int MODE>
 __device__ __forceinline__ float scale_fast(float v, const BlockScale &b)
 {
-    if (MODE == LP_SCALE_POW2) return ldexpf(v, -b.exp2);
-    if (MODE == LP_SCALE_DIV) return div_by_recip(v, b.div, b.recip);
+    if (pow2_like(MODE)) return ldexpf(v, -b.exp2);
+    if (div_like(MODE)) return div_by_recip(v, b.div, b.recip);
     return v * b.div;
 }
 
@@ -64,8 +76,8 @@ template <int MODE>
 __device__ __forceinline__ uint8_t quant_slow(float v, const BlockScale &b)
 {
     float y;
-    if (MODE == LP_SCALE_POW2) y = v / b.stored;
-    else if (MODE == LP_SCALE_DIV) y = v / b.div;
+    if (pow2_like(MODE)) y = v / b.stored;
+    else if (div_like(MODE)) y = v / b.div;
     else y = v * b.div;
     if (y > kE4M3Max) y = kE4M3Max;
     if (y < -kE4M3Max) y = -kE4M3Max;

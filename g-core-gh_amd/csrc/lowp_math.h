@@ -105,6 +105,15 @@ __device__ __forceinline__ float sw_e2m1_to_f32(uint32_t code, bool neg_zero)
     return u2f(bits);
 }
 
+// e2m1 code of y with ties to the smaller magnitude; the sign bit of y (also of -0) is bit 3
+__device__ __forceinline__ uint32_t sw_f32_to_e2m1_half_down(float y)
+{
+    const float a = __builtin_fabsf(y);
+    uint32_t code = (a > 0.25f) + (a > 0.75f) + (a > 1.25f) + (a > 1.75f) + (a > 2.5f) + (a > 3.5f) + (a > 5.0f);
+    if (a != a) code = 7u;                      // NaN: above every boundary
+    return code | ((f2u(y) >> 28) & 8u);
+}
+
 // Correctly rounded v / s from a correctly rounded reciprocal y = RN(1/s):
 // two residual corrections.  After the first, q1 is a faithful rounding of
 // v/s; the second then lands on RN(v/s) (Markstein).  Requires that neither

@@ -18,15 +18,6 @@ using namespace lowp;
 
 namespace {
 
-// e2m1 code of y with ties to the smaller magnitude; the sign bit of y (also of -0) is bit 3
-__device__ __forceinline__ uint32_t sw_f32_to_e2m1_half_down(float y)
-{
-    const float a = __builtin_fabsf(y);
-    uint32_t code = (a > 0.25f) + (a > 0.75f) + (a > 1.25f) + (a > 1.75f) + (a > 2.5f) + (a > 3.5f) + (a > 5.0f);
-    if (a != a) code = 7u;                      // NaN: above every boundary
-    return code | ((f2u(y) >> 28) & 8u);
-}
-
 // scale exponent from the sign-cleared amax bits (finite): see the file comment
 __device__ __forceinline__ int fp4_scale_exp(uint32_t mbits)
 {

@@ -82,16 +82,16 @@ __global__ __launch_bounds__(256) void quant_tile128(const void *__restrict__ xi
     const float amax = u2f(has_nan ? 0x7FC00000u : mbits);
 
     BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
-    if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
+    if (has_nan && div_like(MODE)) { bs.div = amax; bs.stored = amax; }
     if (t == 0) {
         store_scale(scale_out, scale_dtype, tile, bs.stored);
         if (has_nan && nan_count) atomicAdd(nan_count, 1);
     }
 
-    const bool slow = special || (MODE == LP_SCALE_DIV && !bs.fast);
+    const bool slow = special || (div_like(MODE) && !bs.fast);
     if (slow) {
         // rare: NaN/inf in the block or a scale outside 2^+-60; literal arithmetic, inputs re-read
-        const float d = MODE == LP_SCALE_POW2 ? bs.stored : bs.div;
+        const float d = pow2_like(MODE) ? bs.stored : bs.div;
 #pragma unroll 1
         for (int i = 0; i < NV; ++i)
             quant_slow_span<MODE>(xin, IS_BF16, (row0 + (int64_t)i * row_step) * cols + col0, IS_BF16 ? 8 : 4, d, q);
@@ -180,11 +180,11 @@ __global__ __launch_bounds__(256) void quant_group128(const void *__restrict__ x
         const bool has_nan = mbits > 0x7F800000u;
         const float amax = u2f(has_nan ? 0x7FC00000u : mbits);
         BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
-        if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
-        const bool slow = special || (MODE == LP_SCALE_DIV && !bs.fast);
+        if (has_nan && div_like(MODE)) { bs.div = amax; bs.stored = amax; }
+        const bool slow = special || (div_like(MODE) && !bs.fast);
         if (slow) {
             if (!CHECKED || g < n_groups)
-                quant_slow_span<MODE>(xin, IS_BF16, g * 128 + lane16 * 8, 8, MODE == LP_SCALE_POW2 ? bs.stored : bs.div, q);
+                quant_slow_span<MODE>(xin, IS_BF16, g * 128 + lane16 * 8, 8, pow2_like(MODE) ? bs.stored : bs.div, q);
         } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = clamp448(scale_fast<MODE>(v[j], bs));
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256) void quant_generic(const void *__restrict__ xi
     const bool has_nan = mbits > 0x7F800000u;
     const float amax = u2f(has_nan ? 0x7FC00000u : mbits);
     BlockScale bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
-    if (has_nan && MODE == LP_SCALE_DIV) { bs.div = amax; bs.stored = amax; }
+    if (has_nan && div_like(MODE)) { bs.div = amax; bs.stored = amax; }
     if (t == 0) {
         store_scale(scale_out, scale_dtype, blk, bs.stored);
         if (has_nan && nan_count) atomicAdd(nan_count, 1);
@@ -304,7 +304,7 @@ extern "C" int lp_quant_fp8_block(const void *x, int x_dtype, int64_t rows, int6
     LP_REQUIRE(rows % bm == 0 && cols % bn == 0,
                "lp_quant_fp8_block: shape (%lld, %lld) not divisible by block (%d, %d)", (long long)rows,
                (long long)cols, bm, bn);
-    LP_REQUIRE(scale_mode >= LP_SCALE_POW2 && scale_mode <= LP_SCALE_MUL, "lp_quant_fp8_block: bad scale_mode");
+    LP_REQUIRE(scale_mode >= LP_SCALE_POW2 && scale_mode <= LP_SCALE_RCP_POW2, "lp_quant_fp8_block: bad scale_mode");
     LP_REQUIRE(zero_rule >= LP_ZERO_NONE && zero_rule <= LP_ZERO_SCALE_TO_ONE, "lp_quant_fp8_block: bad zero_rule");
     LP_REQUIRE(amax_floor >= 0.0f, "lp_quant_fp8_block: amax_floor must be >= 0");
     if (rows == 0 || cols == 0) return LP_OK;
@@ -318,6 +318,12 @@ extern "C" int lp_quant_fp8_block(const void *x, int x_dtype, int64_t rows, int6
     case LP_SCALE_DIV:
         return launch_mode<LP_SCALE_DIV>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
                                          scale_dtype, nan_count, st);
+    case LP_SCALE_RCP:
+        return launch_mode<LP_SCALE_RCP>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
+                                         scale_dtype, nan_count, st);
+    case LP_SCALE_RCP_POW2:
+        return launch_mode<LP_SCALE_RCP_POW2>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
+                                              scale_dtype, nan_count, st);
     default:
         return launch_mode<LP_SCALE_MUL>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
                                          scale_dtype, nan_count, st);

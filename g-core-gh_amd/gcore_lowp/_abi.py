@@ -16,7 +16,7 @@ LIB_PATH = os.environ.get("LOWP_LIB") or os.path.join(_HERE, "_lib", "liblowp.so
 # enum lp_dtype
 F32, BF16, E8M0, E4M3 = 0, 1, 2, 3
 # enum lp_scale_mode
-SCALE_POW2, SCALE_DIV, SCALE_MUL = 0, 1, 2
+SCALE_POW2, SCALE_DIV, SCALE_MUL, SCALE_RCP, SCALE_RCP_POW2 = 0, 1, 2, 3, 4
 # enum lp_zero_rule
 ZERO_NONE, ZERO_AMAX_TO_ONE, ZERO_SCALE_TO_ONE = 0, 1, 2
 # enum lp_fp4_zero
@@ -30,6 +30,8 @@ PROTOTYPES = {
     "lp_last_error": (ctypes.c_char_p, []),
     "lp_quant_fp8_block": (_i32, [_p, _i32, _i64, _i64, _i32, _i32, _i32, _f32, _i32, _p, _p, _i32, _p, _p]),
     "lp_quant_fp4_block": (_i32, [_p, _i32, _i64, _i64, _i32, _i32, _p, _p, _p, _p]),
+    "lp_qdq_fp8_tile128": (_i32, [_p, _i64, _i64, _p, _p]),
+    "lp_fp4_qat_to_fp8": (_i32, [_p, _i64, _i64, _p, _p, _p]),
     "lp_dequant_fp8_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _p, _i32, _p]),
     "lp_dequant_fp4_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _p, _i32, _p]),
     "lp_fp4_to_fp8_rebase": (_i32, [_p, _p, _i64, _i64, _p, _p, _i32, _p]),

@@ -48,7 +48,14 @@ enum lp_scale_mode {
     LP_SCALE_DIV = 1,
     /* f = fl(fl(1/amax) * 448), q = cast(clamp(x * f)), stored scale = fl(1/f);
      * tools/convert_fp8/qwen3_5/qwen3_mtp_fp8_postprocess.py:138-149 */
-    LP_SCALE_MUL = 2
+    LP_SCALE_MUL = 2,
+    /* s = max(amax, amax_floor) * fl32(1/448), q = cast(clamp(x / s));
+     * gpatch_v4/kernel/quantize/qat.py:116-223 (act_quant, amax_floor = 1e-4) */
+    LP_SCALE_RCP = 3,
+    /* as LP_SCALE_RCP with s rounded up to a power of two from its bits
+     * (exponent field - 127, + 1 when a mantissa bit is set); act_quant with
+     * scale_fmt set: qat.py:98-113 */
+    LP_SCALE_RCP_POW2 = 4
 };
 
 enum lp_zero_rule {
@@ -152,6 +159,23 @@ int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t rows, int6
  */
 int lp_quant_fp4_block(const void *x, int x_dtype, int64_t rows, int64_t cols, int bm, int bn,
                        void *packed_out, void *scale_out, int32_t *nan_count, lp_stream_t stream);
+
+/*
+ * bf16 [rows, cols] -> e4m3fn with one power-of-two scale per 128 x 128 tile -> bf16, fused:
+ * s = 2^ceil(log2(max(amax, 1e-30) / 448)) from the bits of the quotient (1 for an
+ * all-zero tile), out = bf16(fp32(e4m3(clamp(x / s))) * s).  rows, cols multiples of 128.
+ * Replaces fp_qat_128x128 (gpatch_v4/kernel/quantize/fused_quant_kernels.py:277-403).
+ */
+int lp_qdq_fp8_tile128(const void *x, int64_t rows, int64_t cols, void *out, lp_stream_t stream);
+
+/*
+ * fp32 [rows, cols] -> e2m1 with one scale max(2^ceil(log2(amax / 6)), 2^-126) per 1 x 32 group
+ * (1 for an all-zero group; ties to the smaller magnitude, -0.0 kept) -> rebased to e4m3fn with
+ * one e8m0 scale max(largest group scale / 64, 2^-126) per 128 x 128 tile.  q_out: [rows, cols]
+ * bytes; scale_out: [rows/128, cols/128] e8m0 bytes.  rows, cols multiples of 128.
+ * Replaces fp4_qat_then_to_fp8 (gpatch_v4/kernel/quantize/fused_quant_kernels.py:102-274).
+ */
+int lp_fp4_qat_to_fp8(const void *x, int64_t rows, int64_t cols, void *q_out, void *scale_out, lp_stream_t stream);
 
 /*
  * Block-scaled FP8 GEMM: C[i,j] = cast(sum_kb (sum_{k in kb} Aq[i,k] Bq[j,k]) * As[i,kb] * Bs[j/128,kb]).

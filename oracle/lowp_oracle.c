@@ -174,7 +174,7 @@ int orc_pow2_exponent(float r, int kind)
     return (e - 127) + (m ? 1 : 0);
 }
 
-enum { ORC_SCALE_POW2 = 0, ORC_SCALE_DIV = 1, ORC_SCALE_MUL = 2 };
+enum { ORC_SCALE_POW2 = 0, ORC_SCALE_DIV = 1, ORC_SCALE_MUL = 2, ORC_SCALE_RCP = 3, ORC_SCALE_RCP_POW2 = 4 };
 enum { ORC_ZERO_NONE = 0, ORC_ZERO_AMAX_TO_ONE = 1, ORC_ZERO_SCALE_TO_ONE = 2 };
 
 /*
@@ -188,6 +188,9 @@ enum { ORC_ZERO_NONE = 0, ORC_ZERO_AMAX_TO_ONE = 1, ORC_ZERO_SCALE_TO_ONE = 2 };
  *     tests/test_gfused/test_deepseek_tilekernels_quant.py:22-58 with
  *     amax_floor = 1e-12; tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:29-72
  *     with zero rule SCALE_TO_ONE): s = amax/448, q = cast(clamp(x / s)).
+ * mode RCP / RCP_POW2 (gpatch_v4/kernel/quantize/qat.py:116-223, act_quant with amax_floor = 1e-4):
+ *     s = max(amax, floor) * fl32(1/448), optionally rounded up to a power of two on its bits,
+ *     q = cast(clamp(x / s)).
  * mode MUL  (tools/convert_fp8/qwen3_5/qwen3_mtp_fp8_postprocess.py:138-149):
  *     f = fl(fl(1/amax) * 448) (1 for a zero block), q = cast(clamp(x * f)),
  *     scale_out = fl(1/f).
@@ -216,6 +219,17 @@ int64_t orc_quant_fp8_block(const float *x, int64_t rows, int64_t cols, int bm, 
                 float r = safe / 448.0f;
                 s = ldexpf(1.0f, orc_pow2_exponent(r, log2_kind));
                 if (!(amax > 0.0f)) s = 1.0f;                        /* where(max_abs > 0, s, 1) */
+            } else if (mode == ORC_SCALE_RCP || mode == ORC_SCALE_RCP_POW2) {
+                /* gpatch_v4/kernel/quantize/qat.py:155-161: amax = max(amax, floor); s = amax * fl32(1/448),
+                 * or 2^ceil(log2 s) built on the bits of s (qat.py:98-113) when the scale is rounded */
+                float a = amax;
+                if (a < amax_floor) a = amax_floor;
+                s = a * (float)(1.0 / 448.0);
+                if (mode == ORC_SCALE_RCP_POW2) {
+                    uint32_t b = f2u(s);
+                    int e = (int)((b >> 23) & 0xFFu) - 127 + ((b & 0x7FFFFFu) ? 1 : 0);
+                    s = u2f((uint32_t)(e + 127) << 23);
+                }
             } else if (mode == ORC_SCALE_DIV) {
                 float a = amax;
                 if (a < amax_floor) a = amax_floor;                  /* clamp(min=floor); floor 0 = off */

@@ -90,6 +90,68 @@ def sgl_expert_to_official(weight: torch.Tensor, scale: torch.Tensor):
     return quant_fp4_e2m1_scale_e8m0_packed(full, (1, 32))
 
 
+# --------------------------------------------------------------------- fused QAT kernels (bit-defined scales)
+
+def _log2_ceil_bits(x: torch.Tensor) -> torch.Tensor:
+    """gpatch_v4/kernel/quantize/fused_quant_kernels.py:32-38 / qat.py:98-103: ceil(log2 x) from the fp32 bits,
+    literally (exponent field - 127, + 1 when any mantissa bit is set)."""
+    b = x.contiguous().view(torch.int32)
+    return ((b >> 23) & 0xFF) - 127 + ((b & 0x7FFFFF) != 0).to(torch.int32)
+
+
+def _pow2_bits(e: torch.Tensor) -> torch.Tensor:
+    """fused_quant_kernels.py:41-44: 2^e built as fp32 bits, literally."""
+    return ((e + 127) << 23).to(torch.int32).view(torch.float32)
+
+
+def fp_qat_128x128(weight: torch.Tensor) -> torch.Tensor:
+    """fused_quant_kernels.py:277-403: bf16 [M, N] -> e4m3 quantise / dequantise with one power-of-two scale per
+    128 x 128 tile, s = 2^ceil(log2(max(amax, 1e-30) / 448)) (1 for a zero tile), back to bf16."""
+    assert weight.dtype == torch.bfloat16 and weight.ndim == 2
+    t = _tiles(weight.float(), 128, 128)
+    amax = _tile_amax(t)
+    s = _pow2_bits(_log2_ceil_bits(amax.clamp(min=1.0e-30) / E4M3_MAX))
+    s = torch.where(amax > 0, s, torch.ones_like(s))
+    q = (t / _bcast(s)).clamp(-E4M3_MAX, E4M3_MAX).to(_E4M3)
+    return (q.float() * _bcast(s)).to(torch.bfloat16).reshape(weight.shape)
+
+
+def fp4_qat_then_to_fp8(weight: torch.Tensor):
+    """fused_quant_kernels.py:102-274: fp32 [M, N] -> e2m1 with a 1 x 32 scale max(2^ceil(log2(amax/6)), 2^-126)
+    (1 for a zero group), value half way between two code points to the smaller magnitude, -0.0 kept; then
+    rebased to e4m3 with one e8m0 scale max(largest group scale / 64, 2^-126) per 128 x 128 tile."""
+    assert weight.dtype == torch.float32 and weight.ndim == 2
+    m, n = weight.shape
+    g = weight.reshape(m, n // 32, 32)
+    amax = g.abs().amax(dim=-1)
+    sg = torch.maximum(_pow2_bits(_log2_ceil_bits(amax / 6.0)), torch.tensor(2.0 ** -126))
+    sg = torch.where(amax > 0, sg, torch.ones_like(sg))
+    y = (g / sg.unsqueeze(-1)).clamp(-6.0, 6.0)
+    pos = torch.tensor(_MAG, dtype=torch.float32)
+    idx = torch.bucketize(y.abs().contiguous(), (pos[1:] + pos[:-1]) / 2.0)
+    q4 = torch.where(torch.signbit(y), -pos[idx], pos[idx])                  # -0.0 survives
+    st = sg.reshape(m // 128, 128, n // 128, 4)
+    outer = (st.amax(dim=(1, 3)) / 64.0).clamp(min=2.0 ** -126)              # [M/128, N/128]
+    off = sg.reshape(m // 128, 128, n // 128, 4) / outer[:, None, :, None]
+    q8 = (q4.reshape(m // 128, 128, n // 128, 4, 32) * off.unsqueeze(-1)).reshape(m, n).to(_E4M3)
+    return q8, outer.to(_E8M0)
+
+
+def act_quant(x: torch.Tensor, block_size: int = 128, scale_fmt=None):
+    """gpatch_v4/kernel/quantize/qat.py:116-223 (inplace=False): 1 x block_size groups along the last dim,
+    s = max(amax, 1e-4) * fl32(1/448), rounded up to a power of two when scale_fmt is set;
+    y = e4m3(clamp(x / s)); returns (y, s fp32 [..., N / block_size])."""
+    n = x.size(-1)
+    assert n % block_size == 0
+    g = x.float().reshape(-1, n // block_size, block_size)
+    amax = g.abs().amax(dim=-1).clamp(min=1e-4)
+    s = amax * torch.tensor(1 / 448.0, dtype=torch.float32)
+    if scale_fmt is not None:
+        s = _pow2_bits(_log2_ceil_bits(s))
+    y = (g / s.unsqueeze(-1)).clamp(-E4M3_MAX, E4M3_MAX).to(_E4M3).reshape(x.shape)
+    return y, s.reshape(*x.shape[:-1], n // block_size)
+
+
 # --------------------------------------------------------------------- a2
 
 def quantize_fp8_blockwise(weight: torch.Tensor, block_size, *, device=None, scale_dtype=torch.bfloat16):
