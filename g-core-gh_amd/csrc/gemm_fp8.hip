@@ -384,7 +384,7 @@ static int launch_small(const void *Aq, const void *As, const void *Bq, const vo
 {
     static const char *mid_min = getenv("LP_GEMM_MID_MIN_M");       // tuning aid
     if (M >= (mid_min ? atoi(mid_min) : 64) && gemm::mid_asm_ok(As, Bs, scale_dtype, M, N, K))
-        return gemm::launch_mid_asm(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);
+        return gemm::launch_mid_asm(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, ldc, out_dtype, st);
     const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
     const int64_t grid = padded_grid(tiles_m, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_block: problem too large");
@@ -404,9 +404,11 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     int rc = check_gemm_args("lp_gemm_fp8_block", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
     if (rc) return rc > 0 ? LP_OK : rc;
     hipStream_t st = (hipStream_t)stream;
-    // The hand-scheduled kernels read fp32 scales: with scratch, e8m0 scales are expanded first (one small launch).
+    // e8m0 scales normally go to the kernels whose matrix instructions apply them.  LP_GEMM_E8M0_EXPAND=1 (tuning
+    // aid) instead expands them to fp32 in the caller's scratch and runs the fp32-scale kernels.
+    static const bool expand = getenv("LP_GEMM_E8M0_EXPAND") != nullptr;
     const int64_t sc_bytes = scale_copy_bytes(M, N, K);
-    if (scale_dtype == LP_E8M0 && sc_bytes > 0 && workspace && workspace_bytes >= sc_bytes && (uintptr_t)workspace % 256 == 0) {
+    if (expand && scale_dtype == LP_E8M0 && sc_bytes > 0 && workspace && workspace_bytes >= sc_bytes && (uintptr_t)workspace % 256 == 0) {
         const int64_t na = M * (K / 128), nb = (N / 128) * (K / 128);
         float *fa = (float *)workspace, *fb = (float *)((char *)workspace + round_up(na * 4, 256));
         hipLaunchKernelGGL(scales_to_f32, dim3((unsigned)((na + nb + 255) / 256)), dim3(256), 0, st, (const uint8_t *)As, na,

@@ -222,14 +222,16 @@ struct AsmTile {
     static constexpr int LDS_BYTES = S_LDS + 2 * TM * 16;                        // two stages of KSUB K blocks + scale groups
 };
 
-template <int TM, int TN, int KSUB>
+// HWS: e8m0 scales applied by the matrix cores (v_mfma_scale_*); As / Bs then point at bytes.
+template <int TM, int TN, int KSUB, bool HWS = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
 {
     using T = AsmTile<TM, TN, KSUB>;
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
-    static_assert(TM / 8 / WAVES == 4 && TN / 8 / WAVES == 4, "four copies per operand and wave");
+    static_assert(TM / 8 / WAVES == 4 && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3), "copies per operand and wave");
+    constexpr int NBC = TN / 8 / WAVES;                 // weight copies per wave and K block
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, lq = lane >> 4;
@@ -249,23 +251,33 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     for (int i = 0; i < 4; ++i) {
         const int row = 8 * (wave + WAVES * i) + ld_row;
         const int64_t m = m0 + row < M ? m0 + row : M - 1;
-        const int64_t n = n0 + row < N ? n0 + row : N - 1;
+        const int64_t n = n0 + row < N ? n0 + row : N - 1;          // i = 3 is unused when there are three copies
         aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
         boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
     }
+    (void)NBC;
     // activation scales travel in groups of four K steps through LDS: the first TM / 64 waves copy one row per lane
     int64_t arow[4];
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) arow[mb] = m0 + wm * 64 + mb * 16 + l16;
     const int64_t srow = m0 + (wave % (TM / 64)) * 64 + lane;
-    const uint32_t soff = (uint32_t)((srow < M ? srow : M - 1) * kblocks * 4);
+    constexpr int SS = HWS ? 1 : 4;                      // bytes per scale
+    const uint32_t soff = (uint32_t)((srow < M ? srow : M - 1) * kblocks * SS);
     const uint32_t copies = __builtin_amdgcn_readfirstlane(wave < TM / 64 ? 1u : 0u);
-    // weight scale row of this wave (its columns lie in one scale block)
+    // weight scale row(s) of this wave.  With TN / 2 = 128 or 64 columns per wave they lie in one scale block;
+    // 96 columns can straddle two, and each pair of 16-column blocks is told which of the two rows it uses.
     const int64_t wcol0 = n0 + wn * (TN / 2);
+    const int64_t last_blk = (N >> 7) - 1;
     int64_t sblk = wcol0 >> 7;
-    if (sblk > (N >> 7) - 1) sblk = (N >> 7) - 1;
-    const float *bs_ptr = Bs + sblk * kblocks;
-    const uint64_t bs_u = uniform(bs_ptr);
+    if (sblk > last_blk) sblk = last_blk;
+    const uint64_t bs_u = uniform((const char *)Bs + sblk * kblocks * SS);
+    int64_t sblk2 = (wcol0 + TN / 2 - 1) >> 7;
+    if (sblk2 > last_blk) sblk2 = last_blk;
+    const uint64_t bs2_u = uniform((const char *)Bs + sblk2 * kblocks * SS);
+    // pair p covers columns wcol0 + 32 p .. + 31 (within one scale block since wcol0 is a multiple of 32)
+    const uint32_t sel1 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 32) >> 7) != (wcol0 >> 7)));
+    const uint32_t sel2 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 64) >> 7) != (wcol0 >> 7)));
+    (void)bs2_u; (void)sel1; (void)sel2;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
     // Layout: activation stages, weight stages, scale groups.
@@ -276,10 +288,29 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
     const uint32_t brd0 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq) * 16;
     const uint32_t brd1 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
-    const uint32_t srd = lds0 + T::S_LDS + arow_l * 16;
+    // scale staging: 16 bytes per activation row (fp32, four K steps), or 4 bytes per row in 1 KB per copying wave (e8m0)
+    const uint32_t srd = HWS ? lds0 + T::S_LDS + wm * 1024 + l16 * 4 : lds0 + T::S_LDS + arow_l * 16;
 
     f32x16v accs[NBW];
-    if constexpr (NBW == 8) {
+    if constexpr (HWS && NBW == 8) {
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
+        asm volatile(
+#include "gemm_big_hw_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
+              "={v[192:207]}"(acc4), "={v[208:223]}"(acc5), "={v[224:239]}"(acc6), "={v[240:255]}"(acc7)
+            : LP_ASM_INPUTS
+            : LP_ASM_CLOBBERS);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+        accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+    } else if constexpr (HWS) {
+        f32x16v acc0, acc1, acc2, acc3;
+        asm volatile(
+#include "gemm_mid_hw_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : LP_ASM_INPUTS
+            : LP_ASM_CLOBBERS);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+    } else if constexpr (NBW == 8) {
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
         asm volatile(
 #include "gemm_big_loop.inc"
@@ -289,6 +320,16 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
         accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+    } else if constexpr (NBW == 6) {
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5;
+        asm volatile(
+#include "gemm_big192_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
+              "={v[192:207]}"(acc4), "={v[208:223]}"(acc5)
+            : LP_ASM_INPUTS, [bsptr2] "s"(bs2_u), [sel1] "s"(sel1), [sel2] "s"(sel2)
+            : LP_ASM_CLOBBERS, "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "s64", "s65", "s66", "s67",
+              "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77");
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4; accs[5] = acc5;
     } else if constexpr (KSUB == 1) {
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
@@ -327,7 +368,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 }
 
 
-template <int TM, int TN, int KSUB>
+template <int TM, int TN, int KSUB, bool HWS = false>
 __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                    const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
                                                    int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
@@ -336,7 +377,7 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
     __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB>::LDS_BYTES];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<TM, TN, KSUB>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+    tile_asm<TM, TN, KSUB, HWS>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
 }
 
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
@@ -414,9 +455,10 @@ namespace gemm {
 
 // The hand-scheduled loop addresses operands with 32-bit offsets and moves scales in 16-byte groups
 // of four K steps.
-static bool asm_shape_ok(const void *As, const void *Bs, int64_t M, int64_t N, int64_t K)
+static bool asm_shape_ok(const void *As, const void *Bs, int64_t M, int64_t N, int64_t K, int scale_dtype = LP_F32)
 {
-    return K % 512 == 0 && (((uintptr_t)As | (uintptr_t)Bs) & 15) == 0 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
+    const uintptr_t align = scale_dtype == LP_E8M0 ? 3 : 15;          // one group of four scales per access
+    return K % 512 == 0 && (((uintptr_t)As | (uintptr_t)Bs) & align) == 0 && M * K < 0xFFFFFFFFll && N * K < 0xFFFFFFFFll &&
            M * (K / 128) * 4 < 0xFFFFFFFFll;
 }
 
@@ -446,12 +488,28 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
         return launch_nb<SDT, 4>(Aq, As, Bq, Bs, M, N, K, C, ldc, out_dtype, st);                            \
     } while (0)
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;       // tuning / test aid
-    if (!no_asm && scale_dtype == LP_F32 && tn == 256 && asm_shape_ok(As, Bs, M, N, K)) {
+    if (!no_asm && scale_dtype == LP_E8M0 && tn == 256 && asm_shape_ok(As, Bs, M, N, K, LP_E8M0)) {
+        // e8m0 scales: the matrix cores apply them (no fold, accumulation in place)
         const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
         const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
-        hipLaunchKernelGGL((gemm_asm<256, 256, 1>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq, (const float *)As,
-                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
+        hipLaunchKernelGGL((gemm_asm<256, 256, 1, true>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                           out_dtype);
+        return check_launch("lp_gemm_fp8_block(asm e8m0)");
+    }
+    if (!no_asm && scale_dtype == LP_F32 && (tn == 256 || tn == 192) && asm_shape_ok(As, Bs, M, N, K)) {
+        const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + tn - 1) / tn;
+        const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
+        if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+        if (tn == 256)
+            hipLaunchKernelGGL((gemm_asm<256, 256, 1>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
+        else
+            hipLaunchKernelGGL((gemm_asm<256, 192, 1>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
         return check_launch("lp_gemm_fp8_block(asm)");
     }
     if (scale_dtype == LP_F32) GO(LP_F32);
@@ -463,15 +521,21 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
 bool mid_asm_ok(const void *As, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K)
 {
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr || getenv("LP_GEMM_NO_MID") != nullptr;
-    return !no_asm && scale_dtype == LP_F32 && asm_shape_ok(As, Bs, M, N, K);
+    return !no_asm && (scale_dtype == LP_F32 || scale_dtype == LP_E8M0) && asm_shape_ok(As, Bs, M, N, K, scale_dtype);
 }
 
-int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-                   int64_t ldc, int out_dtype, hipStream_t st)
+int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
+                   int64_t K, void *C, int64_t ldc, int out_dtype, hipStream_t st)
 {
     const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+    if (scale_dtype == LP_E8M0) {
+        hipLaunchKernelGGL((gemm_asm<128, 128, 1, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                           out_dtype);
+        return check_launch("lp_gemm_fp8_block(asm128 e8m0)");
+    }
     // With two K blocks per stage a workgroup keeps twice the bytes in flight but owns the CU's LDS alone:
     // better while there is at most about one tile per CU, worse when two workgroups could share a CU.
     static const char *force = getenv("LP_GEMM_MID_KSUB");           // tuning aid

@@ -35,16 +35,20 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128."""
-    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, lines
+    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, lines
+    HW = hw
     assert tm == 64 * waves_m
     WAVES = waves_m * waves_n
     KSUB = ksub
     A_BYTES, B_BYTES = tm * 128, tn * 128
     SCL_LDS = 2 * ksub * (A_BYTES + B_BYTES)               # activation-scale buffer: 2 halves x tm rows x 16 bytes
-    SCL_HALF = tm * 16
+    SCL_HALF = tm * 16        # (the e8m0 variant uses 4 of every 16 bytes: one wave writes 64 rows x 4 bytes per KB)
     NB = tn // waves_n // 16
+    # a wave whose columns are not a multiple of 128 wide can straddle two weight-scale blocks: two scale rows
+    # are loaded and each pair of 16-column blocks takes the one the set-up code selected for it
+    SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64
     assert (tm // 8) % WAVES == 0 and (tn // 8) % WAVES == 0
     lines = []
 
@@ -60,6 +64,7 @@ def b_lds(stage, sub):
 
 
 ACC, P, AF, SC, SAN = 128, 96, 64, 44, 40
+SCP = (44, 224, 228)        # scale products per pair of 16-column blocks when a wave straddles two weight-scale blocks
 WFB = (48, 56)
 RA0, RA1, RB0, RB1 = 30, 31, 32, 33
 SRD0, SRD = 34, 35
@@ -98,17 +103,26 @@ def scale_group_copy(tag):
     emit("s_add_u32 m0, s48, s54")
     emit(f"s_add_u32 m0, m0, {SCL_LDS}")
     emit("s_nop 0")
-    emit("global_load_lds_dwordx4 %[soff], s[44:45]")
+    emit("global_load_lds_dword %[soff], s[44:45]" if HW else "global_load_lds_dwordx4 %[soff], s[44:45]")
     emit(f"Lnosc{tag}%=:")
-    emit("s_add_u32 s44, s44, 16")
+    emit(f"s_add_u32 s44, s44, {4 if HW else 16}")
     emit("s_addc_u32 s45, s45, 0")
 
 
 def weight_scale_load():
-    """The four weight scales of the next group into s[60:63]."""
+    """The four weight scales of the next group into s[60:63] (and those of the second scale row into s[68:71])."""
+    if HW:
+        emit("s_load_dword s60, s[46:47], 0x0")          # four e8m0 bytes = four K steps
+        emit("s_add_u32 s46, s46, 4")
+        emit("s_addc_u32 s47, s47, 0")
+        return
     emit("s_load_dwordx4 s[60:63], s[46:47], 0x0")
     emit("s_add_u32 s46, s46, 16")
     emit("s_addc_u32 s47, s47, 0")
+    if SPLIT:
+        emit("s_load_dwordx4 s[68:71], s[72:73], 0x0")
+        emit("s_add_u32 s72, s72, 16")
+        emit("s_addc_u32 s73, s73, 0")
 
 
 def read_frag(dst, addr0, addr1, off):
@@ -117,18 +131,34 @@ def read_frag(dst, addr0, addr1, off):
 
 
 def read_scales(col):
-    """Raw activation scales of the lane's four block rows for one K step (column col of the group half at v35)."""
+    """Raw activation scales of the lane's four block rows for one K step (column col of the group half at v35).
+    e8m0 variant: the four bytes of the next group, once per trip, into the spare set v[44:47]."""
+    if HW:
+        if col == 0:
+            for mb in range(MB):
+                emit(f"ds_read_b32 v{SC + mb}, v{SRD} offset:{mb * 64}")
+        return
     for mb in range(MB):
         emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256 + col * 4}")
 
 
-def mfma(nb, mb):
+def mfma(nb, mb, c=0):
+    if HW:
+        # scales applied by the matrix core: byte c of the weight-scale register (uniform) and of the lane's
+        # activation-scale register; accumulation in place
+        acc = vr(ACC + 16 * nb + 4 * mb, 4)
+        emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, v36, v{SAN + mb} "
+             f"op_sel:[{c & 1},{c & 1},0] op_sel_hi:[{c >> 1},{c >> 1},0]")
+        return
     emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * (nb & 1) + 4 * mb, 4)}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, 0")
 
 
 def fold(nb, mb):
+    if HW:
+        return
+    sc = SCP[nb >> 1] if SPLIT else SC
     for r in range(4):
-        emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * (nb & 1) + 4 * mb + r}, v{SC + mb}")
+        emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * (nb & 1) + 4 * mb + r}, v{sc + mb}")
 
 
 def step(c):
@@ -143,8 +173,21 @@ def step(c):
     nstage, nsub = (stage ^ 1, 0) if flip else (stage, sub + 1)
     aoff, boff = a_lds(stage, sub), b_lds(stage, sub)
     naoff, nboff = a_lds(nstage, nsub), b_lds(nstage, nsub)
-    for mb in range(MB):
-        emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
+    if HW:
+        pass
+    elif SPLIT:
+        # pairs 1 and 2 take the second scale row when their flag (s74, s75) is set
+        emit("s_cmp_eq_u32 s74, 1")
+        emit(f"s_cselect_b32 s76, s{64 + c}, s{56 + c}")
+        emit("s_cmp_eq_u32 s75, 1")
+        emit(f"s_cselect_b32 s77, s{64 + c}, s{56 + c}")
+        for mb in range(MB):
+            emit(f"v_mul_f32 v{SCP[0] + mb}, s{56 + c}, v{SAN + mb}")
+            emit(f"v_mul_f32 v{SCP[1] + mb}, s76, v{SAN + mb}")
+            emit(f"v_mul_f32 v{SCP[2] + mb}, s77, v{SAN + mb}")
+    else:
+        for mb in range(MB):
+            emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
     if c == 0:
         # next group of scales: into the other half of the scale buffer
         emit("s_cmp_eq_u32 s50, 1")
@@ -161,13 +204,14 @@ def step(c):
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
     for mb in range(MB):
         emit(f"s_waitcnt lgkmcnt({8 - 2 * mb})")
-        mfma(0, mb)
+        mfma(0, mb, c)
     read_scales((c + 1) & 3)
     for nb in range(1, NB):
         if nb + 1 < NB:
             read_frag(WFB[(nb + 1) & 1], RB0, RB1, boff + (nb + 1) * 2048)
         if nb == 1:
-            emit(f"s_waitcnt lgkmcnt({6 if NB > 2 else 4})")        # 4 scales and wf2 may still be outstanding
+            pending = 4 if (not HW or c == 3) else 0                # scale reads issued after block 0
+            emit(f"s_waitcnt lgkmcnt({pending + (2 if NB > 2 else 0)})")        # those and wf2 may still be outstanding
         elif nb + 1 < NB:
             emit("s_waitcnt lgkmcnt(2)")
         if nb + 1 == NB:
@@ -179,7 +223,7 @@ def step(c):
                 emit("s_waitcnt lgkmcnt(0)")
             read_frag(WFB[0], RB0, RB1, nboff)
         for mb in range(MB):
-            mfma(nb, mb)
+            mfma(nb, mb, c)
             fold(nb - 1, mb)
             if nb + 1 == NB:
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
@@ -203,6 +247,10 @@ def generate():
     emit("s_mov_b64 s[42:43], %[bbase]")
     emit("s_mov_b64 s[44:45], %[sbase]")
     emit("s_mov_b64 s[46:47], %[bsptr]")
+    if SPLIT:
+        emit("s_mov_b64 s[72:73], %[bsptr2]")
+        emit("s_mov_b32 s74, %[sel1]")
+        emit("s_mov_b32 s75, %[sel2]")
     emit("s_mov_b32 s48, %[m0base]")
     emit("s_mov_b32 s49, %[trips]")
     emit("s_mov_b32 s53, %[copies]")
@@ -210,7 +258,7 @@ def generate():
     emit("s_mov_b32 s55, 0")
     for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
         emit(f"v_mov_b32 v{reg}, %[{name}]")
-    for r in range(128):
+    for r in range(16 * NB):
         emit(f"v_mov_b32 v{ACC + r}, 0")
     scale_group_copy("a")
     weight_scale_load()
@@ -219,15 +267,23 @@ def generate():
     emit("s_barrier")
     dma(1)                                   # K >= 512: there are at least four steps, which two stages hold at most
     for mb in range(MB):
-        emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256}")
+        emit(f"ds_read_b32 v{(SC if HW else SAN) + mb}, v{SRD} offset:{mb * (64 if HW else 256)}")
     emit("s_waitcnt lgkmcnt(0)")
     read_frag(WFB[0], RB0, RB1, 0)
     for mb in range(MB):
         read_frag(AF + 8 * mb, RA0, RA1, mb * 2048)
     # ---- main loop: one trip = four K steps = one group of scales
     emit("Lloop%=:")
+    if HW:
+        # scales of this group: the lane's activation-scale bytes and the weight-scale bytes (uniform)
+        for mb in range(MB):
+            emit(f"v_mov_b32 v{SAN + mb}, v{SC + mb}")
+        emit("v_mov_b32 v36, s60")
     emit("s_mov_b64 s[56:57], s[60:61]")
     emit("s_mov_b64 s[58:59], s[62:63]")
+    if SPLIT:
+        emit("s_mov_b64 s[64:65], s[68:69]")
+        emit("s_mov_b64 s[66:67], s[70:71]")
     emit("s_sub_u32 s49, s49, 1")
     emit("s_cmp_eq_u32 s49, 0")
     emit("s_cselect_b32 s50, 1, 0")
@@ -236,13 +292,17 @@ def generate():
     emit("s_cmp_lg_u32 s50, 1")
     emit("s_cbranch_scc1 Lloop%=")
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    if HW:
+        emit("s_nop 15")                         # the last MFMAs have written the accumulators before they are read
+        emit("s_nop 15")
 
 
 
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
-    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)),
-                      ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2))):
+    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
+                      ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
+                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True)), ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True))):
         configure(*cfg)
         generate()
         with open(os.path.join(here, name), "w") as f:
