@@ -159,7 +159,21 @@ def main():
     qa_ms, _ = time_launches([lambda: quant_into(a_bf, 1, 128, aq, a_s)], 20, 3)
     extras["c2_act_quant_1x128"] = {"ms": qa_ms, "GB/s": (M * K * 3 + M * K // 32) / qa_ms / 1e6,
                                     "hbm_frac": (M * K * 3 + M * K // 32) / qa_ms / 1e6 / HBM_PEAK_GBS}
-    del bq, b_s, c, a_bf
+    # the same problem with power-of-two (e8m0) scales on both operands, the reference's default scale_dtype
+    # (gfused/mygemm_fp8.py:55): the matrix instructions apply the scales themselves
+    a_s8 = torch.empty(M, K // 128, dtype=torch.uint8, device=dev)
+    chk(L.lp_quant_fp8_block(a_bf.data_ptr(), A.BF16, M, K, 1, 128, A.SCALE_POW2, 0.0, 0, aq.data_ptr(), a_s8.data_ptr(),
+                             A.E8M0, None, stream()))
+    b_s8 = [torch.randint(118, 124, (N // 128, K // 128), dtype=torch.uint8, device=dev) for _ in range(n_sets)]
+
+    def gemm8_call(i):
+        return lambda: chk(L.lp_gemm_fp8_block(aq.data_ptr(), a_s8.data_ptr(), bq[i].data_ptr(), b_s8[i].data_ptr(), A.E8M0,
+                                                M, N, K, c.data_ptr(), A.BF16, None, 0, stream()))
+
+    ms8, _ = time_launches([gemm8_call(i) for i in range(n_sets)], args.steps, args.warmup)
+    extras["c2_gemm_e8m0_scales"] = {"ms": ms8, "tflops": flops / (ms8 * 1e-3) / 1e12,
+                                     "mfma_frac": flops / (ms8 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
+    del bq, b_s, c, a_bf, a_s8, b_s8
     torch.cuda.empty_cache()
 
     if not args.no_extras:

@@ -486,7 +486,7 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
     LP_REQUIRE(m_offsets, "lp_gemm_fp8_grouped: null m_offsets");
     // many rows per expert on average: 256-row tiles on the hand-scheduled kernel
     if (gemm::big_grouped_ok(As, Bs, scale_dtype, M_total, N, K))
-        return gemm::launch_big_grouped(Aq, As, Bq, Bs, m_offsets, E, M_total, N, K, C, out_dtype, (hipStream_t)stream);
+        return gemm::launch_big_grouped(Aq, As, Bq, Bs, scale_dtype, m_offsets, E, M_total, N, K, C, out_dtype, (hipStream_t)stream);
     const int64_t max_mtiles = M_total / TM + E, tiles_n = N / TN;
     const int64_t grid = padded_grid(max_mtiles, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_grouped: problem too large");

@@ -388,7 +388,7 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
 //   2  what PART 1 leaves, i.e. the last M_e % 256 rows, in tiles of TM
 // Launching 1 with 256 x 256 tiles and then 2 with 128 x 128 tiles keeps the large tiles full and bounds the
 // padding of an expert by 127 rows.
-template <int TM, int TN, int KSUB, int PART>
+template <int TM, int TN, int KSUB, int PART, bool HWS = false>
 __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                            const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
                                                            const int32_t *__restrict__ m_offsets, int E, int64_t N,
@@ -432,8 +432,9 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
     const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
     const int64_t first = PART == 2 ? row_begin + (row_end - row_begin) / 256 * 256 : row_begin;
     const int64_t kblocks = K / KB;
-    tile_asm<TM, TN, KSUB>(smem, Aq, As, Bq + (int64_t)e * N * K, Bs + (int64_t)e * (N / 128) * kblocks,
-                           first + (gmt - found_first) * TM, row_end, tn * TN, N, K, C, N, out_dtype);
+    const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
+    tile_asm<TM, TN, KSUB, HWS>(smem, Aq, As, Bq + (int64_t)e * N * K, bs_e, first + (gmt - found_first) * TM, row_end,
+                                tn * TN, N, K, C, N, out_dtype);
 }
 
 template <int SDT, int NB>
@@ -555,12 +556,24 @@ int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *B
 bool big_grouped_ok(const void *As, const void *Bs, int scale_dtype, int64_t M_total, int64_t N, int64_t K)
 {
     static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;
-    return !no_asm && scale_dtype == LP_F32 && N % 256 == 0 && asm_shape_ok(As, Bs, M_total, N, K);
+    return !no_asm && (scale_dtype == LP_F32 || scale_dtype == LP_E8M0) && N % 256 == 0 &&
+           asm_shape_ok(As, Bs, M_total, N, K, scale_dtype);
 }
 
-int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,
-                       int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype, hipStream_t st)
+int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                       const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype,
+                       hipStream_t st)
 {
+    if (scale_dtype == LP_E8M0) {
+        // e8m0 scales: 128 x 128 tiles on the kernel whose matrix instructions apply the scales
+        const int64_t mtiles = M_total / 128 + E;
+        const int64_t grid = padded_grid(mtiles, N / 128);
+        if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
+        hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 0, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, mtiles, N / 128, C,
+                           out_dtype);
+        return check_launch("lp_gemm_fp8_grouped(asm 128 e8m0)");
+    }
     // Few rows per expert on average: the weights of most experts are read for one or two row tiles, so the launch
     // is as much a weight stream as a GEMM.  128 x 128 tiles (two workgroups per CU, tiles taken from both ends
     // of the expert list) let streaming tiles and compute-bound tiles overlap and bound the padding per expert

@@ -160,6 +160,24 @@ def test_gemm_grouped(G, case):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("case", [(8, 512, 512, [700, 0, 300, 1, 255, 256, 257, 600]), (4, 256, 1024, [300, 0, 255, 513]),
+                                  (3, 384, 512, [300, 0, 77])], ids=lambda c: "E%d_N%d_K%d" % c[:3])
+def test_gemm_grouped_e8m0_scales(G, case):
+    """power-of-two scales on both operands: the kernels whose matrix instructions apply the scales"""
+    E, N, K, m_splits = case
+    M = sum(m_splits)
+    say("gemm grouped e8m0", E, N, K, "M=", M)
+    x = I.act_like(M, K, E + N)
+    w = (torch.randn(E, N, K, generator=torch.Generator().manual_seed(E)) * 0.02).to(torch.bfloat16)
+    xq, xs = T.quant_fp8_e4m3_scale_e8m0(x, (1, 128))
+    wq, ws = T.quant_fp8_e4m3_scale_e8m0(w, (128, 128))
+    offs = torch.zeros(E + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+    out = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda())
+    ref = T.grouped_gemm_fp8_ref(xq, xs.float(), wq, ws.float(), m_splits)
+    check(out, ref, f"grouped e8m0 {case[:3]}")
+
+
 def test_grouped_linear_module(G):
     E, N, K = 4, 256, 512
     m_splits = [100, 0, 31, 200]
