@@ -330,6 +330,14 @@ def main():
                                 for i in range(qs)], 18, 6)
         extras["fp_qat_128x128_2048x7168"] = {"ms": msq, "GB/s": eq * 4 / msq / 1e6, "hbm_frac": eq * 4 / msq / 1e6 / HBM_PEAK_GBS,
                                               "bytes": eq * 4}
+        msq, _ = time_launches([(lambda i=i: chk(L.lp_fp4_qdq_row32(wqb[i].data_ptr(), eq, bo.data_ptr(), None, stream())))
+                                for i in range(qs)], 18, 6)
+        extras["fp4_simulate_qat_2048x7168"] = {"ms": msq, "GB/s": eq * 4 / msq / 1e6, "hbm_frac": eq * 4 / msq / 1e6 / HBM_PEAK_GBS,
+                                                "bytes": eq * 4}
+        msq, _ = time_launches([(lambda i=i: chk(L.lp_act_qdq_group(wqb[i].data_ptr(), eq, 64, 1, 0, bo.data_ptr(), None, stream())))
+                                for i in range(qs)], 18, 6)
+        extras["fp8_simulate_qat_1x64_2048x7168"] = {"ms": msq, "GB/s": eq * 4 / msq / 1e6,
+                                                     "hbm_frac": eq * 4 / msq / 1e6 / HBM_PEAK_GBS, "bytes": eq * 4}
         del wq32, wqb, q8o, s8o, bo
         del bufs, bouts
         torch.cuda.empty_cache()

@@ -32,6 +32,8 @@ PROTOTYPES = {
     "lp_quant_fp4_block": (_i32, [_p, _i32, _i64, _i64, _i32, _i32, _p, _p, _p, _p]),
     "lp_qdq_fp8_tile128": (_i32, [_p, _i64, _i64, _p, _p]),
     "lp_fp4_qat_to_fp8": (_i32, [_p, _i64, _i64, _p, _p, _p]),
+    "lp_fp4_qdq_row32": (_i32, [_p, _i64, _p, _p, _p]),
+    "lp_act_qdq_group": (_i32, [_p, _i64, _i32, _i32, _i32, _p, _p, _p]),
     "lp_dequant_fp8_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _p, _i32, _p]),
     "lp_dequant_fp4_block": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _p, _i32, _p]),
     "lp_fp4_to_fp8_rebase": (_i32, [_p, _p, _i64, _i64, _p, _p, _i32, _p]),

@@ -178,6 +178,30 @@ int lp_qdq_fp8_tile128(const void *x, int64_t rows, int64_t cols, void *out, lp_
 int lp_fp4_qat_to_fp8(const void *x, int64_t rows, int64_t cols, void *q_out, void *scale_out, lp_stream_t stream);
 
 /*
+ * bf16 -> e2m1 with one power-of-two scale per 32 consecutive values -> bf16, fused.  n values
+ * (n % 32 == 0; a [.., N] tensor with N % 32 == 0 is passed flat):
+ * s = 2^e, e = ceil(log2(max(amax, 6 * 2^-126) * fl32(1/6))) taken from the bits of the product;
+ * out = bf16(e2m1(clamp(x / s, +-6)) * s), ties of the e2m1 rounding to the smaller magnitude,
+ * -0.0 kept.  scale_out (optional, may be NULL): n / 32 e8m0 bytes (e + 127).
+ * Replaces _fp4_quant_kernel / _fp4_simulate (gpatch_v4/kernel/quantize/qat.py:226-279, 350-366).
+ */
+int lp_fp4_qdq_row32(const void *x, int64_t n, void *out, void *scale_out, lp_stream_t stream);
+
+/*
+ * bf16 -> 8-bit grid with one scale per `group` consecutive values -> bf16, fused.  n values
+ * (n % group == 0, group a power of two in 8..512):
+ * s = max(amax, 1e-4) * fl32(1/448), rounded up to a power of two on its bits when pow2_scale.
+ *   through_bf16 == 0: out = bf16(fp32(e4m3(clamp(x / s, +-448))) * s)    (pow2_scale must be 1)
+ *     = act_quant(x, group, "ue8m0") followed by per_token_cast_back, i.e. _fp8_simulate
+ *     (gpatch_v4/kernel/quantize/qat.py:286-301).
+ *   through_bf16 == 1: out = bf16(fp32(bf16(clamp(x / s, +-448))) * s), what act_quant(inplace=True)
+ *     computes (qat.py:131,163-175: the branch casts the quotient to its output type, bf16).
+ * scale_out (optional, may be NULL): n / group fp32 scales.
+ */
+int lp_act_qdq_group(const void *x, int64_t n, int group, int pow2_scale, int through_bf16, void *out,
+                     void *scale_out, lp_stream_t stream);
+
+/*
  * Block-scaled FP8 GEMM: C[i,j] = cast(sum_kb (sum_{k in kb} Aq[i,k] Bq[j,k]) * As[i,kb] * Bs[j/128,kb]).
  * Aq: device e4m3fn [M,K]; As: device [M,K/128]; Bq: device e4m3fn [N,K];
  * Bs: device [N/128,K/128]; scales of scale_dtype (LP_F32 or LP_E8M0);

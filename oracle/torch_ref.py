@@ -152,6 +152,46 @@ def act_quant(x: torch.Tensor, block_size: int = 128, scale_fmt=None):
     return y, s.reshape(*x.shape[:-1], n // block_size)
 
 
+def act_quant_inplace(x: torch.Tensor, block_size: int = 128, scale_fmt=None) -> torch.Tensor:
+    """gpatch_v4/kernel/quantize/qat.py:116-223 with inplace=True: the kernel's output type is then the input type
+    (:131), so the quotient is cast to bf16, not to e4m3 (:163-175): bf16(fp32(bf16(clamp(x / s))) * s)."""
+    assert x.dtype == torch.bfloat16
+    n = x.size(-1)
+    g = x.float().reshape(-1, n // block_size, block_size)
+    s = g.abs().amax(dim=-1).clamp(min=1e-4) * torch.tensor(1 / 448.0, dtype=torch.float32)
+    if scale_fmt is not None:
+        s = _pow2_bits(_log2_ceil_bits(s))
+    s = s.unsqueeze(-1)
+    y = (g / s).clamp(-E4M3_MAX, E4M3_MAX).to(torch.bfloat16)
+    return (y.float() * s).to(torch.bfloat16).reshape(x.shape)
+
+
+def fp8_simulate(x: torch.Tensor, block_size: int) -> torch.Tensor:
+    """qat.py:286-301: act_quant(x, block_size, "ue8m0") then tile_kernels' per_token_cast_back, which is
+    fp32(y) * s cast to the output type (bf16)."""
+    assert x.dtype == torch.bfloat16
+    y, s = act_quant(x, block_size, "ue8m0")
+    n = x.size(-1)
+    out = y.float().reshape(-1, n // block_size, block_size) * s.reshape(-1, n // block_size, 1)
+    return out.to(torch.bfloat16).reshape(x.shape)
+
+
+def fp4_simulate(x: torch.Tensor, block_size: int = 32) -> torch.Tensor:
+    """qat.py:226-279, 350-366: bf16 -> e2m1 quantise / dequantise per 1 x 32 group with
+    s = 2^ceil(log2(max(amax, 6 * 2^-126) * fl32(1/6))) taken from the bits of the product; a quotient half way
+    between two code points goes to the smaller magnitude (fused_quant_kernels.py:65-99); -0.0 is kept."""
+    assert x.dtype == torch.bfloat16 and block_size == 32
+    n = x.size(-1)
+    g = x.float().reshape(-1, n // 32, 32)
+    amax = g.abs().amax(dim=-1).clamp(min=6.0 * 2.0 ** -126)
+    s = _pow2_bits(_log2_ceil_bits(amax * torch.tensor(1.0 / 6.0, dtype=torch.float32))).unsqueeze(-1)
+    y = (g / s).clamp(-6.0, 6.0)
+    pos = torch.tensor(_MAG, dtype=torch.float32)
+    idx = torch.bucketize(y.abs().contiguous(), (pos[1:] + pos[:-1]) / 2.0)
+    q4 = torch.where(torch.signbit(y), -pos[idx], pos[idx])
+    return (q4 * s).to(torch.bfloat16).reshape(x.shape)
+
+
 # --------------------------------------------------------------------- a2
 
 def quantize_fp8_blockwise(weight: torch.Tensor, block_size, *, device=None, scale_dtype=torch.bfloat16):

@@ -112,5 +112,143 @@ def test_act_quant(fmt, dtype):
     y, s = act_quant(x.cuda()[..., :256].contiguous(), 64, fmt)          # another group size
     wy, ws = T.act_quant(x[..., :256].contiguous(), 64, fmt)
     assert torch.equal(u8(y), u8(wy)) and np.array_equal(s.cpu().numpy().view(np.uint32), ws.numpy().view(np.uint32))
-    with pytest.raises(NotImplementedError):
-        act_quant(x.cuda(), 128, fmt, inplace=True)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# fake-quantisers of training with their straight-through wrappers (gpatch_v4/kernel/quantize/qat.py:226-431)
+
+def bits16(t):
+    return t.detach().cpu().contiguous().view(torch.int16)
+
+
+def test_fp4_simulate_qat_known_answer_and_ste():
+    """tests/test_gfused/test_deepseek_v4_fp4_qat.py:37-80"""
+    from gcore_lowp.qat import fp4_simulate_qat
+    from tests.test_oracle_qat import fp4_known_answer
+    say("fp4_simulate_qat known answer")
+    x, want = fp4_known_answer()
+    x = x.cuda().requires_grad_()
+    g = torch.randn_like(x)
+    y = fp4_simulate_qat(x)
+    y.backward(g)
+    assert y.shape == x.shape and y.dtype == x.dtype and torch.isfinite(y).all()
+    assert torch.equal(y.detach().cpu(), want)
+    assert torch.equal(x.grad, g)
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (3, 5, 96), (1, 32), (4096, 7168), (1000, 1056)])
+def test_fp4_simulate_qat_matches_oracle(shape):
+    from gcore_lowp.qat import fp4_simulate_qat
+    say("fp4_simulate_qat", shape)
+    torch.manual_seed(29)
+    x = torch.randn(shape) * torch.logspace(-3, 3, shape[-1] // 32).repeat_interleave(32)
+    x.view(-1)[:32] = 0
+    x.view(-1)[5] = -0.0
+    x = x.bfloat16()
+    got = fp4_simulate_qat(x.cuda())
+    assert torch.equal(bits16(got), bits16(T.fp4_simulate(x)))
+
+
+def test_fp4_simulate_qat_equals_export_weight():
+    """test_deepseek_v4_fp4_qat.py:97-160: the training forward equals the weight the export path produces, on random
+    data, on exact midpoints and after a step across the group-scale boundaries (two different kernels here)."""
+    from gcore_lowp.eager_quant_kernels import dequant_fp4_e2m1_fp8_scale_e8m0_packed
+    from gcore_lowp.fused_quant_kernels import fp4_qat_then_to_fp8
+    from gcore_lowp.qat import fp4_simulate_qat
+    from tests.test_oracle_qat import FP4_MIDPOINTS
+
+    def export(w):
+        q, s = fp4_qat_then_to_fp8(w.bfloat16().float())
+        return dequant_fp4_e2m1_fp8_scale_e8m0_packed(q, s).float()
+
+    say("fp4 qat forward == export")
+    torch.manual_seed(29)
+    w = torch.randn(256, 512, device="cuda").bfloat16().float()
+    assert torch.equal(fp4_simulate_qat(w.bfloat16()).float(), export(w))
+    row = torch.tensor(FP4_MIDPOINTS, device="cuda").repeat(16)
+    w = row.expand(128, 128).clone()
+    w[1::2] *= -1.0
+    assert torch.equal(fp4_simulate_qat(w.bfloat16()).float(), export(w))
+    torch.manual_seed(31)
+    w = fp4_simulate_qat(torch.randn(256, 512, device="cuda").bfloat16()).float()
+    signs = torch.randint(0, 2, w.shape, device="cuda").float()
+    stepped = w + (signs * 2.0 - 1.0) * 1e-6
+    assert torch.equal(fp4_simulate_qat(stepped.bfloat16()).float(), export(stepped))
+
+
+def test_fp4_simulate_qat_tiny_magnitudes():
+    from gcore_lowp.qat import fp4_simulate_qat
+    say("fp4_simulate_qat tiny")
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(64, 256, generator=g)
+    x[:, :64] *= 1e-36
+    x[:, 64:128] *= 1e-38
+    x[:, 128:160] = 0
+    x = x.bfloat16()
+    assert torch.equal(bits16(fp4_simulate_qat(x.cuda())), bits16(T.fp4_simulate(x)))
+
+
+@pytest.mark.parametrize("bs", [64, 128])
+def test_fp8_simulate_qat_and_ste(bs):
+    from gcore_lowp.qat import fp8_simulate_qat
+    say("fp8_simulate_qat", bs)
+    torch.manual_seed(5)
+    x = (torch.randn(6, 5, 512) * torch.logspace(-6, 3, 6).view(6, 1, 1)).bfloat16()
+    xg = x.cuda().requires_grad_()
+    y = fp8_simulate_qat(xg, bs)
+    g = torch.randn_like(xg)
+    y.backward(g)
+    assert torch.equal(bits16(y), bits16(T.fp8_simulate(x, bs)))
+    assert torch.equal(xg.grad, g)
+    big = torch.randn(4096, 7168, generator=torch.Generator().manual_seed(1)).bfloat16()
+    assert torch.equal(bits16(fp8_simulate_qat(big.cuda(), bs)), bits16(T.fp8_simulate(big, bs)))
+
+
+def test_fp8_simulate_qat_128x128_and_linears():
+    """tests/test_gfused/test_fp_qat_128x128.py:204-221,279-292,337-353"""
+    from gcore_lowp.qat import fp4_qat_linear, fp8_qat_linear, fp8_simulate_qat_128x128
+    say("fp8_simulate_qat_128x128 + linears")
+    torch.manual_seed(3)
+    w = torch.randn(128, 256, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    g = torch.randn_like(w)
+    y = fp8_simulate_qat_128x128(w)
+    assert torch.equal(bits16(y), bits16(T.fp_qat_128x128(w.detach().cpu())))
+    y.backward(g)
+    assert torch.equal(w.grad, g)
+    torch.manual_seed(29)
+    gate_up = torch.randn(2, 256, 128, device="cuda", dtype=torch.bfloat16)
+    stacked = fp8_simulate_qat_128x128(gate_up)
+    per = torch.stack([fp8_simulate_qat_128x128(gate_up[i]) for i in range(2)])
+    assert torch.equal(bits16(stacked), bits16(per))
+    assert torch.equal(bits16(stacked), bits16(T.fp_qat_128x128(gate_up.cpu().view(-1, 128)).view_as(gate_up)))
+    with pytest.raises(ValueError):
+        fp8_simulate_qat_128x128(torch.zeros(128, device="cuda"))
+    torch.manual_seed(23)
+    lin = torch.nn.Linear(128, 256, bias=False, device="cuda", dtype=torch.bfloat16)
+    x = torch.randn(4, 128, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        want = torch.nn.functional.linear(x, T.fp_qat_128x128(lin.weight.detach().cpu()).cuda())
+    assert torch.equal(bits16(fp8_qat_linear(lin, x, 128)), bits16(want))
+    with pytest.raises(AssertionError):
+        fp8_qat_linear(lin, x, 64)
+    mod = torch.nn.Linear(64, 32, device="cuda", dtype=torch.bfloat16)
+    xi = torch.randn(4, 64, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    out = fp4_qat_linear(mod, xi)
+    out.float().square().mean().backward()
+    assert out.shape == (4, 32) and torch.isfinite(out).all()
+    assert mod.weight.grad is not None and torch.isfinite(mod.weight.grad).all()
+    with torch.no_grad():
+        want = torch.nn.functional.linear(xi, T.fp4_simulate(mod.weight.detach().cpu()).cuda(), mod.bias)
+    assert torch.equal(bits16(out), bits16(want))
+
+
+@pytest.mark.parametrize("fmt", [None, "ue8m0"])
+def test_act_quant_inplace_branch(fmt):
+    from gcore_lowp.qat import act_quant
+    say("act_quant inplace", fmt)
+    torch.manual_seed(9)
+    x = (torch.randn(7, 33, 384) * torch.logspace(-6, 3, 7).view(7, 1, 1)).bfloat16()
+    xg = x.cuda()
+    r = act_quant(xg, 128, fmt, inplace=True)
+    assert r is xg
+    assert torch.equal(bits16(xg), bits16(T.act_quant_inplace(x, 128, fmt)))

@@ -80,3 +80,70 @@ def test_act_quant_against_c_restatement_and_invariants(corc):
         back = y.float().reshape(64, 4, 128) * s.unsqueeze(-1)
         err = (back - x.float().reshape(64, 4, 128)).abs()
         assert bool((err <= s.unsqueeze(-1) * 16.0 + 1e-12).all())     # half an e4m3 step at the top binade
+
+
+# tests/test_gfused/test_deepseek_v4_fp4_qat.py:37-62: the reference's own known-answer vector for the FP4
+# fake-quantiser (amax 6 -> scale 1; the doubled row -> scale 2)
+FP4_QAT_VALUES = [-5.5, -4.75, -3.75, -3.25, -2.75, -2.25, -1.85, -1.65, -1.35, -1.15, -0.9, -0.6, -0.4, -0.2, -0.1, 0.0,
+                  0.1, 0.2, 0.4, 0.6, 0.9, 1.15, 1.35, 1.65, 1.85, 2.25, 2.75, 3.25, 3.75, 4.75, 5.25, 6.0]
+FP4_QAT_EXPECTED = [-6.0, -4.0, -4.0, -3.0, -3.0, -2.0, -2.0, -1.5, -1.5, -1.0, -1.0, -0.5, -0.5, 0.0, 0.0, 0.0,
+                    0.0, 0.0, 0.5, 0.5, 1.0, 1.0, 1.5, 1.5, 2.0, 2.0, 3.0, 3.0, 4.0, 4.0, 6.0, 6.0]
+FP4_MIDPOINTS = (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0)
+
+
+def fp4_known_answer():
+    v = torch.tensor(FP4_QAT_VALUES, dtype=torch.bfloat16)
+    e = torch.tensor(FP4_QAT_EXPECTED, dtype=torch.bfloat16)
+    x = torch.stack([torch.cat([v, v]), torch.cat([v * 2, v * 2])]).unsqueeze(1).expand(-1, 3, -1).clone()
+    want = torch.stack([torch.cat([e, e]), torch.cat([e * 2, e * 2])]).unsqueeze(1).expand(-1, 3, -1)
+    return x, want
+
+
+def sgl_export_effective(weight):
+    """test_deepseek_v4_fp4_qat.py:29-35: what the sampler multiplies by after the export of an FP4-QAT expert"""
+    q, s = T.fp4_qat_then_to_fp8(weight.bfloat16().float())
+    return T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(q, s).float()
+
+
+def test_fp4_simulate_known_answer_and_export_agreement():
+    x, want = fp4_known_answer()
+    got = T.fp4_simulate(x)
+    assert torch.equal(got.float().abs(), want.float().abs()) and torch.equal(torch.signbit(got) | (got == 0), torch.signbit(want) | (want == 0))
+    # :97-133: the training forward equals the exported weight, on random data and on exact midpoints
+    torch.manual_seed(29)
+    w = torch.randn(256, 512).bfloat16().float()
+    assert torch.equal(T.fp4_simulate(w.bfloat16()).float(), sgl_export_effective(w))
+    row = torch.tensor(FP4_MIDPOINTS).repeat(16)
+    w = row.expand(128, 128).clone()
+    w[1::2] *= -1.0
+    assert torch.equal(T.fp4_simulate(w.bfloat16()).float(), sgl_export_effective(w))
+    # :136-160: still equal after a step that crosses the group-scale boundaries
+    torch.manual_seed(31)
+    w = T.fp4_simulate(torch.randn(256, 512).bfloat16()).float()
+    signs = torch.randint(0, 2, w.shape).float()
+    stepped = w + (signs * 2.0 - 1.0) * 1e-6
+    assert torch.equal(T.fp4_simulate(stepped.bfloat16()).float(), sgl_export_effective(stepped))
+    # scale bits: the product with fl32(1/6) gives the smallest 2^e with 6 * 2^e >= amax for every bf16 amax
+    bits = torch.arange(0x01C0, 0x7F00, dtype=torch.int32)          # from the floor 6 * 2^-126 up
+    amax = (bits << 16).view(torch.float32)
+    e = T._log2_ceil_bits(amax * torch.tensor(1.0 / 6.0, dtype=torch.float32)).double()
+    a = amax.double()
+    assert bool((6.0 * torch.exp2(e) >= a).all()) and bool((6.0 * torch.exp2(e - 1) < a).all())
+
+
+def test_fp8_simulate_and_inplace_branch():
+    torch.manual_seed(5)
+    x = (torch.randn(6, 5, 256) * torch.logspace(-6, 3, 6).view(6, 1, 1)).bfloat16()
+    for bs in (64, 128):
+        y = T.fp8_simulate(x, bs)
+        # quantise (pinned act_quant) then multiply back: every product is exact and fits bf16
+        q, s = T.act_quant(x, bs, "ue8m0")
+        ref = (q.float().reshape(6, 5, 256 // bs, bs).double() * s.double().unsqueeze(-1)).reshape(x.shape)
+        assert torch.equal(y.double(), ref)
+        # with a power-of-two scale the in-place branch of the activation quantiser is the identity:
+        # the quotient is exact, bf16 holds it, and the product restores x
+        assert torch.equal(T.act_quant_inplace(x, bs, "ue8m0").view(torch.int16), x.view(torch.int16))
+        # without rounding of the scale it is a genuine double rounding through bf16, within 2 ulp of x
+        z = T.act_quant_inplace(x, bs, None)
+        rel = ((z.double() - x.double()).abs() / x.double().abs().clamp(min=1e-30)).max()
+        assert 0 < rel < 2.0 ** -7
