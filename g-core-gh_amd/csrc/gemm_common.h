@@ -60,6 +60,10 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
 
 // gemm_skinny.hip: at most 64 activation rows
 constexpr int kSkinnyBlocks = 7;          // K blocks one workgroup handles
+// at most 16 activation rows: one workgroup per 16 weight rows over all of K (gemm_thin.hip)
+bool thin_ok(int64_t M, int64_t N, int64_t K);
+int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
+                void *C, int out_dtype, hipStream_t st);
 void skinny_plan(int64_t N, int64_t K, int &splits, int &per);
 int64_t skinny_workspace_bytes(int64_t N, int splits);
 int launch_skinny(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,

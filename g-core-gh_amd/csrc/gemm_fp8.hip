@@ -419,6 +419,8 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
                                  workspace_bytes - sc_bytes, stream);
     }
     static const bool no_skinny = getenv("LP_GEMM_NO_SKINNY") != nullptr;       // tuning aid
+    static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;           // tuning aid
+    if (!no_thin && gemm::thin_ok(M, N, K)) return gemm::launch_thin(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, st);
     if (M <= 64 && !no_skinny) {
         // decode-sized: the weight-streaming kernel, when the caller gave scratch for its K ranges and one range
         // fits its window of K blocks (longer ranges are better served by the tiled kernels below)

@@ -71,6 +71,8 @@ DENSE_SHAPES = [
     # between the 256 x 256 and the 128 x 128 kernel (576 tiles on 256 CUs)
     (333, 8320, 512), (200, 16384, 256), (2048, 4224, 384), (256, 32768, 128), (1000, 9216, 640),
     (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536), (32, 128, 7168), (48, 16384, 2048), (64, 2048, 7168),
+    # at most 16 rows: one workgroup per 16 weight rows over the whole of K (ragged K-block runs, M < 16, one K block)
+    (16, 4096, 7168), (1, 4096, 7168), (5, 3072, 2048), (16, 7168, 2560), (13, 18432, 128), (16, 3200, 6528),
 ]
 
 
