@@ -1,20 +1,22 @@
 // Block-scaled FP8 GEMM for at most 16 activation rows (single-token decode batches) on gfx950.
 //
 // The problem is one pass over the weights (M = 16, N = 4096, K = 7168: 29 MB against 0.1 MB of activations),
-// so the kernel is cut for the memory system rather than for the matrix cores:
+// so the kernels are cut for the memory system rather than for the matrix cores.  Common to both:
 //   * a workgroup owns 16 weight rows (16 output columns) over the whole of K, which gives N / 16 workgroups
 //     (256 for N = 4096: one per CU) without cutting K across workgroups, so there are no partial tiles to
 //     write, no second kernel and no workspace;
-//   * its 8 waves take contiguous runs of at most 7 K blocks each.  A wave requests its whole run at once,
-//     weights (non-temporal) and activations (served by L2 after the first workgroups), 28 16-byte loads per
-//     lane, so every byte the CU needs is in flight within the first few hundred cycles;
-//   * the loads land in MFMA operand layout directly: lane (row r = lane % 16, part c = lane / 16) reads bytes
-//     [16 c, 16 c + 16) and [64 + 16 c, 64 + 16 c + 16) of its row's 128-byte K block.  That is a permutation
-//     of K inside the block compared with the canonical layout, the same one for both operands, and a dot
-//     product does not care;
+//   * its 8 waves take contiguous runs of at most 7 K blocks each;
 //   * v_mfma_f32_16x16x128_f8f6f4 with a zero C per scale block, folded into the accumulators with As * Bs;
 //     the 8 partial sums of a workgroup are added through LDS in wave order (deterministic).
+// gemm_thin_ring moves the operands with LDS-direct loads: a request covers 8 rows x 128 contiguous bytes
+// (8 cache lines per instruction, the cheapest shape for the address path) and lands in a wave-private ring of
+// K-block slots in LDS, from where two 16-byte reads per operand give the MFMA layout.  No barrier is involved,
+// a wave waits on its own request counter only, and a slot is requested again as soon as it has been read.
+// gemm_thin loads straight into MFMA operand layout instead (lane = one row, so 16 cache lines per
+// instruction): fewer steps, but its requests cost the address path about twice as much; it is kept for
+// comparison behind LP_GEMM_THIN_DIRECT.
 #include "gemm_common.h"
+#include <utility>
 
 using namespace lowp;
 
@@ -113,6 +115,329 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin(const uint8_t *__re
     }
 }
 
+#define LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
+#define GLB_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
+
+__device__ __forceinline__ u32x4 lds_read16(uint32_t addr)
+{
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_requests()          // at most N of the wave's global requests still in flight
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <class F, int... J>
+__device__ __forceinline__ void unrolled(F &&f, std::integer_sequence<int, J...>)
+{
+    (f(std::integral_constant<int, J>{}), ...);
+}
+
+// SLOTS K blocks of (16 weight rows + 16 activation rows) x 128 bytes per wave: 4 KB a slot.
+template <int SDT, int PER, int SLOTS>
+__global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                                  const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                                  int M, int64_t N, int64_t K, void *__restrict__ C,
+                                                                  int out_dtype)
+{
+    constexpr int S0 = SLOTS < PER ? SLOTS : PER;        // blocks requested before the first one is used
+    __shared__ __attribute__((aligned(1024))) uint8_t ring[kThinWaves * SLOTS * 4096];
+    __shared__ f32x4v red[kThinWaves][64];
+    __shared__ float sSa[2 * 64 * kThinWaves];           // activation scales, [row][K block] as in memory (896 used at most)
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int kblocks = (int)(K / 128);
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int kb0 = wave * PER;
+    const int m = l16 < M ? l16 : M - 1;
+
+    // The activation-scale table [16, kblocks] goes through LDS (consecutive lanes on consecutive addresses
+    // instead of 16-row gathers by every wave).  Its two requests per lane and everything that touches LDS before
+    // the rings are drained are written as asm with hand-placed waits: the compiler waits for every LDS-direct
+    // request in flight before anything of its own that depends on the request counter.
+    uint32_t sv[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int i = t + 64 * kThinWaves * q;
+        const int last = M * kblocks - 1;
+        const int idx = i < last ? i : last;
+        if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
+        else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
+    }
+    // request plan: lane = (row lane / 8 of the 8 rows of one request, 16-byte position lane % 8); the position
+    // holds chunk position ^ row, so that the operand reads below (16 rows, one chunk each) spread over the banks
+    const int ld_row = lane >> 3, chunk = (lane & 7) ^ ld_row;
+    const uint8_t *bsrc = Bq + (n0 + ld_row) * K + chunk * 16;
+    const int ma0 = ld_row < M ? ld_row : M - 1, ma1 = ld_row + 8 < M ? ld_row + 8 : M - 1;
+    const uint8_t *asrc0 = Aq + (int64_t)ma0 * K + chunk * 16, *asrc1 = Aq + (int64_t)ma1 * K + chunk * 16;
+    uint8_t *wring = ring + wave * (SLOTS * 4096);
+    auto request = [&](int j) {                          // block j of the run into slot j % SLOTS: 4 requests
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        uint8_t *dst = wring + (j % SLOTS) * 4096;
+        const int64_t off = (int64_t)kb * 128;
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + off), LDS_PTR(dst), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + off), LDS_PTR(dst + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(asrc0 + off), LDS_PTR(dst + 2048), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(asrc1 + off), LDS_PTR(dst + 3072), 16, 0, 0);
+    };
+#pragma unroll
+    for (int j = 0; j < S0; ++j) request(j);
+
+    float sb[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * kblocks + kb);
+    }
+    const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(sv[0]), "+v"(sv[1]) : "n"(4 * S0) : "memory");          // the two oldest requests
+    if (SDT != LP_F32) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) sv[q] = sv[q] == 0u ? 0x00400000u : (sv[q] == 0xFFu ? 0x7FC00000u : sv[q] << 23);   // e8m0 -> fp32 bits
+    }
+    asm volatile("ds_write_b32 %0, %1\n\tds_write_b32 %0, %2 offset:2048\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier"
+                 :: "v"(ssa0 + 4 * t), "v"(sv[0]), "v"(sv[1]) : "memory");
+    float sa[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        asm volatile("ds_read_b32 %0, %1" : "=v"(sa[j]) : "v"(ssa0 + 4 * (m * kblocks + kb)));
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sa[j])::"memory");
+        sa[j] = kb0 + j < kblocks ? sa[j] * sb[j] : 0.0f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // operand reads: lane (row lane % 16, part lane / 16) takes chunks 2 part and 2 part + 1 of its row
+    const uint32_t ring0 = (uint32_t)(uintptr_t)LDS_PTR(wring);
+    const uint32_t rd0 = ring0 + l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rd1 = ring0 + l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
+    f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto step = [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        // requests made so far: blocks 0 .. min(PER, S0 + j) - 1; block j has landed when at most the
+        // 4 * (that - (j + 1)) younger ones are still in flight
+        constexpr int issued = (S0 + j < PER ? S0 + j : PER);
+        wait_requests<4 * (issued - (j + 1))>();
+        const uint32_t so = (j % SLOTS) * 4096;
+        u32x4 w0 = lds_read16(rd0 + so), w1 = lds_read16(rd1 + so), x0 = lds_read16(rd0 + so + 2048), x1 = lds_read16(rd1 + so + 2048);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w0), "+v"(w1), "+v"(x0), "+v"(x1)::"memory");
+        if constexpr (j + SLOTS < PER) request(j + SLOTS);        // the slot has been read: ask for its next block
+        const i32x8 wf = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+        const i32x8 af = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        const f32x4v p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, zero, 0, 0, 0, 0, 0, 0);
+        acc.x = __builtin_fmaf(p.x, sa[j], acc.x);
+        acc.y = __builtin_fmaf(p.y, sa[j], acc.y);
+        acc.z = __builtin_fmaf(p.z, sa[j], acc.z);
+        acc.w = __builtin_fmaf(p.w, sa[j], acc.w);
+    };
+    unrolled(step, std::make_integer_sequence<int, PER>{});
+
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave != 0 || l16 >= M) return;
+    f32x4v sum = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < kThinWaves; ++w) {
+        const f32x4v v = red[w][lane];
+        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    const int64_t n = n0 + 4 * lq;
+    if (out_dtype == LP_BF16) {
+        const u32x2 o = {pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+        *(u32x2 *)((uint16_t *)C + (int64_t)l16 * N + n) = o;
+    } else {
+        *(f32x4v *)((float *)C + (int64_t)l16 * N + n) = sum;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// 17 to 64 activation rows: the same cut (16 weight rows x all of K per workgroup), but the activations of a K
+// block are now 2 to 4 row groups of 16, up to 8 KB against 2 KB of weights, and would fill a common ring with
+// bytes that come from L2.  So the two operands get rings of their own: weights 4 K blocks deep (what HBM
+// latency asks for), activations two units of 32 rows (L2 latency), a K block being one or two units.
+// Plan of the requests of one wave, in issue order, so that every wait can name how many younger requests may
+// still be in flight: weight blocks 0 .. BS-1 (2 requests each), activation units 0 and 1 (4 each); then at
+// step u, after the reads, unit u + 2 and, on the first unit of a block j, weight block j + BS.
+template <int PER, int U, int BS>
+struct RingPlan {
+    int a_end[PER * U];          // requests issued up to and including activation unit u
+    int b_end[PER];              // ... weight block j
+    int before[PER * U];         // requests issued before the wait of step u
+    constexpr RingPlan() : a_end{}, b_end{}, before{}
+    {
+        int n = 0;
+        for (int j = 0; j < (BS < PER ? BS : PER); ++j) { n += 2; b_end[j] = n; }
+        for (int u = 0; u < (2 < PER * U ? 2 : PER * U); ++u) { n += 4; a_end[u] = n; }
+        for (int u = 0; u < PER * U; ++u) {
+            before[u] = n;
+            if (u + 2 < PER * U) { n += 4; a_end[u + 2] = n; }
+            if (u % U == 0 && u / U + BS < PER) { n += 2; b_end[u / U + BS] = n; }
+        }
+    }
+};
+
+template <int SDT, int PER, int MB>
+__global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                                   int M, int64_t N, int64_t K, void *__restrict__ C,
+                                                                   int out_dtype)
+{
+    constexpr int U = (MB + 1) / 2, BS = 4, UNITS = PER * U;
+    constexpr int B0 = BS < PER ? BS : PER, A0 = 2 < UNITS ? 2 : UNITS;
+    constexpr int SV = (16 * MB * kThinWaves * kThinRun + 64 * kThinWaves - 1) / (64 * kThinWaves);      // table entries per lane
+    constexpr RingPlan<PER, U, BS> plan{};
+    __shared__ __attribute__((aligned(1024))) uint8_t bring[kThinWaves * BS * 2048];
+    __shared__ __attribute__((aligned(1024))) uint8_t aring[kThinWaves * 2 * 4096];      // later: the waves' partial sums
+    __shared__ float sSa[SV * 64 * kThinWaves];          // activation scales, [row][K block] as in memory
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int kblocks = (int)(K / 128);
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int kb0 = wave * PER;
+
+    // scale table through LDS, requests and LDS accesses as asm with hand-placed waits (see gemm_thin_ring)
+    uint32_t sv[SV];
+#pragma unroll
+    for (int q = 0; q < SV; ++q) {
+        const int i = t + 64 * kThinWaves * q;
+        const int last = M * kblocks - 1;
+        const int idx = i < last ? i : last;
+        if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
+        else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
+    }
+
+    const int ld_row = lane >> 3, chunk = (lane & 7) ^ ld_row;
+    const uint8_t *bsrc = Bq + (n0 + ld_row) * K + chunk * 16;
+    uint8_t *wb = bring + wave * (BS * 2048), *wa = aring + wave * (2 * 4096);
+    auto request_b = [&](int j) {
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        uint8_t *dst = wb + (j % BS) * 2048;
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + (int64_t)kb * 128), LDS_PTR(dst), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + (int64_t)kb * 128), LDS_PTR(dst + 1024), 16, 0, 0);
+    };
+    auto request_a = [&](int u) {                        // unit u: rows 32 (u % U) .. + 31 of block u / U
+        const int j = u / U, v = u % U;
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        uint8_t *dst = wa + (u % 2) * 4096;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = 32 * v + 8 * i + ld_row;
+            const uint8_t *src = Aq + (int64_t)(row < M ? row : M - 1) * K + chunk * 16 + (int64_t)kb * 128;
+            __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(dst + i * 1024), 16, 0, 0);
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < B0; ++j) request_b(j);
+#pragma unroll
+    for (int u = 0; u < A0; ++u) request_a(u);
+
+    float sb[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * kblocks + kb);
+    }
+    const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * B0 + 4 * A0) : "memory");          // the table requests are the oldest
+#pragma unroll
+    for (int q = 0; q < SV; ++q) {
+        asm volatile("" : "+v"(sv[q]));
+        if (SDT != LP_F32) sv[q] = sv[q] == 0u ? 0x00400000u : (sv[q] == 0xFFu ? 0x7FC00000u : sv[q] << 23);       // e8m0 -> fp32 bits
+        asm volatile("ds_write_b32 %0, %1" ::"v"(ssa0 + 4 * (t + 64 * kThinWaves * q)), "v"(sv[q]) : "memory");
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float sa[MB][PER];
+#pragma unroll
+    for (int g = 0; g < MB; ++g) {
+        const int m = 16 * g + l16 < M ? 16 * g + l16 : M - 1;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+            asm volatile("ds_read_b32 %0, %1" : "=v"(sa[g][j]) : "v"(ssa0 + 4 * (m * kblocks + kb)));
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < MB; ++g)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sa[g][j])::"memory");
+            sa[g][j] = kb0 + j < kblocks ? sa[g][j] * sb[j] : 0.0f;
+        }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint32_t rdo0 = l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rdo1 = l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
+    const uint32_t wb0 = (uint32_t)(uintptr_t)LDS_PTR(wb), wa0 = (uint32_t)(uintptr_t)LDS_PTR(wa);
+    f32x4v acc[MB];
+#pragma unroll
+    for (int g = 0; g < MB; ++g) acc[g] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+    const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    u32x4 w0, w1;                                        // weight fragment of the current block, kept over its units
+    auto step = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, j = u / U, v = u % U;
+        constexpr int need = (v == 0 && plan.b_end[j] > plan.a_end[u]) ? plan.b_end[j] : plan.a_end[u];
+        wait_requests<plan.before[u] - need>();
+        constexpr bool two = 2 * v + 1 < MB;             // the unit holds a second row group
+        const uint32_t ao = wa0 + (u % 2) * 4096;
+        u32x4 x0 = lds_read16(ao + rdo0), x1 = lds_read16(ao + rdo1), y0 = x0, y1 = x1;
+        if constexpr (two) { y0 = lds_read16(ao + 2048 + rdo0); y1 = lds_read16(ao + 2048 + rdo1); }
+        if constexpr (v == 0) { w0 = lds_read16(wb0 + (j % BS) * 2048 + rdo0); w1 = lds_read16(wb0 + (j % BS) * 2048 + rdo1); }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x0), "+v"(x1), "+v"(y0), "+v"(y1), "+v"(w0), "+v"(w1)::"memory");
+        if constexpr (u + 2 < UNITS) request_a(u + 2);
+        if constexpr (v == 0 && j + BS < PER) request_b(j + BS);
+        const i32x8 wf = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+        {
+            constexpr int g = 2 * v;
+            const i32x8 af = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+            const f32x4v p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, zero, 0, 0, 0, 0, 0, 0);
+            acc[g].x = __builtin_fmaf(p.x, sa[g][j], acc[g].x);
+            acc[g].y = __builtin_fmaf(p.y, sa[g][j], acc[g].y);
+            acc[g].z = __builtin_fmaf(p.z, sa[g][j], acc[g].z);
+            acc[g].w = __builtin_fmaf(p.w, sa[g][j], acc[g].w);
+        }
+        if constexpr (two) {
+            constexpr int g = 2 * v + 1;
+            const i32x8 af = {(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+            const f32x4v p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, af, zero, 0, 0, 0, 0, 0, 0);
+            acc[g].x = __builtin_fmaf(p.x, sa[g][j], acc[g].x);
+            acc[g].y = __builtin_fmaf(p.y, sa[g][j], acc[g].y);
+            acc[g].z = __builtin_fmaf(p.z, sa[g][j], acc[g].z);
+            acc[g].w = __builtin_fmaf(p.w, sa[g][j], acc[g].w);
+        }
+    };
+    unrolled(step, std::make_integer_sequence<int, UNITS>{});
+
+    // partial sums into the wave's own (drained) activation ring, then row group g is added up by wave g
+    f32x4v *red = (f32x4v *)aring;                       // [wave][8][lane]: the first 4 KB of each wave's own 8 KB
+#pragma unroll
+    for (int g = 0; g < MB; ++g) red[(wave * 8 + g) * 64 + lane] = acc[g];
+    __syncthreads();
+    if (wave >= MB) return;
+    const int row = 16 * wave + l16;
+    f32x4v sum = red[wave * 64 + lane];                  // wave 0's partial of group `wave`
+#pragma unroll
+    for (int w = 1; w < kThinWaves; ++w) {
+        const f32x4v x = red[(w * 8 + wave) * 64 + lane];
+        sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+    }
+    if (row >= M) return;
+    const int64_t n = n0 + 4 * lq;
+    if (out_dtype == LP_BF16) {
+        const u32x2 o = {pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+        *(u32x2 *)((uint16_t *)C + (int64_t)row * N + n) = o;
+    } else {
+        *(f32x4v *)((float *)C + (int64_t)row * N + n) = sum;
+    }
+}
+
 }  // namespace
 
 namespace lowp {
@@ -120,20 +445,30 @@ namespace gemm {
 
 bool thin_ok(int64_t M, int64_t N, int64_t K)
 {
-    // one run of K blocks per wave; enough workgroups to cover the chip (fewer are better served by the K-split kernels)
-    return M >= 1 && M <= 16 && N % 16 == 0 && K % 128 == 0 && K / 128 <= kThinWaves * kThinRun && N / 16 >= 192 &&
-           N / 16 <= 0x7FFFFFFF;
+    // one run of K blocks per wave, and enough workgroups to cover the chip (fewer are better served by the
+    // K-split kernels).  Above 16 rows a workgroup holds 128 KB of LDS and its activations (M / 16 times the
+    // bytes of its weights) come through the same request path, so beyond about two workgroups per CU the
+    // K-split kernel, which shares the activations between 128 weight rows, is ahead (measured at N = 18432).
+    if (M < 1 || M > 64 || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun) return false;
+    const int64_t groups = N / 16;
+    return groups >= 192 && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
 }
 
 template <int SDT, int PER>
 void launch_thin_per(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-                     int out_dtype, int per, hipStream_t st)
+                     int out_dtype, int per, int kind, hipStream_t st)
 {
     if constexpr (PER > 1) {
-        if (per < PER) return launch_thin_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, st);
+        if (per < PER) return launch_thin_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
     }
-    hipLaunchKernelGGL((gemm_thin<SDT, PER>), dim3((unsigned)(N / 16)), dim3(64 * kThinWaves), 0, st, (const uint8_t *)Aq, As,
-                       (const uint8_t *)Bq, Bs, (int)M, N, K, C, out_dtype);
+    const dim3 grid((unsigned)(N / 16)), block(64 * kThinWaves);
+    const uint8_t *a = (const uint8_t *)Aq, *b = (const uint8_t *)Bq;
+    if (M > 48) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else if (M > 32) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else if (M > 16) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else if (kind == 0) hipLaunchKernelGGL((gemm_thin<SDT, PER>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else if (kind == 4) hipLaunchKernelGGL((gemm_thin_ring<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else hipLaunchKernelGGL((gemm_thin_ring<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
 }
 
 int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
@@ -141,8 +476,14 @@ int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, 
 {
     const int kblocks = (int)(K / 128);
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
-    if (scale_dtype == LP_F32) launch_thin_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, st);
-    else launch_thin_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, st);
+    // ring depth 2 (64 KB of LDS: two workgroups share a CU and one's tail overlaps the other's start) measured
+    // as fast as depth 4 with one workgroup per CU at N = 4096 and faster beyond
+    static const char *env = getenv("LP_GEMM_THIN_DIRECT");                      // tuning aids
+    static const char *slots_env = getenv("LP_GEMM_THIN_SLOTS");
+    int kind = env ? 0 : 2;
+    if (!env && slots_env) kind = atoi(slots_env) == 4 ? 4 : 2;
+    if (scale_dtype == LP_F32) launch_thin_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
+    else launch_thin_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
     return check_launch("lp_gemm_fp8_block(thin)");
 }
 

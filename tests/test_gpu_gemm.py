@@ -73,6 +73,8 @@ DENSE_SHAPES = [
     (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536), (32, 128, 7168), (48, 16384, 2048), (64, 2048, 7168),
     # at most 16 rows: one workgroup per 16 weight rows over the whole of K (ragged K-block runs, M < 16, one K block)
     (16, 4096, 7168), (1, 4096, 7168), (5, 3072, 2048), (16, 7168, 2560), (13, 18432, 128), (16, 3200, 6528),
+    # 17 to 64 rows: the same cut with separate rings for weights and activations (2, 3, 4 row groups)
+    (17, 4096, 7168), (32, 3072, 1024), (40, 3200, 6528), (48, 4096, 896), (50, 3072, 4096), (64, 18432, 2048),
 ]
 
 
