@@ -53,6 +53,10 @@ __device__ __forceinline__ BlockScale derive_scale(float amax, float amax_floor,
         b.stored = s;
         b.fast = recip_div_safe(s);
         b.recip = 1.0f / s;
+    } else if (MODE == LP_SCALE_MUL_FLOOR) {
+        const float a = amax < amax_floor ? amax_floor : amax;
+        b.div = (1.0f / a) * kE4M3Max;
+        b.stored = a / kE4M3Max;
     } else {
         // `448 / tensor` in torch is reciprocal(tensor) * 448: two roundings
         float f = amax > 0.0f ? (1.0f / amax) * kE4M3Max : 1.0f;

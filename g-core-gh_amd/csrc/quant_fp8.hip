@@ -304,7 +304,7 @@ extern "C" int lp_quant_fp8_block(const void *x, int x_dtype, int64_t rows, int6
     LP_REQUIRE(rows % bm == 0 && cols % bn == 0,
                "lp_quant_fp8_block: shape (%lld, %lld) not divisible by block (%d, %d)", (long long)rows,
                (long long)cols, bm, bn);
-    LP_REQUIRE(scale_mode >= LP_SCALE_POW2 && scale_mode <= LP_SCALE_RCP_POW2, "lp_quant_fp8_block: bad scale_mode");
+    LP_REQUIRE(scale_mode >= LP_SCALE_POW2 && scale_mode <= LP_SCALE_MUL_FLOOR, "lp_quant_fp8_block: bad scale_mode");
     LP_REQUIRE(zero_rule >= LP_ZERO_NONE && zero_rule <= LP_ZERO_SCALE_TO_ONE, "lp_quant_fp8_block: bad zero_rule");
     LP_REQUIRE(amax_floor >= 0.0f, "lp_quant_fp8_block: amax_floor must be >= 0");
     if (rows == 0 || cols == 0) return LP_OK;
@@ -324,6 +324,9 @@ extern "C" int lp_quant_fp8_block(const void *x, int x_dtype, int64_t rows, int6
     case LP_SCALE_RCP_POW2:
         return launch_mode<LP_SCALE_RCP_POW2>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
                                               scale_dtype, nan_count, st);
+    case LP_SCALE_MUL_FLOOR:
+        return launch_mode<LP_SCALE_MUL_FLOOR>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
+                                               scale_dtype, nan_count, st);
     default:
         return launch_mode<LP_SCALE_MUL>(x, bf, rows, cols, bm, bn, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,
                                          scale_dtype, nan_count, st);

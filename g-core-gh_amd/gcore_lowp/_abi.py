@@ -16,7 +16,7 @@ LIB_PATH = os.environ.get("LOWP_LIB") or os.path.join(_HERE, "_lib", "liblowp.so
 # enum lp_dtype
 F32, BF16, E8M0, E4M3 = 0, 1, 2, 3
 # enum lp_scale_mode
-SCALE_POW2, SCALE_DIV, SCALE_MUL, SCALE_RCP, SCALE_RCP_POW2 = 0, 1, 2, 3, 4
+SCALE_POW2, SCALE_DIV, SCALE_MUL, SCALE_RCP, SCALE_RCP_POW2, SCALE_MUL_FLOOR = 0, 1, 2, 3, 4, 5
 # enum lp_zero_rule
 ZERO_NONE, ZERO_AMAX_TO_ONE, ZERO_SCALE_TO_ONE = 0, 1, 2
 # enum lp_fp4_zero

@@ -55,7 +55,12 @@ enum lp_scale_mode {
     /* as LP_SCALE_RCP with s rounded up to a power of two from its bits
      * (exponent field - 127, + 1 when a mantissa bit is set); act_quant with
      * scale_fmt set: qat.py:98-113 */
-    LP_SCALE_RCP_POW2 = 4
+    LP_SCALE_RCP_POW2 = 4,
+    /* a = max(amax, amax_floor), f = fl(fl(1/a) * 448), q = cast(clamp(x * f)), stored scale = a / 448:
+     * the published per_block_cast_to_fp8 of SGLang / DeepGEMM (x * (448.0 / amax) with amax clamped at
+     * 1e-4; scale amax / 448), which the weight-update path calls
+     * (gpatch_v4/generation_backend/sglang_model_specific/sglang_weight_update_dsv4.py:205-223,309-310) */
+    LP_SCALE_MUL_FLOOR = 5
 };
 
 enum lp_zero_rule {

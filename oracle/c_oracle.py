@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "_build", "liblowp_oracle.so")
 
 POW2, DIV, MUL = 0, 1, 2
-SCALE_RCP, SCALE_RCP_POW2 = 3, 4
+SCALE_RCP, SCALE_RCP_POW2, SCALE_MUL_FLOOR = 3, 4, 5
 ZERO_NONE, ZERO_AMAX_TO_ONE, ZERO_SCALE_TO_ONE = 0, 1, 2
 LOG2_LIBM, LOG2_EXACT = 0, 1
 

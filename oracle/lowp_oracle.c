@@ -174,7 +174,7 @@ int orc_pow2_exponent(float r, int kind)
     return (e - 127) + (m ? 1 : 0);
 }
 
-enum { ORC_SCALE_POW2 = 0, ORC_SCALE_DIV = 1, ORC_SCALE_MUL = 2, ORC_SCALE_RCP = 3, ORC_SCALE_RCP_POW2 = 4 };
+enum { ORC_SCALE_POW2 = 0, ORC_SCALE_DIV = 1, ORC_SCALE_MUL = 2, ORC_SCALE_RCP = 3, ORC_SCALE_RCP_POW2 = 4, ORC_SCALE_MUL_FLOOR = 5 };
 enum { ORC_ZERO_NONE = 0, ORC_ZERO_AMAX_TO_ONE = 1, ORC_ZERO_SCALE_TO_ONE = 2 };
 
 /*
@@ -236,6 +236,14 @@ int64_t orc_quant_fp8_block(const float *x, int64_t rows, int64_t cols, int bm, 
                 s = a / 448.0f;
                 if (zero_rule == ORC_ZERO_SCALE_TO_ONE && s == 0.0f) s = 1.0f;
                 if (zero_rule == ORC_ZERO_AMAX_TO_ONE && !(amax > 0.0f) && amax == amax) s = 1.0f;
+            } else if (mode == ORC_SCALE_MUL_FLOOR) {
+                /* per_block_cast_to_fp8 as published by SGLang / DeepGEMM (the library itself is not in the
+                 * reference tree): amax.clamp(1e-4); x * (448.0 / amax) -> e4m3; scale amax / 448.0 */
+                float a = amax;
+                if (a < amax_floor) a = amax_floor;
+                float rinv = 1.0f / a;
+                f = rinv * 448.0f;
+                s = a / 448.0f;
             } else {
                 float safe = amax > 0.0f ? amax : 1.0f;              /* NaN amax also lands on 1 */
                 /* the reference writes `448 / tensor`, which torch evaluates as
@@ -251,7 +259,7 @@ int64_t orc_quant_fp8_block(const float *x, int64_t rows, int64_t cols, int bm, 
                 for (int j = 0; j < bn; ++j) {
                     int64_t idx = (br * bm + i) * cols + bc * bn + j;
                     float v = x[idx];
-                    float y = (mode == ORC_SCALE_MUL) ? v * f : v / s;
+                    float y = (mode == ORC_SCALE_MUL || mode == ORC_SCALE_MUL_FLOOR) ? v * f : v / s;
                     if (y > 448.0f) y = 448.0f;                      /* clamp keeps NaN */
                     if (y < -448.0f) y = -448.0f;
                     q[idx] = orc_f32_to_e4m3fn(y);

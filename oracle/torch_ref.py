@@ -211,6 +211,22 @@ def quantize_fp8_blockwise(weight: torch.Tensor, block_size, *, device=None, sca
     return q, (1.0 / f).to(scale_dtype)
 
 
+def per_block_cast_to_fp8(x: torch.Tensor):
+    """SGLang / DeepGEMM per_block_cast_to_fp8 as published (the dense quantiser the weight-update path imports,
+    gpatch_v4/generation_backend/sglang_model_specific/sglang_weight_update_dsv4.py:205-223,309-310; the library
+    is not in the reference tree, so this restatement is not pinned by any fixture): 128 x 128 blocks, ragged edge
+    zero-padded, amax clamped at 1e-4, x * (448 / amax) -> e4m3fn, scale amax / 448 in fp32."""
+    assert x.dim() == 2
+    m, n = x.shape
+    mp, np_ = -(-m // 128) * 128, -(-n // 128) * 128
+    pad = torch.zeros(mp, np_, dtype=x.dtype)
+    pad[:m, :n] = x
+    v = pad.view(-1, 128, np_ // 128, 128)
+    amax = v.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    q = (v * (448.0 / amax)).to(_E4M3)
+    return q.view(mp, np_)[:m, :n].contiguous(), (amax / 448.0).view(v.size(0), v.size(2))
+
+
 # ---------------------------------------------------------------- a3 / a4
 
 def quant_block_fp32_scale(x: torch.Tensor, block_size, *, amax_floor=1e-12, zero_scale_to_one=False):

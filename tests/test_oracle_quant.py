@@ -172,3 +172,19 @@ def test_gemm_reference_indexing(corc):
     # swapping the scale axes must be visible
     wrong = T.gemm_fp8_block_scaling_ref(aq, a_s.flip(1), bq, b_s).numpy()
     assert not np.allclose(c, wrong, rtol=1e-3, atol=1e-2)
+
+
+def test_c_oracle_mul_floor_equals_published_per_block_cast(corc):
+    """The multiply form with a floored amax and a stored scale amax / 448 (the per_block_cast_to_fp8 that the
+    weight-update path imports from SGLang): C restatement against the torch restatement, including a tile
+    under the 1e-4 clamp and a zero tile.  Neither is pinned by a fixture: the library is not in the reference tree."""
+    for x in (I.weight_like(256, 384, 1), I.act_like(256, 384, 2), I.weight_like(256, 256, 3, dtype=torch.float32)):
+        x = x.float()
+        x[:128, :128] = 0
+        x[128:, :128] *= 1e-5
+        q, s, _, nan = corc.quant_fp8_block(x.numpy(), 128, 128, corc.SCALE_MUL_FLOOR, amax_floor=1e-4)
+        tq, ts = T.per_block_cast_to_fp8(x)
+        assert nan == 0
+        assert np.array_equal(q, _u8(tq))
+        assert np.array_equal(s.view(np.uint32), _bits(ts).view(np.uint32))
+        assert s[0, 0] == np.float32(1e-4) / np.float32(448.0)
