@@ -37,6 +37,7 @@ struct alignas(16) Smem {
     uint8_t a[2][TILE_BYTES];
     uint8_t b[2][TILE_BYTES];
     float as[2][TM];
+    float bs[2][TN];     // per-row weight scales (row-scaled variant only)
 };
 
 struct TileArgs {
@@ -56,7 +57,8 @@ struct TileArgs {
 // accumulators of one wave: acc[mb][nb] is a 32(n) x 32(m) block
 struct Acc { f32x16 v[2][2]; };
 
-template <int SDT>
+// BROW: the second operand carries one scale per row and K block ([N, K/128]) instead of one per 128 x 128 block
+template <int SDT, bool BROW = false>
 __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc)
 {
     const int t = threadIdx.x;
@@ -87,6 +89,8 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
         if (t < TM) {
             const int64_t m = ta.m0 + t;
             gas = m < ta.m_end ? scale_at<SDT>(ta.As, m * ta.kblocks + kb) : 0.0f;
+        } else if (BROW) {
+            gas = scale_at<SDT>(ta.Bs, (ta.n0 + t - TM) * ta.kblocks + kb);
         }
     };
     auto sstore = [&](int buf) {
@@ -98,6 +102,7 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
             *(u32x4 *)(sm.b[buf] + row * LDS_ROW + col) = gb[i];
         }
         if (t < TM) sm.as[buf][t] = gas;
+        else if (BROW) sm.bs[buf][t - TM] = gas;
     };
 
     gload(ta.kb_begin);
@@ -109,7 +114,7 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
         const bool more = kb + 1 < ta.kb_end;
         if (more) gload(kb + 1);
 
-        const float bscale = scale_at<SDT>(ta.Bs, (ta.n0 >> 7) * ta.kblocks + kb);
+        const float bscale = BROW ? 1.0f : scale_at<SDT>(ta.Bs, (ta.n0 >> 7) * ta.kblocks + kb);
 
         // operand fragments: lane reads 32 bytes of its row per 64-wide K half
         i32x8 wf[2][2], af[2][2];
@@ -140,11 +145,18 @@ __device__ __forceinline__ void gemm_tile(const TileArgs &ta, Smem &sm, Acc &acc
                 const int pm = (blk - 1) >> 1, pn = (blk - 1) & 1;
                 const float sc = pm ? sc1 : sc0;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc.v[pm][pn][r] = __builtin_fmaf(p[blk - 1][r], sc, acc.v[pm][pn][r]);
+                for (int r = 0; r < 16; ++r) {
+                    // element r of a 32 x 32 block sits in weight row 8 (r / 4) + 4 (lane / 32) + r % 4
+                    const float sr = BROW ? sc * sm.bs[buf][wn * 64 + pn * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3)] : sc;
+                    acc.v[pm][pn][r] = __builtin_fmaf(p[blk - 1][r], sr, acc.v[pm][pn][r]);
+                }
             }
         }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc.v[1][1][r] = __builtin_fmaf(p[3][r], sc1, acc.v[1][1][r]);
+        for (int r = 0; r < 16; ++r) {
+            const float sr = BROW ? sc1 * sm.bs[buf][wn * 64 + 32 + 8 * (r >> 2) + 4 * lhi + (r & 3)] : sc1;
+            acc.v[1][1][r] = __builtin_fmaf(p[3][r], sr, acc.v[1][1][r]);
+        }
         if (more) sstore(buf ^ 1);
         __syncthreads();
     }
@@ -186,7 +198,7 @@ __device__ __forceinline__ void store_tile(const Acc &acc, int64_t m0, int64_t m
     });
 }
 
-template <int SDT>
+template <int SDT, bool BROW = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_dense(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                   int scale_dtype, int64_t M, int64_t N, int64_t K, int64_t tiles_m,
@@ -200,7 +212,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     ta.K = K; ta.kblocks = K / TK; ta.m0 = tm * TM; ta.m_end = M; ta.n0 = tn * TN;
     ta.kb_begin = 0; ta.kb_end = (int)(K / TK);
     Acc acc;
-    gemm_tile<SDT>(ta, sm, acc);
+    gemm_tile<SDT, BROW>(ta, sm, acc);
     store_tile(acc, ta.m0, M, ta.n0, ldc, C, out_dtype);
 }
 
@@ -395,6 +407,24 @@ static int launch_small(const void *Aq, const void *As, const void *Bq, const vo
         hipLaunchKernelGGL(gemm_dense<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
                            (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
     return check_launch("lp_gemm_fp8_block");
+}
+
+extern "C" int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M,
+                                    int64_t N, int64_t K, void *C, int out_dtype, lp_stream_t stream)
+{
+    int rc = check_gemm_args("lp_gemm_fp8_rowscale", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
+    const int64_t grid = padded_grid(tiles_m, tiles_n);
+    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_rowscale: problem too large");
+    hipStream_t st = (hipStream_t)stream;
+    if (scale_dtype == LP_F32)
+        hipLaunchKernelGGL((gemm_dense<LP_F32, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+    else
+        hipLaunchKernelGGL((gemm_dense<LP_E8M0, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+    return check_launch("lp_gemm_fp8_rowscale");
 }
 
 extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,

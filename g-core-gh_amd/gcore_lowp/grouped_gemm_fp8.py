@@ -2,7 +2,7 @@
 
 * m_grouped_gemm_fp8_fp8_bf16_nt_contiguous -- the DeepGEMM-style call the
   reference makes at tests/test_gpatch_v4/test_deep_gemm_grouped_gemm_fp8.py:106-109.
-* MyTeGroupedLinearFp8 -- forward of gpatch_v4/models/deepseek_v4/fp8.py:346-394:
+* MyTeGroupedLinearFp8 -- gpatch_v4/models/deepseek_v4/fp8.py:180-394, forward and backward:
   activations are quantised per 1 x 128, weights per 128 x 128 (or taken
   pre-quantised), one grouped GEMM; no per-expert row padding copies.
 """
@@ -13,7 +13,8 @@ import torch
 from . import _abi as A
 from . import ops
 
-__all__ = ["grouped_gemm_fp8", "m_grouped_gemm_fp8_fp8_bf16_nt_contiguous", "MyTeGroupedLinearFp8"]
+__all__ = ["grouped_gemm_fp8", "m_grouped_gemm_fp8_fp8_bf16_nt_contiguous", "MyTeGroupedLinearFp8", "quant_fp8_colwise_t",
+           "gemm_fp8_rowscale"]
 
 
 def _scale_arg(s, dev):
@@ -62,10 +63,101 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs, rhs, out: torch.Tensor, m_ind
     grouped_gemm_fp8(xq, xs, wq, ws, offs, out=out)
 
 
+def quant_fp8_colwise_t(x: torch.Tensor, m_offsets: torch.Tensor, m_splits):
+    """Column-wise quantisation of expert-grouped rows with transposed output (the operands of the weight-gradient
+    GEMM): x [M, C] bf16/fp32 on the GPU -> (codes uint8 [C * P], e8m0 scales [C * P / 128], blocks per expert),
+    expert e's [C, P_e] / [C, P_e / 128] matrices stored one after the other, P_e = ceil(M_e / 128) * 128."""
+    assert x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
+    rows, cols = x.shape
+    nblk = [(int(m) + 127) // 128 for m in m_splits]
+    total = sum(nblk)
+    q = torch.empty(cols * total * 128, dtype=torch.uint8, device=x.device)
+    s = torch.empty(cols * total, dtype=ops.E8M0, device=x.device)
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        A.check(A.lib().lp_quant_fp8_colwise_t(x.data_ptr(), A.BF16 if x.dtype == torch.bfloat16 else A.F32, rows, cols,
+                                               m_offsets.data_ptr(), len(nblk), total, q.data_ptr(), s.data_ptr(), A.E8M0,
+                                               A.stream_ptr()))
+    return q, s, nblk
+
+
+def gemm_fp8_rowscale(aq, a_s, bq, b_s, M, N, K, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = sum over K blocks of (aq . bq^T) * a_s[m, kb] * b_s[n, kb]: e8m0 scales per row and 128 of K on
+    both operands; aq / bq are flat uint8 views of [M, K] / [N, K]."""
+    assert out.is_contiguous() and tuple(out.shape) == (M, N) and out.dtype in (torch.bfloat16, torch.float32)
+    with torch.cuda.device(out.device):
+        A.check(A.lib().lp_gemm_fp8_rowscale(aq.data_ptr(), a_s.data_ptr(), bq.data_ptr(), b_s.data_ptr(), A.E8M0, M, N, K,
+                                             out.data_ptr(), A.BF16 if out.dtype == torch.bfloat16 else A.F32, A.stream_ptr()))
+    return out
+
+
+def _offsets(m_splits, dev):
+    offs = torch.zeros(len(m_splits) + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits, dtype=torch.int64), 0).to(torch.int32)
+    return offs.to(dev)
+
+
+class _GroupedGemmFp8(torch.autograd.Function):
+    """gpatch_v4/models/deepseek_v4/fp8.py:180-343 without TransformerEngine, Float8BlockScaling with power-of-two
+    scales: forward y_e = x_e W_e^T on 1 x 128 activations and 128 x 128 weights; backward
+      dgrad  dx_e = dY_e W_e      (layout NN): dY quantised 1 x 128 along N, the weight's codes and scales transposed
+                                  (a 128 x 128 block scaling is its own transpose);
+      wgrad  dW_e = dY_e^T X_e    (layout NT over column-wise operands): dY and X quantised per (column, 128 rows of
+                                  the expert), transposed, one row-scaled GEMM per expert straight into dW[e].
+    The reference pads every expert to a multiple of 16 rows for TE (fp8.py:29-58); here a ragged expert needs no
+    padding in the forward and dgrad (tiles are masked), and the column-wise operands are zero-padded to 128 rows,
+    which does not change any block's amax or sum."""
+
+    @staticmethod
+    def forward(ctx, inp, weight, wq, ws, m_splits, out_dtype):
+        E, n_out, k_in = wq.shape
+        x = inp.reshape(-1, k_in)
+        from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
+        xq, xs = quant_fp8_e4m3_scale_e8m0(x, block_size=(1, 128))
+        offs = _offsets(m_splits, x.device)
+        out = grouped_gemm_fp8(xq, xs, wq, ws, offs, out_dtype=out_dtype)
+        ctx.need_wgrad = weight is not None and weight.requires_grad
+        ctx.need_dgrad = inp.requires_grad
+        saved = [wq.view(torch.uint8), ws.view(torch.uint8), offs]
+        if ctx.need_wgrad:
+            xtq, xts, _ = quant_fp8_colwise_t(x.detach(), offs, m_splits)
+            saved += [xtq, xts.view(torch.uint8)]
+        ctx.save_for_backward(*saved)
+        ctx.m_splits, ctx.inp_shape, ctx.dims, ctx.out_dtype = m_splits, inp.shape, (E, n_out, k_in), out_dtype
+        return out.view(*inp.shape[:-1], n_out)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
+        E, n_out, k_in = ctx.dims
+        wq, ws, offs = ctx.saved_tensors[:3]
+        dy = grad_output.contiguous().view(-1, n_out)
+        dgrad = wgrad = None
+        if ctx.need_dgrad:
+            dyq, dys = quant_fp8_e4m3_scale_e8m0(dy, block_size=(1, 128))
+            wt = wq.transpose(1, 2).contiguous().view(ops.E4M3)
+            wst = ws.transpose(1, 2).contiguous().view(ops.E8M0)
+            dgrad = grouped_gemm_fp8(dyq, dys, wt, wst, offs, out_dtype=ctx.out_dtype).view(ctx.inp_shape)
+        if ctx.need_wgrad:
+            xtq, xts = ctx.saved_tensors[3:5]
+            dtq, dts, nblk = quant_fp8_colwise_t(dy, offs, ctx.m_splits)
+            wgrad = torch.empty((E, n_out, k_in), dtype=ctx.out_dtype, device=dy.device)
+            done = 0                                       # blocks of the experts before e
+            for e in range(E):
+                if nblk[e] == 0:
+                    wgrad[e].zero_()
+                    continue
+                p = nblk[e] * 128
+                gemm_fp8_rowscale(dtq[n_out * done * 128:], dts.view(torch.uint8)[n_out * done:],
+                                  xtq[k_in * done * 128:], xts[k_in * done:], n_out, k_in, p, wgrad[e])
+                done += nblk[e]
+        return dgrad, wgrad, None, None, None, None
+
+
 class MyTeGroupedLinearFp8(torch.nn.Module):
-    """Forward of fp8.py:346-394 without TransformerEngine: weight is passed in
-    ([E,N,K] bf16/fp32, or a pre-quantised (data, scale) pair / object with
-    `_data` and `_scale`), rows of `inp` are concatenated in expert order."""
+    """fp8.py:346-394 without TransformerEngine: weight is passed in ([E,N,K] bf16/fp32, or pre-quantised: a
+    (data, scale) pair or a tensor / object with `_data` and `_scale`, 128 x 128 power-of-two scales), rows of `inp`
+    are concatenated in expert order.  Differentiable in `inp` and in a tensor `weight` (fp8.py:285-343)."""
 
     def __init__(self, num_gemms: int, recipe=None):
         super().__init__()
@@ -85,17 +177,15 @@ class MyTeGroupedLinearFp8(torch.nn.Module):
         assert len(shape) == 3 and shape[0] == self.num_gemms, (tuple(shape), m_splits)
         n_out, k_in = shape[1], shape[2]
         assert inp.size(-1) == k_in, (inp.size(-1), k_in)
-        x = inp.reshape(-1, k_in)
-        assert sum(m_splits) == x.shape[0], (sum(m_splits), x.shape[0])
+        assert sum(m_splits) == inp.numel() // k_in, (sum(m_splits), inp.numel() // k_in)
         from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
-        # Float8BlockScaling recipe: power-of-two scales for activations and weights
-        xq, xs = quant_fp8_e4m3_scale_e8m0(x, block_size=(1, 128))
         if wq is None:
-            wq, ws = quant_fp8_e4m3_scale_e8m0(weight, block_size=(128, 128))
+            # Float8BlockScaling recipe: power-of-two scales for activations and weights
+            wq, ws = quant_fp8_e4m3_scale_e8m0(weight.detach(), block_size=(128, 128))
         if wq.dtype == torch.uint8:
             wq = wq.view(ops.E4M3)
-        offs = torch.zeros(self.num_gemms + 1, dtype=torch.int32)
-        offs[1:] = torch.cumsum(torch.tensor(m_splits, dtype=torch.int64), 0).to(torch.int32)
-        out = grouped_gemm_fp8(xq, xs, wq, ws, offs.to(x.device), out_dtype=inp.dtype
-                               if inp.dtype in (torch.bfloat16, torch.float32) else torch.bfloat16)
-        return out.view(*inp.shape[:-1], n_out)
+        if ws.dtype != ops.E8M0:
+            raise TypeError(f"pre-quantised weight scales must be float8_e8m0fnu (power of two), got {ws.dtype}")
+        wt = weight if isinstance(weight, torch.Tensor) else None
+        out_dtype = inp.dtype if inp.dtype in (torch.bfloat16, torch.float32) else torch.bfloat16
+        return _GroupedGemmFp8.apply(inp, wt, wq.detach(), ws.detach(), m_splits, out_dtype)

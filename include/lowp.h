@@ -250,6 +250,31 @@ int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const vo
                         void *C, int out_dtype, lp_stream_t stream);
 
 /*
+ * Block-scaled FP8 GEMM with a scale per row and 128-wide K group on BOTH operands:
+ * C[m, n] = sum_kb (Aq[m, kb] . Bq[n, kb]) * As[m, kb] * Bs[n, kb], Bs [N, K/128].
+ * Same shapes, dtypes and checks as lp_gemm_fp8_block otherwise.  This is the weight-gradient GEMM of
+ * the grouped linear (layout "NT" over column-wise quantised operands,
+ * gpatch_v4/models/deepseek_v4/fp8.py:325-341): A = dY_e^T, B = X_e^T from lp_quant_fp8_colwise_t.
+ */
+int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                         int64_t M, int64_t N, int64_t K, void *C, int out_dtype, lp_stream_t stream);
+
+/*
+ * Column-wise quantiser with transposed output for expert-grouped rows.  x: device [rows, cols]
+ * (LP_BF16 or LP_F32), rows of expert e = m_offsets[e] .. m_offsets[e+1]-1 (device int32 [E+1]),
+ * cols % 128 == 0.  Per expert, P_e = ceil(M_e / 128) * 128 and
+ *   qT block e: [cols, P_e] e4m3fn at byte offset cols * (P_0 + .. + P_{e-1}), zero codes in the pad,
+ *   sT block e: [cols, P_e / 128] scales at element offset cols * (P_0 + .. + P_{e-1}) / 128,
+ * scale = 2^ceil(log2(amax / 448)) per (column, 128 rows of the expert), 1 for an all-zero block
+ * (LP_SCALE_POW2).  padded_blocks = sum_e P_e / 128 (the caller knows the row counts: the reference
+ * passes m_splits as a host list, fp8.py:193).  Replaces the column-wise half of tex.split_quantize
+ * (fp8.py:231,292-294) for Float8BlockScaling with power-of-two scales.
+ */
+int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, int64_t cols, const int32_t *m_offsets,
+                           int E, int64_t padded_blocks, void *qT, void *sT, int scale_dtype,
+                           lp_stream_t stream);
+
+/*
  * On-device self tests of the gfx950 conversion instructions against the
  * library's software casts.  Each writes the number of mismatching inputs to
  * *mismatches (device uint64, zeroed by the call).  No reference counterpart.

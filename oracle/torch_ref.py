@@ -377,3 +377,31 @@ def grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits) -> torch.Tensor:
             out[r:r + cnt] = x[r:r + cnt] @ w[e].T
         r += cnt
     return out
+
+
+def quant_colwise_t(x: torch.Tensor, m_splits):
+    """Column-wise operands of the grouped linear's weight-gradient GEMM
+    (gpatch_v4/models/deepseek_v4/fp8.py:292-294,325-341; Float8BlockScaling with power-of-two scales): per expert,
+    blocks of 128 rows x 1 column restarting at the expert's first row, scale 2^ceil(log2(amax / 448)) (1 for a
+    zero block, as quant_fp8_e4m3_scale_e8m0), output transposed and zero-padded to whole blocks.
+    Returns per expert (codes e4m3fn [C, P_e], scales e8m0 [C, P_e / 128])."""
+    out, r = [], 0
+    for m in m_splits:
+        p = (m + 127) // 128 * 128
+        xe = torch.zeros(p, x.shape[1], dtype=torch.float32)
+        xe[:m] = x[r:r + m].float()
+        r += m
+        if p == 0:
+            out.append((torch.zeros(x.shape[1], 0, dtype=_E4M3), torch.zeros(x.shape[1], 0, dtype=_E8M0)))
+            continue
+        q, s = quant_fp8_e4m3_scale_e8m0(xe.t().contiguous(), (1, 128))
+        out.append((q, s))
+    return out
+
+
+def gemm_rowscale_ref(aq, a_s, bq, b_s) -> torch.Tensor:
+    """fp32 reference of the GEMM with a scale per row and 128 of K on both operands."""
+    a = dequant_act_f32(aq, a_s.float())
+    b = dequant_act_f32(bq, b_s.float())
+    return a.double() @ b.double().T
+

@@ -239,3 +239,90 @@ def test_gemm_impl_errors_and_cpu_inputs(G):
         G.gemm_impl(a.half(), b.half(), dtype=torch.float16)
     with pytest.raises(Exception):
         G.gemm_impl(a[:, :100].contiguous(), b[:, :100].contiguous())      # K not a multiple of 64
+
+
+# ---------------------------------------------------------------------------------------------
+# backward of the grouped linear (gpatch_v4/models/deepseek_v4/fp8.py:285-343)
+def test_quant_colwise_t_matches_oracle(G):
+    say("quant_fp8_colwise_t")
+    m_splits = [300, 0, 128, 1, 77, 513]
+    x = I.act_like(sum(m_splits), 384, 21)
+    x[5, 7] = 0.0
+    offs = torch.zeros(len(m_splits) + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+    for dt in (torch.bfloat16, torch.float32):
+        xin = x.to(dt)
+        q, s, nblk = G.quant_fp8_colwise_t(xin.cuda(), offs.cuda(), m_splits)
+        want = T.quant_colwise_t(xin, m_splits)
+        assert nblk == [3, 0, 1, 1, 1, 5]
+        done = 0
+        for e, (wq, ws) in enumerate(want):
+            p = nblk[e] * 128
+            got_q = q[384 * done * 128:384 * (done * 128 + p)].view(384, p).cpu()
+            got_s = s.view(torch.uint8)[384 * done:384 * (done + nblk[e])].view(384, nblk[e]).cpu()
+            assert torch.equal(got_q, wq.view(torch.uint8)), (dt, e)
+            assert torch.equal(got_s, ws.view(torch.uint8)), (dt, e)
+            done += nblk[e]
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 128), (512, 384, 256), (300, 256, 1024), (4096, 7168, 384)],
+                         ids=lambda s: "M%d_N%d_K%d" % s)
+def test_gemm_rowscale(G, shape):
+    M, N, K = shape
+    say("gemm rowscale", shape)
+    a = I.act_like(M, K, 3)
+    b = I.act_like(N, K, 4) * 0.05
+    aq, a_s = T.quant_fp8_e4m3_scale_e8m0(a, (1, 128))
+    bq, b_s = T.quant_fp8_e4m3_scale_e8m0(b, (1, 128))
+    out = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    G.gemm_fp8_rowscale(aq.view(torch.uint8).cuda(), a_s.view(torch.uint8).cuda(), bq.view(torch.uint8).cuda(),
+                        b_s.view(torch.uint8).cuda(), M, N, K, out)
+    ref = (T.dequant_act_f32(aq.cuda(), a_s.float().cuda()) @ T.dequant_act_f32(bq.cuda(), b_s.float().cuda()).T)
+    check(out, ref, f"rowscale {shape}")
+
+
+@pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200]], ids=["even", "uneven", "empty"])
+def test_grouped_linear_backward(G, m_splits):
+    """tests/test_gfused/test_te_gemm_fp8.py:543-585: forward, input gradient and weight gradient within 5 % (norm)
+    of per-expert bf16 matmuls; TransformerEngine itself is not available, so its bit-exact comparison (:475-503)
+    has no counterpart here."""
+    E, H_IN, H_OUT = len(m_splits), 256, 512
+    say("grouped linear fwd+bwd", m_splits)
+    torch.manual_seed(11)
+    x = torch.randn(sum(m_splits), H_IN, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    w = torch.randn(E, H_OUT, H_IN, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    xr, wr = x.detach().clone().requires_grad_(True), w.detach().clone().requires_grad_(True)
+    outs, off = [], 0
+    for i, m in enumerate(m_splits):
+        outs.append(xr[off:off + m] @ wr[i].T)
+        off += m
+    ref = torch.cat(outs)
+    g = torch.randn_like(ref)
+    ref.backward(g)
+    lin = G.MyTeGroupedLinearFp8(E)
+    out = lin(x, w, m_splits)
+    out.backward(g)
+    rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()
+    assert out.shape == ref.shape and rel(out, ref) < 0.05
+    assert x.grad.shape == x.shape and rel(x.grad, xr.grad) < 0.05
+    assert w.grad.shape == w.shape and rel(w.grad, wr.grad) < 0.05
+    assert torch.isfinite(out).all() and torch.isfinite(x.grad).all() and torch.isfinite(w.grad).all()
+    for e, m in enumerate(m_splits):
+        if m == 0:
+            assert not w.grad[e].any()
+    # exact identities of the construction: dgrad = quantised dY times the dequantised weight, in fp32
+    from gcore_lowp.eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
+    wq, ws = quant_fp8_e4m3_scale_e8m0(w.detach(), block_size=(128, 128))
+    gq, gs = quant_fp8_e4m3_scale_e8m0(g, block_size=(1, 128))
+    wd = T.dequant_weight_f32(wq.view(E * H_OUT, H_IN), ws.float().view(-1, H_IN // 128)).view(E, H_OUT, H_IN)
+    gd = T.dequant_act_f32(gq, gs.float())
+    off = 0
+    for e, m in enumerate(m_splits):
+        if m:
+            check(x.grad[off:off + m], gd[off:off + m] @ wd[e], f"dgrad expert {e}")
+        off += m
+    # pre-quantised weights give the same forward and input gradient (:587-612)
+    x2 = x.detach().clone().requires_grad_(True)
+    out2 = lin(x2, (wq, ws), m_splits)
+    out2.backward(g)
+    assert torch.equal(out2, out) and torch.equal(x2.grad, x.grad)
