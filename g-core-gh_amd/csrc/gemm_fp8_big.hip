@@ -212,30 +212,47 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
-        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(kblocks / 4), [copies] "s"(copies)
+        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies)
 
-template <int TM, int TN, int KSUB>
+template <int TM, int TN, int KSUB, int NST = 2>
 struct AsmTile {
     static constexpr int WAVES = TM / 64 * 2, NBW = TN / 32;
     static constexpr int A_BYTES = TM * KB, B_BYTES = TN * KB;                   // one K block of 128
-    static constexpr int B_LDS = 2 * KSUB * A_BYTES, S_LDS = 2 * KSUB * (A_BYTES + B_BYTES);
-    static constexpr int LDS_BYTES = S_LDS + 2 * TM * 16;                        // two stages of KSUB K blocks + scale groups
+    static constexpr int B_LDS = NST * KSUB * A_BYTES, S_LDS = NST * KSUB * (A_BYTES + B_BYTES);
+    static constexpr int LDS_BYTES = S_LDS + 2 * TM * 16;                        // NST stages of KSUB K blocks + scale groups
 };
 
 // HWS: e8m0 scales applied by the matrix cores (v_mfma_scale_*); As / Bs then point at bytes.
-template <int TM, int TN, int KSUB, bool HWS = false>
+// DUAL: two groups of WAVES waves work on the same tile, each on one half of K with LDS stages of its own (the loop
+// itself is unchanged: both groups run the same trips and meet at the same barriers), and the second group's
+// accumulators are added through LDS at the end.  For problems with about one tile per CU, where a workgroup's
+// time is its chain of K steps rather than its arithmetic: the chain halves.
+// NST: LDS stages (2, or 4 for the 128 x 128 tile with one K block per stage: three K steps in flight).
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
 {
-    using T = AsmTile<TM, TN, KSUB>;
+    using T = AsmTile<TM, TN, KSUB, NST>;
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
+    static_assert(!DUAL || (TM == 128 && TN == 128), "the K split inside a workgroup is built for the 128 x 128 tile");
+    static_assert(NST == 2 || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "four stages: 128 x 128 tile only");
     static_assert(TM / 8 / WAVES == 4 && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3), "copies per operand and wave");
     constexpr int NBC = TN / 8 / WAVES;                 // weight copies per wave and K block
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63, wave = DUAL ? (t >> 6) & (WAVES - 1) : t >> 6;
+    const int kg = DUAL ? __builtin_amdgcn_readfirstlane(t >> 6) / WAVES : 0;                 // which half of K
     const int wm = wave >> 1, wn = wave & 1;
     const int l16 = lane & 15, lq = lane >> 4;
     const uint32_t kblocks = (uint32_t)(K / KB);
+    const uint32_t trips = (DUAL ? kblocks / 2 : kblocks) / 4;
+    constexpr int SS = HWS ? 1 : 4;                      // bytes per scale
+    if (DUAL) {
+        smem += kg * T::LDS_BYTES;
+        Aq += (int64_t)kg * (K / 2);
+        Bq += (int64_t)kg * (K / 2);
+        As = (const float *)((const char *)As + (int64_t)kg * (kblocks / 2) * SS);
+        Bs = (const float *)((const char *)Bs + (int64_t)kg * (kblocks / 2) * SS);
+    }
     // the bases go into scalar registers: tell the compiler they are wave-uniform
     auto uniform = [](const void *p) -> uint64_t {
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)p);
@@ -261,7 +278,6 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) arow[mb] = m0 + wm * 64 + mb * 16 + l16;
     const int64_t srow = m0 + (wave % (TM / 64)) * 64 + lane;
-    constexpr int SS = HWS ? 1 : 4;                      // bytes per scale
     const uint32_t soff = (uint32_t)((srow < M ? srow : M - 1) * kblocks * SS);
     const uint32_t copies = __builtin_amdgcn_readfirstlane(wave < TM / 64 ? 1u : 0u);
     // weight scale row(s) of this wave.  With TN / 2 = 128 or 64 columns per wave they lie in one scale block;
@@ -302,6 +318,22 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
         accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+    } else if constexpr (HWS && NST == 4) {
+        f32x16v acc0, acc1, acc2, acc3;
+        asm volatile(
+#include "gemm_mid4_hw_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : LP_ASM_INPUTS
+            : LP_ASM_CLOBBERS);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+    } else if constexpr (NST == 4) {
+        f32x16v acc0, acc1, acc2, acc3;
+        asm volatile(
+#include "gemm_mid4_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : LP_ASM_INPUTS
+            : LP_ASM_CLOBBERS);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     } else if constexpr (HWS) {
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
@@ -348,6 +380,23 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     }
 
+    if constexpr (DUAL) {
+        // second half of K: accumulators to LDS (that group's own stages, drained), first half adds and stores
+        __syncthreads();
+        f32x16v *dump = (f32x16v *)(smem - kg * T::LDS_BYTES + T::LDS_BYTES);          // group 1's region, seen by both
+        if (kg == 1) {
+#pragma unroll
+            for (int nb = 0; nb < NBW; ++nb) dump[(wave * NBW + nb) * 64 + lane] = accs[nb];
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb) {
+            const f32x16v o = dump[(wave * NBW + nb) * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accs[nb][r] += o[r];
+        }
+    }
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
         if (arow[mb] >= M) continue;
@@ -368,16 +417,29 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 }
 
 
-template <int TM, int TN, int KSUB, bool HWS = false>
+template <int TM, int TN, int KSUB, bool HWS = false, int NST = 2>
 __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                    const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
                                                    int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
                                                    void *__restrict__ C, int64_t ldc, int out_dtype)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB>::LDS_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB, NST>::LDS_BYTES];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<TM, TN, KSUB, HWS>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+    tile_asm<TM, TN, KSUB, HWS, false, NST>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+}
+
+// 128 x 128 tile with the K split inside the workgroup (see tile_asm): 8 waves, two sets of LDS stages.
+template <int KSUB, bool HWS>
+__global__ __launch_bounds__(512) void gemm_asm_dual(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                     const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
+                                                     int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                     void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * AsmTile<128, 128, KSUB>::LDS_BYTES];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    tile_asm<128, 128, KSUB, HWS, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
@@ -531,6 +593,33 @@ int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *B
     const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+    // About one tile per CU or fewer: split K inside the workgroup (needs whole scale groups of 512 in each half)
+    static const char *dual_env = getenv("LP_GEMM_MID_DUAL");        // tuning aid: 0 / 1 forces it off / on
+    const bool dual = K % 1024 == 0 && (dual_env ? atoi(dual_env) != 0 : tiles_m * tiles_n <= 320);
+    static const char *deep_env = getenv("LP_GEMM_MID_STAGES");      // tuning aid: 4 forces the four-stage loop, 2 forbids it
+    const bool four = deep_env ? atoi(deep_env) == 4 : false;
+    if (four) {
+        if (scale_dtype == LP_E8M0)
+            hipLaunchKernelGGL((gemm_asm<128, 128, 1, true, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
+        else
+            hipLaunchKernelGGL((gemm_asm<128, 128, 1, false, 4>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
+        return check_launch("lp_gemm_fp8_block(asm128 four stages)");
+    }
+    if (dual) {
+        if (scale_dtype == LP_E8M0)
+            hipLaunchKernelGGL((gemm_asm_dual<1, true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
+        else
+            hipLaunchKernelGGL((gemm_asm_dual<1, false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                               (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
+                               out_dtype);
+        return check_launch("lp_gemm_fp8_block(asm128 dual)");
+    }
     if (scale_dtype == LP_E8M0) {
         hipLaunchKernelGGL((gemm_asm<128, 128, 1, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
                            (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,

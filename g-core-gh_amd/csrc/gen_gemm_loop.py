@@ -35,15 +35,19 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False):
-    """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128."""
-    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, lines
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2):
+    """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
+    stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
+    for problems of about one tile per CU whose time is the chain of K steps)."""
+    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, lines
     HW = hw
+    NSTAGE = nstage
+    assert nstage == 2 or (nstage == 4 and ksub == 1)
     assert tm == 64 * waves_m
     WAVES = waves_m * waves_n
     KSUB = ksub
     A_BYTES, B_BYTES = tm * 128, tn * 128
-    SCL_LDS = 2 * ksub * (A_BYTES + B_BYTES)               # activation-scale buffer: 2 halves x tm rows x 16 bytes
+    SCL_LDS = nstage * ksub * (A_BYTES + B_BYTES)          # activation-scale buffer: 2 halves x tm rows x 16 bytes
     SCL_HALF = tm * 16        # (the e8m0 variant uses 4 of every 16 bytes: one wave writes 64 rows x 4 bytes per KB)
     NB = tn // waves_n // 16
     # a wave whose columns are not a multiple of 128 wide can straddle two weight-scale blocks: two scale rows
@@ -59,7 +63,7 @@ def a_lds(stage, sub):
 
 
 def b_lds(stage, sub):
-    """Same for the weight rows, relative to the first weight block (at 2 * KSUB * A_BYTES)."""
+    """Same for the weight rows, relative to the first weight block (at NSTAGE * KSUB * A_BYTES)."""
     return (stage * KSUB + sub) * B_BYTES
 
 
@@ -79,7 +83,7 @@ def vr(base, n):
 
 def dma(stage):
     """Issue the global->LDS copies of one stage; the operand bases advance by one K block after each."""
-    bbase = 2 * KSUB * A_BYTES
+    bbase = NSTAGE * KSUB * A_BYTES
     for sub in range(KSUB):
         for i in range(A_BYTES // 1024 // WAVES):
             emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
@@ -168,9 +172,9 @@ def step(c):
     previous step's last block).  After the last K block of a stage comes the stage flip (wait for the copies
     of the next stage, barrier, issue the copies that overwrite the stage just finished); it and the first
     fragment reads of the next step happen inside the last block, so the matrix pipe keeps working across it."""
-    stage, sub = (c // KSUB) & 1, c % KSUB
+    stage, sub = (c // KSUB) % NSTAGE, c % KSUB
     flip = sub == KSUB - 1
-    nstage, nsub = (stage ^ 1, 0) if flip else (stage, sub + 1)
+    nstage, nsub = ((stage + 1) % NSTAGE, 0) if flip else (stage, sub + 1)
     aoff, boff = a_lds(stage, sub), b_lds(stage, sub)
     naoff, nboff = a_lds(nstage, nsub), b_lds(nstage, nsub)
     if HW:
@@ -217,7 +221,24 @@ def step(c):
         if nb + 1 == NB:
             if flip:
                 # every wave has read all of this stage and its share of the next stage has landed
-                emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+                if NSTAGE == 2:
+                    emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+                else:
+                    # four stages: the copies of the two steps after the next one may stay in flight (the group's
+                    # scale copy, one more request of some waves, is then counted with them: it makes the wait a
+                    # request stricter and has itself landed by the flip of step 2, before step 3 reads the group).
+                    # On the last trip nothing new is requested, so fewer are left behind each step.
+                    per = (A_BYTES + B_BYTES) // 1024 // WAVES
+                    steady, last = 2 * per, max(0, (2 - c) * per)
+                    if last != steady:
+                        emit("s_cmp_eq_u32 s50, 1")
+                        emit(f"s_cbranch_scc1 Lwl{c}%=")
+                    emit(f"s_waitcnt vmcnt({steady}) lgkmcnt(0)")
+                    if last != steady:
+                        emit(f"s_branch Lwj{c}%=")
+                        emit(f"Lwl{c}%=:")
+                        emit(f"s_waitcnt vmcnt({last}) lgkmcnt(0)")
+                        emit(f"Lwj{c}%=:")
                 emit("s_barrier")
             else:
                 emit("s_waitcnt lgkmcnt(0)")
@@ -229,7 +250,7 @@ def step(c):
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
                 if mb == 0 and flip:
                     # copies for the K blocks after the next stage overwrite the stage just finished
-                    cond = c + 1 + KSUB >= 4
+                    cond = NSTAGE == 4 or c + 1 + KSUB >= 4
                     if cond:
                         emit("s_cmp_eq_u32 s50, 1")
                         emit(f"s_cbranch_scc1 Lnodma{c}%=")
@@ -263,9 +284,16 @@ def generate():
     scale_group_copy("a")
     weight_scale_load()
     dma(0)
-    emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
-    emit("s_barrier")
-    dma(1)                                   # K >= 512: there are at least four steps, which two stages hold at most
+    if NSTAGE == 2:
+        emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        emit("s_barrier")
+        dma(1)                               # K >= 512: there are at least four steps, which two stages hold at most
+    else:
+        per = (A_BYTES + B_BYTES) // 1024 // WAVES
+        for st in range(1, NSTAGE):          # K >= 512: the four stages hold exactly the first four steps
+            dma(st)
+        emit(f"s_waitcnt vmcnt({(NSTAGE - 1) * per}) lgkmcnt(0)")
+        emit("s_barrier")
     for mb in range(MB):
         emit(f"ds_read_b32 v{(SC if HW else SAN) + mb}, v{SRD} offset:{mb * (64 if HW else 256)}")
     emit("s_waitcnt lgkmcnt(0)")
@@ -302,7 +330,8 @@ def main():
     here = os.path.dirname(os.path.abspath(__file__))
     for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
-                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True)), ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True))):
+                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True)), ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
+                      ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4))):
         configure(*cfg)
         generate()
         with open(os.path.join(here, name), "w") as f:
