@@ -32,9 +32,10 @@ sys.path.insert(0, os.path.join(ROOT, "g-core-gh_amd"))
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
-# HBM bytes per launch of the dominant GEMM kernel (FETCH_SIZE + WRITE_SIZE from two counter runs of this
-# script, scaled by the same counters' reading for the calibration copy); None until measured.
-GEMM_BIG_TRAFFIC_BYTES = 253.1e6   # profiles/gemm_fp8_block_config2_hbm_traffic.txt
+# Bytes per launch of the dominant GEMM kernel between its L2s and the memory side (Infinity Cache / HBM): reads from
+# the request-size counters (32 / 64 / 128-byte TCC->EA reads, exact; the derived FETCH_SIZE prices the 128-byte
+# requests of LDS-direct and non-temporal loads at 64) plus WRITE_SIZE, from counter runs of this script.
+GEMM_BIG_TRAFFIC_BYTES = 434.4e6   # profiles/gemm_fp8_block_config2_hbm_traffic.txt
 
 
 def main():
@@ -436,7 +437,7 @@ def main():
                      "frac": big_tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_BIG_TRAFFIC_BYTES,
                      "kernel": "gemm_asm<256,256,1>: M=2048, weight rows 0..16383 of 18432, K=7168 (512 tiles)",
                      "launch_ms": big_ms, "flops_per_launch": big_flops,
-                     "whole_call": {"launches": "gemm_asm<256,256,1> + gemm_asm<128,128,2> on the last 2048 weight rows",
+                     "whole_call": {"launches": "gemm_asm<256,256,1> + gemm_asm_dual (128x128 tiles) on the last 2048 weight rows",
                                     "ms": ms, "tflops": tflops, "frac": tflops / FP8_PEAK_TFLOPS,
                                     "wall_ms_per_step": wall_ms}},
         "cpu_baseline": cpu,
