@@ -29,6 +29,20 @@
  *       bf16-grid amax (exhaustive test); for raw fp32 amax within a few ulp
  *       above a power of two the reference itself depends on the log2
  *       implementation of its device -- parity unpinned on that set.
+ *   scale modes RCP / RCP_POW2 (act_quant)  : bit-defined in the reference (qat.py:98-113); equality with the
+ *       eager-torch restatement, which the compositions the reference's tests equate it with pin
+ *       (tests/test_oracle_qat.py).  The non-power-of-two quotient x / s is an fp32 division whose flavour the
+ *       reference leaves to its kernel compiler: parity unpinned for scale_fmt=None beyond IEEE division.
+ *   scale mode MUL_FLOOR (per_block_cast_to_fp8 of SGLang / DeepGEMM, called at
+ *       sglang_weight_update_dsv4.py:205-223,309-310): the library is not in the reference tree and the repo
+ *       pins no version; restated from the published function, equality with the eager-torch restatement
+ *       only -- parity unpinned.
+ * Restated in oracle/torch_ref.py only (eager torch, no C twin): fp4_simulate (pinned by the reference's
+ * known-answer vector tests/test_gfused/test_deepseek_v4_fp4_qat.py:37-62 and its forward == export property),
+ * fp8_simulate, act_quant_inplace, fp_qat_128x128 / fp4_qat_then_to_fp8 (pinned by the eager compositions the
+ * reference's tests equate them with), quant_colwise_t (TransformerEngine's column-wise Float8BlockScaling
+ * quantiser, restated from the recipe's definition through the pinned 1 x 128 quantiser: TE is not in the tree,
+ * parity with TE unpinned).
  */
 #include <math.h>
 #include <stdint.h>
