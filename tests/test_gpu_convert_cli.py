@@ -168,3 +168,58 @@ def test_official_to_sgl_and_back(tmp_path):
             assert same(out2[k], t[k]), k
     with pytest.raises(RuntimeError):
         D.convert_checkpoint(src, str(tmp_path / "x"), "official2sgl", device="cpu")
+
+
+def test_compare_checkpoints(tmp_path, capsys):
+    """tools/dsv4_quant_and_dequant/compare_hf_ckpts.py drop-in: a converted checkpoint equals its source after each
+    side's dequantisation (the expert rebase is lossless), a planted difference and a missing key are reported."""
+    from gcore_lowp import compare_hf_ckpts as V
+    from gcore_lowp import dsv4_convert as D
+    say("compare_hf_ckpts")
+    src, mid, back = str(tmp_path / "official"), str(tmp_path / "sgl"), str(tmp_path / "official2")
+    t, shard_of = make_official(src)
+    D.convert_checkpoint(src, mid, "official2sgl")
+    D.convert_checkpoint(mid, back, "sgl2official")
+    # across the two layouts every shared tensor agrees in value; the keys differ by wo_a's scale (bf16 in the SGLang
+    # layout), which the reference's verdict counts as a problem too
+    assert V.main(["--a", src, "--b", mid, "--a-name", "official", "--b-name", "sgl"]) == 1
+    text = capsys.readouterr().out
+    assert "shared=%d" % (len(t) - 2) in text and "bad=0" in text and "expert/torch.int8" in text
+    assert "only_official=2" in text and "layers.0.ffn.experts.E.w1.weight" in text      # experts folded into one line
+    # same layout on both sides: the round trip of the converters
+    assert V.main(["--a", src, "--b", back, "--a-name", "official", "--b-name", "roundtrip"]) == 0
+    text = capsys.readouterr().out
+    assert "shared=%d" % len(t) in text and "bad=0" in text and "ALL CONSISTENT" in text
+    assert V.main(["--a", src, "--b", mid, "--dtype-only"]) == 1
+    # plant a difference in one dense weight and drop one key from the index of the copy
+    bad = str(tmp_path / "official_bad")
+    os.makedirs(bad)
+    out, where = load_dir(back)
+    k = "layers.1.attn.wq_a.weight"
+    out[k] = (-out[k].float()).to(E4M3)                           # cosine -1
+    wm = dict(where)
+    del out["embed.weight"], wm["embed.weight"]
+    for shard in sorted(set(where.values())):
+        save_file({kk: v for kk, v in out.items() if where[kk] == shard}, os.path.join(bad, shard))
+    with open(os.path.join(bad, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": wm}, f)
+    assert V.main(["--a", src, "--b", bad]) == 1
+    text = capsys.readouterr().out
+    assert "[DIFF] " + k in text and "only_A=1" in text and "[only in A] embed.weight" in text and "PROBLEMS FOUND" in text
+
+
+def test_convert_json(tmp_path):
+    """tools/convert_fp8/convert_json.py drop-in (no GPU work; kept with the other checkpoint tools)"""
+    from gcore_lowp import convert_json as J
+    src, dst = tmp_path / "in", tmp_path / "out"
+    src.mkdir()
+    dst.mkdir()
+    (src / "config.json").write_text(json.dumps({"a": 1, "quantization_config": {"x": 1}, "num_nextn_predict_layers": 1}))
+    (src / "model.safetensors.index.json").write_text(json.dumps({"metadata": {"total_size": 3}, "weight_map": {
+        "model.layers.0.w.weight": "f1", "model.layers.0.w.weight_scale_inv": "f1", "model.layers.61.w.weight": "f2"}}))
+    J.main(["--load_hf_dir", str(src), "--save_hf_dir", str(dst), "--remove_fp8", "--remove_mtp"])
+    assert json.loads((dst / "config.json").read_text()) == {"a": 1}
+    assert json.loads((dst / "model.safetensors.index.json").read_text()) == {
+        "metadata": {"total_size": 3}, "weight_map": {"model.layers.0.w.weight": "f1"}}
+    J.main(["--load_hf_dir", str(src), "--save_hf_dir", str(dst)])
+    assert len(json.loads((dst / "model.safetensors.index.json").read_text())["weight_map"]) == 3
