@@ -381,6 +381,34 @@ def main():
             torch.cuda.empty_cache()
         extras["c4_grouped_gemm"] = res4
 
+        # -------------------------------------------------------------- backward of the grouped linear (wgrad pair)
+        # column-wise quantiser with transposed output on the gate_up gradient [rows, 4096], and one expert's
+        # weight-gradient GEMM dW[4096, 7168] = dY^T[4096, P] X^T[7168, P]^T at P = 1024 rows
+        nblk4 = [(int(m) + 127) // 128 for m in m_splits.tolist()]
+        pb4 = sum(nblk4)
+        dy = randn(Mt, 4096)
+        qT = torch.empty(4096 * pb4 * 128, dtype=torch.uint8, device=dev)
+        sT = torch.empty(4096 * pb4, dtype=torch.uint8, device=dev)
+        fnq = lambda: chk(L.lp_quant_fp8_colwise_t(dy.data_ptr(), A.BF16, Mt, 4096, offs_d.data_ptr(), E4, pb4,  # noqa: E731
+                                                   qT.data_ptr(), sT.data_ptr(), A.E8M0, stream()))
+        msq, _ = time_launches([fnq], 5, 2)
+        byq = Mt * 4096 * 2 + 4096 * pb4 * 129
+        Pw = 1024
+        a_w = torch.randint(0, 120, (4096, Pw), dtype=torch.uint8, device=dev)
+        b_w = torch.randint(0, 120, (7168, Pw), dtype=torch.uint8, device=dev)
+        sa_w = torch.full((4096, Pw // 128), 120, dtype=torch.uint8, device=dev)
+        sb_w = torch.full((7168, Pw // 128), 121, dtype=torch.uint8, device=dev)
+        dw = torch.empty(4096, 7168, dtype=torch.bfloat16, device=dev)
+        fnw = lambda: chk(L.lp_gemm_fp8_rowscale(a_w.data_ptr(), sa_w.data_ptr(), b_w.data_ptr(), sb_w.data_ptr(), A.E8M0,  # noqa: E731
+                                                 4096, 7168, Pw, dw.data_ptr(), A.BF16, stream()))
+        msw, _ = time_launches([fnw], 10, 3)
+        extras["grouped_linear_backward"] = {
+            "quant_colwise_t_65536x4096": {"ms": msq, "GB/s": byq / msq / 1e6, "hbm_frac": byq / msq / 1e6 / HBM_PEAK_GBS, "bytes": byq},
+            "wgrad_gemm_rowscale_4096x7168xP1024": {"ms": msw, "tflops": 2.0 * 4096 * 7168 * Pw / msw / 1e9,
+                                                    "mfma_frac": 2.0 * 4096 * 7168 * Pw / msw / 1e9 / FP8_PEAK_TFLOPS}}
+        del dy, qT, sT, a_w, b_w, sa_w, sb_w, dw
+        torch.cuda.empty_cache()
+
     # ------------------------------------------------------------------ CPU baseline (oracle, bounded sample)
     cpu = None
     if not args.no_cpu:

@@ -7,8 +7,12 @@
 // multiple of 128.  Blocks restart at every expert; the rows that pad the last block are zero codes and take no
 // part in the block's amax.  Expert e's matrices start at cols * (P_0 + .. + P_{e-1}) in the code buffer and at
 // that over 128 in the scale buffer, so each expert's pair is a contiguous operand for lp_gemm_fp8_rowscale.
-// One workgroup = 128 rows x 128 columns: read along the rows (coalesced), turned in LDS, one thread per column
-// quantises its 128 values and writes them as one 128-byte line.
+// One workgroup (256 threads) = 128 rows x 128 columns.  A thread owns 8 consecutive rows x 8 consecutive columns
+// (16 lanes cover the 256 bytes of a row, all 8 row loads are issued before anything else); the column amax goes
+// thread -> the 4 lanes of a wave that share the columns (two shuffles) -> the 4 waves (1 KB of LDS, one barrier);
+// every thread then holds the scales of its 8 columns, quantises, and writes, per column, its 8 codes (8 consecutive
+// rows = 8 contiguous bytes of the transposed output) directly: the 16 threads that share a column fill its 128-byte
+// line between them, so no transposing pass through LDS is needed.
 #include "lowp_device.h"
 
 using namespace lowp;
@@ -16,61 +20,139 @@ using namespace lowp;
 namespace {
 
 template <bool IS_BF16>
-__global__ __launch_bounds__(128) void quant_colwise_t(const void *__restrict__ x, int64_t cols, const int32_t *__restrict__ m_offsets,
+__global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ x, int64_t cols, const int32_t *__restrict__ m_offsets,
                                                        int E, uint8_t *__restrict__ qT, void *__restrict__ sT, int scale_dtype)
 {
-    __shared__ float tile[128][128];                     // [row][column]
-    const int t = threadIdx.x;
+    __shared__ u32x4 wave_max[4][16][2];                 // [wave][column chunk][8 columns as fp32-bit maxima, 4 + 4]
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int cc = t & 15, rg = t >> 4;                  // column chunk (8 columns), row group (8 rows)
     const int64_t blk = blockIdx.x, c0 = (int64_t)blockIdx.y * 128;
-    // which expert owns padded block `blk` (every thread walks the offsets; E is a few hundred at most)
+    // which expert owns padded block `blk`: thread t counts the blocks of experts t, t + 256, ..., a prefix sum over the
+    // workgroup (wave shuffles, then the four wave totals through LDS) finds the one whose range holds blk
+    __shared__ int wave_total[4];
+    __shared__ int hit_e, hit_pb;
+    if (t == 0) hit_e = -1;
     int64_t pb = 0;
-    int e = 0, nblk = 0, r_begin = 0, r_end = 0;
-    for (; e < E; ++e) {
-        r_begin = m_offsets[e];
-        r_end = m_offsets[e + 1];
-        nblk = (r_end - r_begin + 127) >> 7;
-        if (blk < pb + nblk) break;
-        pb += nblk;
+    for (int e0 = 0; e0 < E; e0 += 256) {
+        const int ee = e0 + t;
+        const int cnt = ee < E ? (m_offsets[ee + 1] - m_offsets[ee] + 127) >> 7 : 0;
+        int incl = cnt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int y = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += y;
+        }
+        if (lane == 63) wave_total[wave] = incl;
+        __syncthreads();
+        int before = 0, chunk = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) before += wave_total[w];
+            chunk += wave_total[w];
+        }
+        const int64_t end = pb + before + incl;           // blocks up to and including this expert
+        if (cnt > 0 && blk >= end - cnt && blk < end) { hit_e = ee; hit_pb = (int)(end - cnt); }
+        pb += chunk;
+        __syncthreads();
+        if (hit_e >= 0 || blk < pb) break;                // uniform: both read after the barrier
     }
-    if (e >= E) return;
+    if (hit_e < 0) return;
+    const int e = hit_e;
+    pb = hit_pb;
+    const int r_begin = m_offsets[e], r_end = m_offsets[e + 1];
+    const int nblk = (r_end - r_begin + 127) >> 7;
     const int lb = (int)(blk - pb);                      // block inside the expert
     const int64_t r0 = (int64_t)r_begin + (int64_t)lb * 128;
     const int valid = r_end - r0 < 128 ? (int)(r_end - r0) : 128;
-    for (int i = 0; i < 128; ++i) {
-        float v = 0.0f;
-        if (i < valid) {
-            const int64_t idx = (r0 + i) * cols + c0 + t;
-            v = IS_BF16 ? u2f((uint32_t)((const uint16_t *)x)[idx] << 16) : ((const float *)x)[idx];
+
+    // ---- loads: row rg * 8 + i, columns c0 + 8 cc .. + 7; rows past the expert's end repeat its last row and
+    // are zeroed afterwards (no branch between the loads)
+    float v[8][8];
+    {
+        u32x4 raw[8][IS_BF16 ? 1 : 2];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = rg * 8 + i;
+            const int64_t r = r0 + (row < valid ? row : valid - 1);
+            if (IS_BF16) {
+                raw[i][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + r * cols + c0 + cc * 8));
+            } else {
+                const u32x4 *src = (const u32x4 *)((const float *)x + r * cols + c0 + cc * 8);
+                raw[i][0] = __builtin_nontemporal_load(src);
+                raw[i][1] = __builtin_nontemporal_load(src + 1);
+            }
         }
-        tile[i][t] = v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool live = rg * 8 + i < valid;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                uint32_t b;
+                if (IS_BF16) b = (j & 1) ? raw[i][0][j >> 1] & 0xFFFF0000u : raw[i][0][j >> 1] << 16;
+                else b = raw[i][(j >> 2) & (IS_BF16 ? 0 : 1)][j & 3];
+                v[i][j] = u2f(live ? b : 0u);
+            }
+        }
+    }
+    // ---- column maxima of |x| as integers on the sign-cleared bits (inf / NaN sort above every finite value)
+    uint32_t m[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        uint32_t a = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t b = f2u(v[i][j]) & 0x7FFFFFFFu;
+            a = b > a ? b : a;
+        }
+        // lanes l, l ^ 16, l ^ 32, l ^ 48 hold the same columns
+        uint32_t o = (uint32_t)__shfl_xor((int)a, 16, 64);
+        a = o > a ? o : a;
+        o = (uint32_t)__shfl_xor((int)a, 32, 64);
+        m[j] = o > a ? o : a;
+    }
+    if (lane < 16) {
+        wave_max[wave][cc][0] = u32x4{m[0], m[1], m[2], m[3]};
+        wave_max[wave][cc][1] = u32x4{m[4], m[5], m[6], m[7]};
     }
     __syncthreads();
-    uint32_t mbits = 0;
-    for (int i = 0; i < 128; ++i) {
-        const uint32_t a = f2u(tile[i][t]) & 0x7FFFFFFFu;
-        mbits = a > mbits ? a : mbits;
-    }
-    const bool special = mbits >= 0x7F800000u;           // inf or NaN in the block: literal arithmetic
-    const float amax = u2f(mbits > 0x7F800000u ? 0x7FC00000u : mbits);
-    const BlockScale bs = derive_scale<LP_SCALE_POW2>(amax, 0.0f, LP_ZERO_NONE);
-    const int64_t P = (int64_t)nblk * 128;
-    const int64_t base = cols * pb * 128;                // codes of the experts before this one
-    uint8_t *dst = qT + base + (c0 + t) * P + (int64_t)lb * 128;
-    store_scale(sT, scale_dtype, cols * pb + (c0 + t) * nblk + lb, bs.stored);
-#pragma unroll 4
-    for (int i = 0; i < 128; i += 16) {
-        uint32_t w[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const u32x4 a = wave_max[w][cc][0], b = wave_max[w][cc][1];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float v0 = tile[i + 4 * j][t], v1 = tile[i + 4 * j + 1][t], v2 = tile[i + 4 * j + 2][t], v3 = tile[i + 4 * j + 3][t];
-            if (special)
-                w[j] = (uint32_t)quant_slow<LP_SCALE_POW2>(v0, bs) | ((uint32_t)quant_slow<LP_SCALE_POW2>(v1, bs) << 8) |
-                       ((uint32_t)quant_slow<LP_SCALE_POW2>(v2, bs) << 16) | ((uint32_t)quant_slow<LP_SCALE_POW2>(v3, bs) << 24);
-            else
-                w[j] = cvt4(clamp448(scale_fast<LP_SCALE_POW2>(v0, bs)), clamp448(scale_fast<LP_SCALE_POW2>(v1, bs)),
-                            clamp448(scale_fast<LP_SCALE_POW2>(v2, bs)), clamp448(scale_fast<LP_SCALE_POW2>(v3, bs)));
+            m[j] = a[j] > m[j] ? a[j] : m[j];
+            m[4 + j] = b[j] > m[4 + j] ? b[j] : m[4 + j];
         }
-        *(u32x4 *)(dst + i) = u32x4{w[0], w[1], w[2], w[3]};
+    }
+    // ---- scales, codes, stores
+    const int64_t P = (int64_t)nblk * 128;
+    const int64_t base = cols * pb * 128;                // codes of the experts before this one
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const bool special = m[j] >= 0x7F800000u;        // inf or NaN in the block: literal arithmetic
+        const float amax = u2f(m[j] > 0x7F800000u ? 0x7FC00000u : m[j]);
+        const BlockScale bs = derive_scale<LP_SCALE_POW2>(amax, 0.0f, LP_ZERO_NONE);
+        const int64_t c = c0 + cc * 8 + j;
+        if (rg == 0) store_scale(sT, scale_dtype, cols * pb + c * nblk + lb, bs.stored);
+        uint32_t lo, hi;
+        if (special) {
+            lo = hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                lo |= (uint32_t)quant_slow<LP_SCALE_POW2>(v[i][j], bs) << (8 * i);
+                hi |= (uint32_t)quant_slow<LP_SCALE_POW2>(v[4 + i][j], bs) << (8 * i);
+            }
+        } else {
+            const float f = u2f((uint32_t)(127 - bs.exp2) << 23);        // 2^-e, exact: |e| <= 126 for finite amax
+            const bool tiny = bs.exp2 < -126 || bs.exp2 > 126;
+            float y[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = clamp448(tiny ? ldexpf(v[i][j], -bs.exp2) : v[i][j] * f);
+            lo = cvt4(y[0], y[1], y[2], y[3]);
+            hi = cvt4(y[4], y[5], y[6], y[7]);
+        }
+        // plain store: the 16 threads that share this 128-byte line sit in 4 waves, and L2 puts the pieces together
+        *(u32x2 *)(qT + base + c * P + (int64_t)lb * 128 + rg * 8) = u32x2{lo, hi};
     }
 }
 
@@ -89,10 +171,10 @@ extern "C" int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, 
     LP_REQUIRE(padded_blocks <= 0x7FFFFFFF && cols / 128 <= 65535, "lp_quant_fp8_colwise_t: problem too large");
     const dim3 grid((unsigned)padded_blocks, (unsigned)(cols / 128));
     if (x_dtype == LP_BF16)
-        hipLaunchKernelGGL(quant_colwise_t<true>, grid, dim3(128), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
+        hipLaunchKernelGGL(quant_colwise_t<true>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
                            scale_dtype);
     else
-        hipLaunchKernelGGL(quant_colwise_t<false>, grid, dim3(128), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
+        hipLaunchKernelGGL(quant_colwise_t<false>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
                            scale_dtype);
     return check_launch("lp_quant_fp8_colwise_t");
 }
