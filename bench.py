@@ -389,7 +389,7 @@ def main():
         dy = randn(Mt, 4096)
         qT = torch.empty(4096 * pb4 * 128, dtype=torch.uint8, device=dev)
         sT = torch.empty(4096 * pb4, dtype=torch.uint8, device=dev)
-        fnq = lambda: chk(L.lp_quant_fp8_colwise_t(dy.data_ptr(), A.BF16, Mt, 4096, offs_d.data_ptr(), E4, pb4,  # noqa: E731
+        fnq = lambda: chk(L.lp_quant_fp8_colwise_t(dy.data_ptr(), A.BF16, Mt, 4096, offs_d.data_ptr(), E4, pb4, 128,  # noqa: E731
                                                    qT.data_ptr(), sT.data_ptr(), A.E8M0, stream()))
         msq, _ = time_launches([fnq], 5, 2)
         byq = Mt * 4096 * 2 + 4096 * pb4 * 129

@@ -58,6 +58,10 @@ int choose_big_tn(int64_t M, int64_t N);
 int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                int64_t K, void *C, int64_t ldc, int out_dtype, int tn, hipStream_t st);
 
+bool rowscale_asm_ok(const void *As, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K);
+int launch_rowscale_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
+                        int out_dtype, hipStream_t st);
+
 // gemm_skinny.hip: at most 64 activation rows
 constexpr int kSkinnyBlocks = 7;          // K blocks one workgroup handles
 // at most 16 activation rows: one workgroup per 16 weight rows over all of K (gemm_thin.hip)

@@ -418,6 +418,7 @@ extern "C" int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *
     const int64_t grid = padded_grid(tiles_m, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_rowscale: problem too large");
     hipStream_t st = (hipStream_t)stream;
+    if (gemm::rowscale_asm_ok(As, Bs, scale_dtype, M, N, K)) return gemm::launch_rowscale_asm(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
     if (scale_dtype == LP_F32)
         hipLaunchKernelGGL((gemm_dense<LP_F32, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
                            (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, N, out_dtype);

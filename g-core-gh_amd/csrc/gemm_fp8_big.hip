@@ -228,7 +228,10 @@ struct AsmTile {
 // accumulators are added through LDS at the end.  For problems with about one tile per CU, where a workgroup's
 // time is its chain of K steps rather than its arithmetic: the chain halves.
 // NST: LDS stages (2, or 4 for the 128 x 128 tile with one K block per stage: three K steps in flight).
-template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2>
+// BROW: the weights carry an e8m0 scale per row and K block ([N, K/128] bytes) instead of per 128 rows; the matrix
+// instruction takes a scale per operand row anyway, so the loop only fetches them differently (hardware-scaled
+// 128 x 128 loop: waves 2 and 3 copy the weight-scale dwords of a group while waves 0 and 1 copy the activations').
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
@@ -237,6 +240,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
     static_assert(!DUAL || (TM == 128 && TN == 128), "the K split inside a workgroup is built for the 128 x 128 tile");
     static_assert(NST == 2 || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "four stages: 128 x 128 tile only");
+    static_assert(!BROW || (HWS && TM == 128 && TN == 128 && KSUB == 1 && !DUAL && NST == 2), "row-scaled weights: hardware-scaled 128 x 128 loop");
     static_assert(TM / 8 / WAVES == 4 && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3), "copies per operand and wave");
     constexpr int NBC = TN / 8 / WAVES;                 // weight copies per wave and K block
     const int t = threadIdx.x, lane = t & 63, wave = DUAL ? (t >> 6) & (WAVES - 1) : t >> 6;
@@ -259,7 +263,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)p >> 32));
         return ((uint64_t)hi << 32) | lo;
     };
-    const uint64_t a_u = uniform(Aq), b_u = uniform(Bq), s_u = uniform(As);
+    const bool copies_weights = BROW && wave >= TM / 64;                 // this wave stages weight scales, not activation scales
+    const uint64_t a_u = uniform(Aq), b_u = uniform(Bq), s_u = uniform(copies_weights ? Bs : As);
 
     // DMA source offsets (bytes from the matrix base; the host guarantees they fit 32 bits)
     const int ld_row = lane >> 3, ld_slot = lane & 7;
@@ -278,8 +283,10 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) arow[mb] = m0 + wm * 64 + mb * 16 + l16;
     const int64_t srow = m0 + (wave % (TM / 64)) * 64 + lane;
-    const uint32_t soff = (uint32_t)((srow < M ? srow : M - 1) * kblocks * SS);
-    const uint32_t copies = __builtin_amdgcn_readfirstlane(wave < TM / 64 ? 1u : 0u);
+    const int64_t wrow = n0 + (wave - TM / 64) * 64 + lane;             // weight row whose scales this lane stages (BROW)
+    const uint32_t soff = copies_weights ? (uint32_t)((wrow < N ? wrow : N - 1) * kblocks * SS)
+                                         : (uint32_t)((srow < M ? srow : M - 1) * kblocks * SS);
+    const uint32_t copies = __builtin_amdgcn_readfirstlane(BROW || wave < TM / 64 ? 1u : 0u);
     // weight scale row(s) of this wave.  With TN / 2 = 128 or 64 columns per wave they lie in one scale block;
     // 96 columns can straddle two, and each pair of 16-column blocks is told which of the two rows it uses.
     const int64_t wcol0 = n0 + wn * (TN / 2);
@@ -306,6 +313,10 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t brd1 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
     // scale staging: 16 bytes per activation row (fp32, four K steps), or 4 bytes per row in 1 KB per copying wave (e8m0)
     const uint32_t srd = HWS ? lds0 + T::S_LDS + wm * 1024 + l16 * 4 : lds0 + T::S_LDS + arow_l * 16;
+    // row-scaled weights: their dwords live behind the two activation halves, 1 KB per copying wave like those
+    const uint32_t sdst = __builtin_amdgcn_readfirstlane((uint32_t)(T::S_LDS + (copies_weights ? 2048 : 0)));
+    const uint32_t srdb = lds0 + T::S_LDS + 4096 + wn * 1024 + l16 * 4;
+    (void)sdst; (void)srdb;
 
     f32x16v accs[NBW];
     if constexpr (HWS && NBW == 8) {
@@ -318,6 +329,14 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
         accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+    } else if constexpr (BROW) {
+        f32x16v acc0, acc1, acc2, acc3;
+        asm volatile(
+#include "gemm_mid_hwrow_loop.inc"
+            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : LP_ASM_INPUTS, [sdst] "s"(sdst), [srdb] "v"(srdb)
+            : LP_ASM_CLOBBERS);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     } else if constexpr (HWS && NST == 4) {
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
@@ -440,6 +459,18 @@ __global__ __launch_bounds__(512) void gemm_asm_dual(const uint8_t *__restrict__
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
     tile_asm<128, 128, KSUB, HWS, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
+}
+
+// 128 x 128 tiles, e8m0 scales per row and K block on both operands (the weight-gradient GEMM of the grouped linear).
+__global__ __launch_bounds__(256) void gemm_asm_rowscale(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                         const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
+                                                         int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                         void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<128, 128, 1>::LDS_BYTES + 4096];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    tile_asm<128, 128, 1, true, false, 2, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
@@ -639,6 +670,25 @@ int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *B
                            (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
                            out_dtype);
     return check_launch("lp_gemm_fp8_block(asm128)");
+}
+
+// Row-scaled weights on the hardware-scaled loop: e8m0 scales, K in whole groups of four blocks, 32-bit operand offsets.
+bool rowscale_asm_ok(const void *As, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K)
+{
+    static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;
+    return !no_asm && scale_dtype == LP_E8M0 && K % 512 == 0 && (uintptr_t)As % 4 == 0 && (uintptr_t)Bs % 4 == 0 &&
+           M * K < 0xFFFFFFFFLL && N * K < 0xFFFFFFFFLL;
+}
+
+int launch_rowscale_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
+                        int out_dtype, hipStream_t st)
+{
+    const int64_t tiles_m = (M + 127) / 128, tiles_n = N / 128;
+    const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_rowscale: problem too large");
+    hipLaunchKernelGGL(gemm_asm_rowscale, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, (const float *)As,
+                       (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+    return check_launch("lp_gemm_fp8_rowscale(asm)");
 }
 
 // Grouped problems on the hand-scheduled kernel: fp32 scales, N a multiple of 256, offsets that fit 32 bits.

@@ -35,13 +35,15 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
-    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, lines
+    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, lines
     HW = hw
     NSTAGE = nstage
+    BROW = brow                 # weight scales per row and K step (e8m0, hardware-scaled loop only) instead of per 128 rows
+    assert not brow or (hw and tm == 128 and tn == 128)
     assert nstage == 2 or (nstage == 4 and ksub == 1)
     assert tm == 64 * waves_m
     WAVES = waves_m * waves_n
@@ -72,6 +74,8 @@ SCP = (44, 224, 228)        # scale products per pair of 16-column blocks when a
 WFB = (48, 56)
 RA0, RA1, RB0, RB1 = 30, 31, 32, 33
 SRD0, SRD = 34, 35
+SRDB0, SRDB = 37, 38        # row-scaled weights: LDS address of the lane's weight-scale dwords (half 0, half in use)
+WSN, WSC = 96, 100          # ... the dwords of this group / of the next one, one per 16-row block
 
 def emit(s):
     lines.append(s)
@@ -105,7 +109,10 @@ def scale_group_copy(tag):
     emit("s_cmp_eq_u32 s53, 0")
     emit(f"s_cbranch_scc1 Lnosc{tag}%=")
     emit("s_add_u32 m0, s48, s54")
-    emit(f"s_add_u32 m0, m0, {SCL_LDS}")
+    if BROW:
+        emit("s_add_u32 m0, m0, s51")                     # activation rows or weight rows: the set-up code says where
+    else:
+        emit(f"s_add_u32 m0, m0, {SCL_LDS}")
     emit("s_nop 0")
     emit("global_load_lds_dword %[soff], s[44:45]" if HW else "global_load_lds_dwordx4 %[soff], s[44:45]")
     emit(f"Lnosc{tag}%=:")
@@ -115,6 +122,8 @@ def scale_group_copy(tag):
 
 def weight_scale_load():
     """The four weight scales of the next group into s[60:63] (and those of the second scale row into s[68:71])."""
+    if BROW:
+        return                                            # they travel with the activation scales, see scale_group_copy
     if HW:
         emit("s_load_dword s60, s[46:47], 0x0")          # four e8m0 bytes = four K steps
         emit("s_add_u32 s46, s46, 4")
@@ -141,6 +150,9 @@ def read_scales(col):
         if col == 0:
             for mb in range(MB):
                 emit(f"ds_read_b32 v{SC + mb}, v{SRD} offset:{mb * 64}")
+            if BROW:
+                for nb in range(NB):
+                    emit(f"ds_read_b32 v{WSC + nb}, v{SRDB} offset:{nb * 64}")
         return
     for mb in range(MB):
         emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256 + col * 4}")
@@ -151,7 +163,8 @@ def mfma(nb, mb, c=0):
         # scales applied by the matrix core: byte c of the weight-scale register (uniform) and of the lane's
         # activation-scale register; accumulation in place
         acc = vr(ACC + 16 * nb + 4 * mb, 4)
-        emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, v36, v{SAN + mb} "
+        wscale = f"v{WSN + nb}" if BROW else "v36"
+        emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, {wscale}, v{SAN + mb} "
              f"op_sel:[{c & 1},{c & 1},0] op_sel_hi:[{c >> 1},{c >> 1},0]")
         return
     emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * (nb & 1) + 4 * mb, 4)}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, 0")
@@ -204,6 +217,8 @@ def step(c):
         # the next step belongs to the next group
         emit(f"s_xor_b32 s55, s55, {SCL_HALF}")
         emit(f"v_add_u32 v{SRD}, s55, v{SRD0}")
+        if BROW:
+            emit(f"v_add_u32 v{SRDB}, s55, v{SRDB0}")
     read_frag(WFB[1], RB0, RB1, boff + 2048)
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
     for mb in range(MB):
@@ -215,6 +230,8 @@ def step(c):
             read_frag(WFB[(nb + 1) & 1], RB0, RB1, boff + (nb + 1) * 2048)
         if nb == 1:
             pending = 4 if (not HW or c == 3) else 0                # scale reads issued after block 0
+            if BROW and c == 3:
+                pending += NB
             emit(f"s_waitcnt lgkmcnt({pending + (2 if NB > 2 else 0)})")        # those and wf2 may still be outstanding
         elif nb + 1 < NB:
             emit("s_waitcnt lgkmcnt(2)")
@@ -279,6 +296,10 @@ def generate():
     emit("s_mov_b32 s55, 0")
     for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
         emit(f"v_mov_b32 v{reg}, %[{name}]")
+    if BROW:
+        emit("s_mov_b32 s51, %[sdst]")
+        emit(f"v_mov_b32 v{SRDB0}, %[srdb]")
+        emit(f"v_mov_b32 v{SRDB}, %[srdb]")
     for r in range(16 * NB):
         emit(f"v_mov_b32 v{ACC + r}, 0")
     scale_group_copy("a")
@@ -296,6 +317,9 @@ def generate():
         emit("s_barrier")
     for mb in range(MB):
         emit(f"ds_read_b32 v{(SC if HW else SAN) + mb}, v{SRD} offset:{mb * (64 if HW else 256)}")
+    if BROW:
+        for nb in range(NB):
+            emit(f"ds_read_b32 v{WSC + nb}, v{SRDB} offset:{nb * 64}")
     emit("s_waitcnt lgkmcnt(0)")
     read_frag(WFB[0], RB0, RB1, 0)
     for mb in range(MB):
@@ -306,7 +330,11 @@ def generate():
         # scales of this group: the lane's activation-scale bytes and the weight-scale bytes (uniform)
         for mb in range(MB):
             emit(f"v_mov_b32 v{SAN + mb}, v{SC + mb}")
-        emit("v_mov_b32 v36, s60")
+        if BROW:
+            for nb in range(NB):
+                emit(f"v_mov_b32 v{WSN + nb}, v{WSC + nb}")
+        else:
+            emit("v_mov_b32 v36, s60")
     emit("s_mov_b64 s[56:57], s[60:61]")
     emit("s_mov_b64 s[58:59], s[62:63]")
     if SPLIT:
@@ -331,7 +359,8 @@ def main():
     for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
                       ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True)), ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
-                      ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4))):
+                      ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
+                      ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)
         generate()
         with open(os.path.join(here, name), "w") as f:

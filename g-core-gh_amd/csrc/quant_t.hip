@@ -4,7 +4,7 @@
 // so both operands are needed with that dimension contiguous and scaled per 128 of it.  This kernel takes a
 // row-major [rows, cols] tensor whose rows are grouped by expert (m_offsets) and writes, per expert, the
 // transposed codes [cols, P_e] with one power-of-two scale per (column, 128 rows), P_e = M_e rounded up to a
-// multiple of 128.  Blocks restart at every expert; the rows that pad the last block are zero codes and take no
+// multiple of pad_rows (128, or 512 so that the row-scaled GEMM can run its K loop in whole groups of four blocks).  Blocks restart at every expert; the rows that pad the last block are zero codes and take no
 // part in the block's amax.  Expert e's matrices start at cols * (P_0 + .. + P_{e-1}) in the code buffer and at
 // that over 128 in the scale buffer, so each expert's pair is a contiguous operand for lp_gemm_fp8_rowscale.
 // One workgroup (256 threads) = 128 rows x 128 columns.  A thread owns 8 consecutive rows x 8 consecutive columns
@@ -21,7 +21,7 @@ namespace {
 
 template <bool IS_BF16>
 __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ x, int64_t cols, const int32_t *__restrict__ m_offsets,
-                                                       int E, uint8_t *__restrict__ qT, void *__restrict__ sT, int scale_dtype)
+                                                       int E, int pad_rows, uint8_t *__restrict__ qT, void *__restrict__ sT, int scale_dtype)
 {
     __shared__ u32x4 wave_max[4][16][2];                 // [wave][column chunk][8 columns as fp32-bit maxima, 4 + 4]
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     int64_t pb = 0;
     for (int e0 = 0; e0 < E; e0 += 256) {
         const int ee = e0 + t;
-        const int cnt = ee < E ? (m_offsets[ee + 1] - m_offsets[ee] + 127) >> 7 : 0;
+        const int cnt = ee < E ? (m_offsets[ee + 1] - m_offsets[ee] + pad_rows - 1) / pad_rows * (pad_rows >> 7) : 0;
         int incl = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -60,10 +60,10 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     const int e = hit_e;
     pb = hit_pb;
     const int r_begin = m_offsets[e], r_end = m_offsets[e + 1];
-    const int nblk = (r_end - r_begin + 127) >> 7;
+    const int nblk = (r_end - r_begin + pad_rows - 1) / pad_rows * (pad_rows >> 7);
     const int lb = (int)(blk - pb);                      // block inside the expert
     const int64_t r0 = (int64_t)r_begin + (int64_t)lb * 128;
-    const int valid = r_end - r0 < 128 ? (int)(r_end - r0) : 128;
+    const int valid = r_end - r0 < 128 ? (r_end - r0 > 0 ? (int)(r_end - r0) : 0) : 128;      // 0: a block of padding only
 
     // ---- loads: row rg * 8 + i, columns c0 + 8 cc .. + 7; rows past the expert's end repeat its last row and
     // are zeroed afterwards (no branch between the loads)
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int row = rg * 8 + i;
-            const int64_t r = r0 + (row < valid ? row : valid - 1);
+            const int64_t r = valid > 0 ? r0 + (row < valid ? row : valid - 1) : r_begin;
             if (IS_BF16) {
                 raw[i][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + r * cols + c0 + cc * 8));
             } else {
@@ -159,8 +159,9 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
 }  // namespace
 
 extern "C" int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, int64_t cols, const int32_t *m_offsets, int E,
-                                      int64_t padded_blocks, void *qT, void *sT, int scale_dtype, lp_stream_t stream)
+                                      int64_t padded_blocks, int pad_rows, void *qT, void *sT, int scale_dtype, lp_stream_t stream)
 {
+    LP_REQUIRE(pad_rows == 128 || pad_rows == 256 || pad_rows == 512, "lp_quant_fp8_colwise_t: pad_rows must be 128, 256 or 512");
     LP_REQUIRE(x_dtype == LP_BF16 || x_dtype == LP_F32, "lp_quant_fp8_colwise_t: x_dtype must be LP_BF16 or LP_F32");
     LP_REQUIRE(scale_dtype == LP_F32 || scale_dtype == LP_E8M0, "lp_quant_fp8_colwise_t: scale_dtype must be LP_F32 or LP_E8M0");
     LP_REQUIRE(rows >= 0 && cols >= 0 && E >= 0 && padded_blocks >= 0, "lp_quant_fp8_colwise_t: bad shape");
@@ -171,10 +172,10 @@ extern "C" int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, 
     LP_REQUIRE(padded_blocks <= 0x7FFFFFFF && cols / 128 <= 65535, "lp_quant_fp8_colwise_t: problem too large");
     const dim3 grid((unsigned)padded_blocks, (unsigned)(cols / 128));
     if (x_dtype == LP_BF16)
-        hipLaunchKernelGGL(quant_colwise_t<true>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
+        hipLaunchKernelGGL(quant_colwise_t<true>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, pad_rows, (uint8_t *)qT, sT,
                            scale_dtype);
     else
-        hipLaunchKernelGGL(quant_colwise_t<false>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, (uint8_t *)qT, sT,
+        hipLaunchKernelGGL(quant_colwise_t<false>, grid, dim3(256), 0, (hipStream_t)stream, x, cols, m_offsets, E, pad_rows, (uint8_t *)qT, sT,
                            scale_dtype);
     return check_launch("lp_quant_fp8_colwise_t");
 }

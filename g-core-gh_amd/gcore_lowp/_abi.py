@@ -41,7 +41,7 @@ PROTOTYPES = {
     "lp_gemm_fp8_block": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p, _i64, _p]),
     "lp_gemm_nt": (_i32, [_p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_gemm_fp8_rowscale": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
-    "lp_quant_fp8_colwise_t": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _i64, _p, _p, _i32, _p]),
+    "lp_quant_fp8_colwise_t": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _i64, _i32, _p, _p, _i32, _p]),
     "lp_gemm_fp8_grouped": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "lp_selftest": (_i32, [_i32, _p, _p]),

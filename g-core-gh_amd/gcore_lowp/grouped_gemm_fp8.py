@@ -63,21 +63,32 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs, rhs, out: torch.Tensor, m_ind
     grouped_gemm_fp8(xq, xs, wq, ws, offs, out=out)
 
 
-def quant_fp8_colwise_t(x: torch.Tensor, m_offsets: torch.Tensor, m_splits):
+def choose_colwise_pad(m_splits) -> int:
+    """Rows every expert is padded to in the column-wise operands: 512 (the row-scaled GEMM then runs its
+    hand-scheduled kernel) unless that pads the rows by more than a quarter over 128."""
+    p128 = sum((int(m) + 127) // 128 for m in m_splits)
+    p512 = sum((int(m) + 511) // 512 * 4 for m in m_splits)
+    return 512 if p512 * 4 <= p128 * 5 else 128
+
+
+def quant_fp8_colwise_t(x: torch.Tensor, m_offsets: torch.Tensor, m_splits, pad_rows: int | None = None):
     """Column-wise quantisation of expert-grouped rows with transposed output (the operands of the weight-gradient
     GEMM): x [M, C] bf16/fp32 on the GPU -> (codes uint8 [C * P], e8m0 scales [C * P / 128], blocks per expert),
-    expert e's [C, P_e] / [C, P_e / 128] matrices stored one after the other, P_e = ceil(M_e / 128) * 128."""
+    expert e's [C, P_e] / [C, P_e / 128] matrices stored one after the other, P_e = M_e rounded up to pad_rows.
+    pad_rows None: choose_colwise_pad(m_splits)."""
     assert x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
     rows, cols = x.shape
-    nblk = [(int(m) + 127) // 128 for m in m_splits]
+    if pad_rows is None:
+        pad_rows = choose_colwise_pad(m_splits)
+    nblk = [(int(m) + pad_rows - 1) // pad_rows * (pad_rows // 128) for m in m_splits]
     total = sum(nblk)
     q = torch.empty(cols * total * 128, dtype=torch.uint8, device=x.device)
     s = torch.empty(cols * total, dtype=ops.E8M0, device=x.device)
     x = x.contiguous()
     with torch.cuda.device(x.device):
         A.check(A.lib().lp_quant_fp8_colwise_t(x.data_ptr(), A.BF16 if x.dtype == torch.bfloat16 else A.F32, rows, cols,
-                                               m_offsets.data_ptr(), len(nblk), total, q.data_ptr(), s.data_ptr(), A.E8M0,
-                                               A.stream_ptr()))
+                                               m_offsets.data_ptr(), len(nblk), total, pad_rows, q.data_ptr(), s.data_ptr(),
+                                               A.E8M0, A.stream_ptr()))
     return q, s, nblk
 
 
@@ -120,7 +131,8 @@ class _GroupedGemmFp8(torch.autograd.Function):
         ctx.need_dgrad = inp.requires_grad
         saved = [wq.view(torch.uint8), ws.view(torch.uint8), offs]
         if ctx.need_wgrad:
-            xtq, xts, _ = quant_fp8_colwise_t(x.detach(), offs, m_splits)
+            ctx.pad_rows = choose_colwise_pad(m_splits)
+            xtq, xts, _ = quant_fp8_colwise_t(x.detach(), offs, m_splits, ctx.pad_rows)
             saved += [xtq, xts.view(torch.uint8)]
         ctx.save_for_backward(*saved)
         ctx.m_splits, ctx.inp_shape, ctx.dims, ctx.out_dtype = m_splits, inp.shape, (E, n_out, k_in), out_dtype
@@ -140,7 +152,7 @@ class _GroupedGemmFp8(torch.autograd.Function):
             dgrad = grouped_gemm_fp8(dyq, dys, wt, wst, offs, out_dtype=ctx.out_dtype).view(ctx.inp_shape)
         if ctx.need_wgrad:
             xtq, xts = ctx.saved_tensors[3:5]
-            dtq, dts, nblk = quant_fp8_colwise_t(dy, offs, ctx.m_splits)
+            dtq, dts, nblk = quant_fp8_colwise_t(dy, offs, ctx.m_splits, ctx.pad_rows)       # padded like X^T in the forward
             wgrad = torch.empty((E, n_out, k_in), dtype=ctx.out_dtype, device=dy.device)
             done = 0                                       # blocks of the experts before e
             for e in range(E):

@@ -262,16 +262,17 @@ int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const v
 /*
  * Column-wise quantiser with transposed output for expert-grouped rows.  x: device [rows, cols]
  * (LP_BF16 or LP_F32), rows of expert e = m_offsets[e] .. m_offsets[e+1]-1 (device int32 [E+1]),
- * cols % 128 == 0.  Per expert, P_e = ceil(M_e / 128) * 128 and
+ * cols % 128 == 0.  Per expert, P_e = ceil(M_e / pad_rows) * pad_rows (pad_rows 128, 256 or 512; with 512
+ * lp_gemm_fp8_rowscale runs on its hand-scheduled kernel) and
  *   qT block e: [cols, P_e] e4m3fn at byte offset cols * (P_0 + .. + P_{e-1}), zero codes in the pad,
  *   sT block e: [cols, P_e / 128] scales at element offset cols * (P_0 + .. + P_{e-1}) / 128,
  * scale = 2^ceil(log2(amax / 448)) per (column, 128 rows of the expert), 1 for an all-zero block
- * (LP_SCALE_POW2).  padded_blocks = sum_e P_e / 128 (the caller knows the row counts: the reference
+ * (LP_SCALE_POW2; blocks of padding only get scale 1 and zero codes).  padded_blocks = sum_e P_e / 128 (the caller knows the row counts: the reference
  * passes m_splits as a host list, fp8.py:193).  Replaces the column-wise half of tex.split_quantize
  * (fp8.py:231,292-294) for Float8BlockScaling with power-of-two scales.
  */
 int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, int64_t cols, const int32_t *m_offsets,
-                           int E, int64_t padded_blocks, void *qT, void *sT, int scale_dtype,
+                           int E, int64_t padded_blocks, int pad_rows, void *qT, void *sT, int scale_dtype,
                            lp_stream_t stream);
 
 /*

@@ -252,7 +252,7 @@ def test_quant_colwise_t_matches_oracle(G):
     offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
     for dt in (torch.bfloat16, torch.float32):
         xin = x.to(dt)
-        q, s, nblk = G.quant_fp8_colwise_t(xin.cuda(), offs.cuda(), m_splits)
+        q, s, nblk = G.quant_fp8_colwise_t(xin.cuda(), offs.cuda(), m_splits, pad_rows=128)
         want = T.quant_colwise_t(xin, m_splits)
         assert nblk == [3, 0, 1, 1, 1, 5]
         done = 0
@@ -263,9 +263,23 @@ def test_quant_colwise_t_matches_oracle(G):
             assert torch.equal(got_q, wq.view(torch.uint8)), (dt, e)
             assert torch.equal(got_s, ws.view(torch.uint8)), (dt, e)
             done += nblk[e]
+    # padding to 512 rows: the same codes and scales, followed by blocks of zero codes with scale 1
+    q5, s5, nblk5 = G.quant_fp8_colwise_t(x.to(torch.bfloat16).cuda(), offs.cuda(), m_splits, pad_rows=512)
+    assert nblk5 == [4, 0, 4, 4, 4, 8]
+    want = T.quant_colwise_t(x.to(torch.bfloat16), m_splits)
+    done = 0
+    for e, (wq, ws) in enumerate(want):
+        p5, nb = nblk5[e] * 128, wq.shape[1] // 128
+        got_q = q5[384 * done * 128:384 * (done * 128 + p5)].view(384, p5).cpu()
+        got_s = s5.view(torch.uint8)[384 * done:384 * (done + nblk5[e])].view(384, nblk5[e]).cpu()
+        if p5:
+            assert torch.equal(got_q[:, :nb * 128], wq.view(torch.uint8)) and not got_q[:, nb * 128:].any()
+            assert torch.equal(got_s[:, :nb], ws.view(torch.uint8)) and bool((got_s[:, nb:] == 127).all())
+        done += nblk5[e]
 
 
-@pytest.mark.parametrize("shape", [(128, 128, 128), (512, 384, 256), (300, 256, 1024), (4096, 7168, 384)],
+@pytest.mark.parametrize("shape", [(128, 128, 128), (512, 384, 256), (300, 256, 1024), (4096, 7168, 384), (128, 128, 512),
+                                   (1000, 640, 2048), (4096, 7168, 1024), (77, 128, 1536)],
                          ids=lambda s: "M%d_N%d_K%d" % s)
 def test_gemm_rowscale(G, shape):
     M, N, K = shape
@@ -281,7 +295,8 @@ def test_gemm_rowscale(G, shape):
     check(out, ref, f"rowscale {shape}")
 
 
-@pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200]], ids=["even", "uneven", "empty"])
+@pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200], [2048, 1024, 0, 4096]],
+                         ids=["even", "uneven", "empty", "pad512"])
 def test_grouped_linear_backward(G, m_splits):
     """tests/test_gfused/test_te_gemm_fp8.py:543-585: forward, input gradient and weight gradient within 5 % (norm)
     of per-expert bf16 matmuls; TransformerEngine itself is not available, so its bit-exact comparison (:475-503)
