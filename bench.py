@@ -50,7 +50,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on ONE GPU (nothing on it communicates); use --gpus 1. "
-                 "How it would shard is described in DESIGN.md.")
+                 "Across GPUs it would split by weight columns, experts or checkpoint shards without collectives.")
 
     import torch
     if not torch.cuda.is_available():
