@@ -52,7 +52,34 @@ def test_host_side_validation(lib):
     assert rc == -1 and "multiple of 128" in lib.last_error()
     rc = L.lp_gemm_fp8_grouped(one, one, one, one, lib.F32, None, 4, 64, 128, 128, one, lib.BF16, None)
     assert rc == -1 and "m_offsets" in lib.last_error()
+    # the entry points added around the path: QAT conversions, FP4 quantiser, backward of the grouped linear
+    rc = L.lp_quant_fp8_block(one, lib.BF16, 128, 128, 128, 128, 6, 0.0, 0, one, one, lib.F32, None, None)
+    assert rc == -1 and "scale_mode" in lib.last_error()
+    rc = L.lp_quant_fp4_block(one, lib.BF16, 128, 100, 1, 32, one, one, None, None)
+    assert rc == -1
+    rc = L.lp_qdq_fp8_tile128(one, 128, 100, one, None)
+    assert rc == -1 and "128 x 128" in lib.last_error()
+    rc = L.lp_fp4_qat_to_fp8(one, 100, 128, one, one, None)
+    assert rc == -1 and "128 x 128" in lib.last_error()
+    rc = L.lp_fp4_qdq_row32(one, 100, one, None, None)
+    assert rc == -1 and "multiple of 32" in lib.last_error()
+    rc = L.lp_act_qdq_group(one, 1024, 48, 1, 0, one, None, None)
+    assert rc == -1 and "power of two" in lib.last_error()
+    rc = L.lp_act_qdq_group(one, 1000, 64, 1, 0, one, None, None)
+    assert rc == -1 and "multiple of the group size" in lib.last_error()
+    rc = L.lp_act_qdq_group(one, 1024, 64, 0, 0, one, None, None)
+    assert rc == -1 and "power-of-two scales" in lib.last_error()
+    rc = L.lp_quant_fp8_colwise_t(one, lib.BF16, 256, 100, one, 2, 2, 128, one, one, lib.E8M0, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
+    rc = L.lp_quant_fp8_colwise_t(one, lib.BF16, 256, 128, one, 2, 2, 100, one, one, lib.E8M0, None)
+    assert rc == -1 and "pad_rows" in lib.last_error()
+    rc = L.lp_gemm_fp8_rowscale(one, one, one, one, lib.E8M0, 64, 100, 128, one, lib.BF16, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
     # empty problems succeed without touching the device
+    assert L.lp_fp4_qdq_row32(None, 0, None, None, None) == 0
+    assert L.lp_act_qdq_group(None, 0, 128, 1, 0, None, None, None) == 0
+    assert L.lp_quant_fp8_colwise_t(None, lib.BF16, 0, 128, None, 0, 0, 128, None, None, lib.E8M0, None) == 0
+    assert L.lp_gemm_fp8_rowscale(None, None, None, None, lib.E8M0, 0, 128, 128, None, lib.BF16, None) == 0
     assert L.lp_quant_fp8_block(None, lib.BF16, 0, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, None, None, lib.F32, None, None) == 0
     assert L.lp_gemm_fp8_block(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None, 0, None) == 0
 
