@@ -198,6 +198,10 @@ class MyTeGroupedLinearFp8(torch.nn.Module):
             wq = wq.view(ops.E4M3)
         if ws.dtype != ops.E8M0:
             raise TypeError(f"pre-quantised weight scales must be float8_e8m0fnu (power of two), got {ws.dtype}")
+        # fp8.py:139-161: codes shaped like the logical weight, one scale per 128 x 128 block
+        assert wq.dtype == ops.E4M3, wq.dtype
+        assert n_out % 128 == 0 and k_in % 128 == 0, (n_out, k_in)
+        assert tuple(ws.shape) == (self.num_gemms, n_out // 128, k_in // 128), (tuple(ws.shape), tuple(shape))
         wt = weight if isinstance(weight, torch.Tensor) else None
         out_dtype = inp.dtype if inp.dtype in (torch.bfloat16, torch.float32) else torch.bfloat16
         return _GroupedGemmFp8.apply(inp, wt, wq.detach(), ws.detach(), m_splits, out_dtype)
