@@ -125,3 +125,41 @@ def test_export_quantised_tensors():
     assert sorted(got) == ["layers.0.attn.wo_a.weight", "layers.0.attn.wo_b.scale", "layers.0.attn.wo_b.weight"]
     assert got["layers.0.attn.wo_a.weight"].dtype == torch.bfloat16 and got["layers.0.attn.wo_b.weight"].dtype == torch.float8_e4m3fn
     assert all(t.is_cuda for t in got.values())
+
+
+@pytest.mark.parametrize("expert_dtype", ["fp4", "fp8"])
+def test_vllm_reload_bucket_quantisation(expert_dtype):
+    """iter_model_aware_quantized_weights (vllm_weight_reload_dsv4.py:1129-1178): experts by expert_dtype, a linear
+    layer that the live model keeps in e4m3 to FP8, everything else untouched; bytes against the CPU oracle on the
+    bf16 view of fp32 master weights."""
+    from gcore_lowp import vllm_weight_reload_dsv4 as R
+    say("iter_model_aware_quantized_weights", expert_dtype)
+
+    class LinearBase(torch.nn.Module):
+        def __init__(self, dtype):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.zeros(2, 2).to(dtype), requires_grad=False)
+
+    model = torch.nn.Module()
+    model.layers = torch.nn.ModuleList([torch.nn.Module()])
+    model.layers[0].attn = torch.nn.Module()
+    model.layers[0].attn.wq_b = LinearBase(torch.float8_e4m3fn)
+    model.layers[0].attn.wo_b = LinearBase(torch.bfloat16)
+    torch.manual_seed(3)
+    expert, dense, kept = torch.randn(256, 384) * 0.1, torch.randn(128, 256) * 0.1, torch.randn(128, 128)
+    bucket = [("layers.0.ffn.experts.1.w2.weight", expert.cuda()), ("layers.0.attn.wq_b.weight", dense.cuda()),
+              ("layers.0.attn.wo_b.weight", kept.cuda())]
+    out = R.iter_model_aware_quantized_weights(model, bucket, expert_dtype=expert_dtype)
+    assert [n for n, _ in out] == ["layers.0.ffn.experts.1.w2.weight", "layers.0.ffn.experts.1.w2.scale",
+                                   "layers.0.attn.wq_b.weight", "layers.0.attn.wq_b.scale", "layers.0.attn.wo_b.weight"]
+    got = dict(out)
+    assert all(t.is_cuda and t.is_contiguous() for t in got.values())
+    src = expert.bfloat16().float()
+    eq, es = T.quant_fp4_e2m1_scale_e8m0_packed(src) if expert_dtype == "fp4" else T.quant_fp8_e4m3_scale_e8m0(src, (128, 128))
+    assert got["layers.0.ffn.experts.1.w2.weight"].dtype == (torch.int8 if expert_dtype == "fp4" else torch.float8_e4m3fn)
+    assert got["layers.0.ffn.experts.1.w2.scale"].dtype == torch.float8_e8m0fnu
+    assert torch.equal(u8(got["layers.0.ffn.experts.1.w2.weight"]), u8(eq))
+    assert torch.equal(u8(got["layers.0.ffn.experts.1.w2.scale"]), u8(es))
+    dq, ds = T.quant_fp8_e4m3_scale_e8m0(dense.bfloat16().float(), (128, 128))
+    assert torch.equal(u8(got["layers.0.attn.wq_b.weight"]), u8(dq)) and torch.equal(u8(got["layers.0.attn.wq_b.scale"]), u8(ds))
+    assert got["layers.0.attn.wo_b.weight"].dtype == torch.float32 and torch.equal(got["layers.0.attn.wo_b.weight"].cpu(), kept)
