@@ -71,6 +71,7 @@ def main(hf_ckpt_path, save_path, layers=None):
     from safetensors.torch import save_file
 
     from . import _abi as A
+    from ._pipeline import run_pipelined
 
     dev = A.require_gpu()
     os.makedirs(save_path, exist_ok=True)
@@ -93,17 +94,27 @@ def main(hf_ckpt_path, save_path, layers=None):
     for path in files:
         shard = os.path.basename(path)
         out = {}
-        with safe_open(path, framework="pt", device="cpu") as f:
-            for name in f.keys():
-                if not _keep(name, layers) or name.endswith(".scale"):
-                    continue                              # scales are consumed with their weight
-                w = f.get_tensor(name)
-                scale_name = name.replace(".weight", ".scale") if name.endswith(".weight") else name + ".scale"
-                if w.dtype == torch.int8 and scale_name in where:
-                    w = cast_e2m1fn_to_bf16(w.to(dev), fetch(scale_name).to(dev)).cpu()
-                elif w.dtype == torch.float8_e4m3fn and scale_name in where:
-                    w = cast_e4m3fn_to_bf16(w.to(dev), fetch(scale_name).to(dev)).cpu()
-                out[name] = w.contiguous()
+
+        def jobs(path=path):
+            with safe_open(path, framework="pt", device="cpu") as f:
+                for name in f.keys():
+                    if not _keep(name, layers) or name.endswith(".scale"):
+                        continue                          # scales are consumed with their weight
+                    w = f.get_tensor(name)
+                    scale_name = name.replace(".weight", ".scale") if name.endswith(".weight") else name + ".scale"
+                    if w.dtype in (torch.int8, torch.float8_e4m3fn) and scale_name in where:
+                        yield name, (w, fetch(scale_name)), True
+                    else:
+                        yield name, (w, None), False
+
+        def compute(name, tensors):
+            w, scale = tensors
+            if scale is None:
+                return {name: w}
+            return {name: cast_e2m1fn_to_bf16(w, scale) if w.dtype == torch.int8 else cast_e4m3fn_to_bf16(w, scale)}
+
+        for _, conv in run_pipelined(dev, jobs(), compute):
+            out.update({k: v.contiguous() for k, v in conv.items()})
         if not out:
             continue
         save_file(out, os.path.join(save_path, shard))

@@ -22,6 +22,7 @@ import time
 import torch
 
 from . import _abi as A
+from ._pipeline import run_pipelined
 from .dsv4_kernels import (is_expert_weight, is_wo_a_weight, official_dense_to_sgl, official_expert_to_sgl,
                            official_wo_a_to_sgl, scale_key, sgl_dense_to_official, sgl_expert_to_official,
                            sgl_wo_a_to_official)
@@ -131,26 +132,35 @@ def _process_shard(src, dst, shard_name, direction, weight_map, dev):
         return handles[fname].get_tensor(sk) if sk in handles[fname].keys() else None
 
     out, n_conv, n_pass = {}, 0, 0
-    with safe_open(os.path.join(src, shard_name), framework="pt", device="cpu") as sf:
-        for name in sf.keys():
-            if name.endswith(".scale"):
-                continue
-            tensor = sf.get_tensor(name)
-            if not name.endswith(".weight"):
-                out[name] = tensor
-                n_pass += 1
-                continue
-            scale = scale_of(scale_key(name))
-            if _needs_gpu(name, tensor, scale, direction):
-                conv = convert_one_weight(name, tensor.to(dev), scale.to(dev) if scale is not None else None, direction)
-                conv = {k: v.cpu().contiguous() for k, v in conv.items()}
-            else:
-                conv = convert_one_weight(name, tensor, scale, direction)
-            out.update(conv)
-            if list(conv.keys()) == [name] and scale is None:
-                n_pass += 1
-            else:
-                n_conv += 1
+
+    def jobs():
+        with safe_open(os.path.join(src, shard_name), framework="pt", device="cpu") as sf:
+            for name in sf.keys():
+                if name.endswith(".scale"):
+                    continue
+                tensor = sf.get_tensor(name)
+                if not name.endswith(".weight"):
+                    yield (name, False, False), (tensor,), False
+                    continue
+                scale = scale_of(scale_key(name))
+                yield (name, True, scale is not None), (tensor, scale), _needs_gpu(name, tensor, scale, direction)
+
+    def compute(tag, tensors):
+        name, is_weight, _ = tag
+        return convert_one_weight(name, tensors[0], tensors[1], direction) if is_weight else {name: tensors[0]}
+
+    if os.environ.get("LP_CONVERT_PIPELINE", "1") != "0":
+        stream = run_pipelined(dev, jobs(), compute)
+    else:                                             # one tensor at a time, every copy synchronous (for comparison)
+        stream = ((tag, {k: v.cpu() for k, v in compute(tag, [t.to(dev) if on_gpu and t is not None else t
+                                                               for t in host]).items()})
+                  for tag, host, on_gpu in jobs())
+    for (name, is_weight, has_scale), conv in stream:
+        out.update({k: v.contiguous() for k, v in conv.items()})
+        if not is_weight or (list(conv.keys()) == [name] and not has_scale):
+            n_pass += 1
+        else:
+            n_conv += 1
     handles.clear()
     if not out:
         return {}, 0, n_conv, n_pass

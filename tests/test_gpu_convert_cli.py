@@ -223,3 +223,41 @@ def test_convert_json(tmp_path):
         "metadata": {"total_size": 3}, "weight_map": {"model.layers.0.w.weight": "f1"}}
     J.main(["--load_hf_dir", str(src), "--save_hf_dir", str(dst)])
     assert len(json.loads((dst / "model.safetensors.index.json").read_text())["weight_map"]) == 3
+
+
+def test_pipeline_order_results_and_errors():
+    """The converters' host <-> device pipeline: every job comes back once with the right payload, host-only jobs
+    pass through, and an exception on the feeding thread or in the compute step surfaces in the caller."""
+    from gcore_lowp._pipeline import run_pipelined
+    say("run_pipelined")
+    dev = torch.device("cuda", 0)
+    src = [torch.full((257, 33), i, dtype=torch.float32) for i in range(40)]
+
+    def jobs():
+        for i, t in enumerate(src):
+            yield i, (t, None), i % 5 != 0
+
+    def compute(tag, tensors):
+        t = tensors[0]
+        assert t.is_cuda == (tag % 5 != 0)
+        return {"double": t * 2, "meta": torch.tensor([tag])}
+
+    got = dict(run_pipelined(dev, jobs(), compute))
+    assert sorted(got) == list(range(40))
+    for i, res in got.items():
+        assert not res["double"].is_cuda and torch.equal(res["double"], src[i] * 2) and int(res["meta"]) == i
+
+    def bad_jobs():
+        yield 0, (src[0],), True
+        raise OSError("shard unreadable")
+
+    with pytest.raises(OSError, match="shard unreadable"):
+        list(run_pipelined(dev, bad_jobs(), lambda tag, t: {"x": t[0]}))
+
+    def bad_compute(tag, tensors):
+        if tag == 3:
+            raise ValueError("no rule for this weight")
+        return {"x": tensors[0]}
+
+    with pytest.raises(ValueError, match="no rule"):
+        list(run_pipelined(dev, jobs(), bad_compute))
