@@ -261,3 +261,83 @@ def test_pipeline_order_results_and_errors():
 
     with pytest.raises(ValueError, match="no rule"):
         list(run_pipelined(dev, jobs(), bad_compute))
+
+
+@pytest.mark.parametrize(("block", "hidden", "inter", "scale_dtype"),
+                         [((2, 2), 4, 2, torch.bfloat16), ((128, 128), 256, 128, torch.float32), ((128, 128), 256, 192, torch.bfloat16)])
+def test_qwen3_mtp_postprocess(tmp_path, block, hidden, inter, scale_dtype):
+    """append_mtp_weights_to_fp8_checkpoint: stacked experts become per-expert gate / up / down weights, skipped
+    modules stay bf16, the rest is FP8 + weight_scale_inv, stale mtp.* index entries go
+    (tools/convert_fp8/qwen3_5/tests/test_qwen3_mtp_fp8_postprocess.py:77-175); every quantised tensor equals the
+    CPU oracle's.  inter = 192 with 128-row blocks: the up / gate halves do not align with the stack's tiles, so the
+    per-part path runs (and a down_proj of 192 columns is refused like in the reference)."""
+    from gcore_lowp import qwen3_mtp_fp8_postprocess as P
+    say("qwen3 mtp postprocess", block, hidden, inter, scale_dtype)
+    g = torch.Generator().manual_seed(hidden + inter)
+    src, dst = tmp_path / "in", tmp_path / "out"
+    src.mkdir(), dst.mkdir()
+    with open(src / "config.json", "w") as f:
+        json.dump({"text_config": {"model_type": "qwen3_5_moe_text", "num_experts": 2, "mtp_num_hidden_layers": 1}}, f)
+    bf = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
+    down_cols = inter if inter % block[1] == 0 else 256
+    t = {"mtp.fc.weight": bf(hidden, 2 * hidden), "mtp.norm.weight": bf(hidden), "mtp.pre_fc_norm_embedding.weight": bf(hidden),
+         "mtp.pre_fc_norm_hidden.weight": bf(hidden)}
+    L = "mtp.layers.0."
+    for k in ("input_layernorm", "post_attention_layernorm", "self_attn.q_norm", "self_attn.k_norm"):
+        t[L + k + ".weight"] = bf(hidden)
+    for k in ("q_proj", "k_proj", "v_proj", "o_proj"):
+        t[L + f"self_attn.{k}.weight"] = bf(hidden, hidden)
+    t[L + "mlp.experts.gate_up_proj"] = bf(2, 2 * inter, hidden)
+    t[L + "mlp.experts.down_proj"] = bf(2, hidden, down_cols)
+    t[L + "mlp.gate.weight"] = bf(2, hidden)
+    t[L + "mlp.shared_expert.gate_proj.weight"] = bf(hidden, hidden)
+    t[L + "mlp.shared_expert.up_proj.weight"] = bf(hidden, hidden)
+    t[L + "mlp.shared_expert.down_proj.weight"] = bf(hidden, hidden)
+    t[L + "mlp.shared_expert_gate.weight"] = bf(1, hidden)
+    save_file(t, str(src / "input.safetensors"))
+    save_file({"model.language_model.embed_tokens.weight": torch.ones(2, 2, dtype=torch.bfloat16)}, str(dst / "model.safetensors"))
+    with open(dst / "model.safetensors.index.json", "w") as f:
+        json.dump({"metadata": {"format": "pt", "total_size": 123},
+                   "weight_map": {"model.language_model.embed_tokens.weight": "model.safetensors",
+                                  "mtp.stale.weight": "mtp.safetensors"}}, f)
+    skip = ["mtp.fc", "mtp.norm", "mtp.pre_fc_norm_embedding", "mtp.pre_fc_norm_hidden", L + "input_layernorm",
+            L + "post_attention_layernorm", L + "self_attn.q_norm", L + "self_attn.k_norm", L + "mlp.gate", L + "mlp.shared_expert_gate"]
+    if inter % block[0]:
+        with pytest.raises(ValueError, match="must be divisible"):
+            P.append_mtp_weights_to_fp8_checkpoint(str(src), str(dst), block_size=block, modules_to_not_convert=skip,
+                                                   device="cpu", scale_dtype=scale_dtype)
+        return
+    written = P.append_mtp_weights_to_fp8_checkpoint(str(src), str(dst), block_size=block, modules_to_not_convert=skip,
+                                                     device="cpu", scale_dtype=scale_dtype)
+    expected = {}
+    for key, w in t.items():
+        if key.endswith("gate_up_proj"):
+            for e in range(2):
+                expected[L + f"mlp.experts.{e}.gate_proj.weight"], expected[L + f"mlp.experts.{e}.up_proj.weight"] = w[e].chunk(2, dim=0)
+        elif key.endswith("experts.down_proj"):
+            for e in range(2):
+                expected[L + f"mlp.experts.{e}.down_proj.weight"] = w[e]
+        else:
+            expected[key] = w
+    n_quant = 0
+    with safe_open(str(dst / "mtp.safetensors"), framework="pt", device="cpu") as f:
+        keys = set(f.keys())
+        assert L + "mlp.experts.gate_up_proj" not in keys and L + "mlp.experts.down_proj" not in keys
+        for key, w in expected.items():
+            module = key[:-len(".weight")]
+            got = f.get_tensor(key)
+            if any(module == s for s in skip):
+                assert same(got, w) and module + ".weight_scale_inv" not in keys
+                continue
+            n_quant += 1
+            q, s = T.quantize_fp8_blockwise(w, block, scale_dtype=scale_dtype)
+            assert got.dtype == E4M3 and same(got, q), key
+            gs = f.get_tensor(module + ".weight_scale_inv")
+            assert gs.dtype == scale_dtype and tuple(gs.shape) == (w.shape[0] // block[0], w.shape[1] // block[1]) and same(gs, s), key
+    assert written == len(keys) == len(expected) + n_quant
+    with open(dst / "model.safetensors.index.json") as f:
+        index = json.load(f)
+    assert index["metadata"]["format"] == "pt" and index["metadata"]["total_size"] > 123
+    wm = index["weight_map"]
+    assert wm["model.language_model.embed_tokens.weight"] == "model.safetensors" and "mtp.stale.weight" not in wm
+    assert all(wm[k] == "mtp.safetensors" for k in keys) and len(wm) == len(keys) + 1
