@@ -341,3 +341,91 @@ def test_qwen3_mtp_postprocess(tmp_path, block, hidden, inter, scale_dtype):
     wm = index["weight_map"]
     assert wm["model.language_model.embed_tokens.weight"] == "model.safetensors" and "mtp.stale.weight" not in wm
     assert all(wm[k] == "mtp.safetensors" for k in keys) and len(wm) == len(keys) + 1
+
+
+def _bf16_ckpt(root):
+    g = torch.Generator().manual_seed(9)
+    bf = lambda *s: (torch.randn(*s, generator=g) * 0.05).to(torch.bfloat16)
+    t = {"model.embed_tokens.weight": bf(64, 128), "lm_head.weight": bf(64, 128), "model.norm.weight": bf(128)}
+    for layer in (0, 1):
+        p = f"model.layers.{layer}."
+        t[p + "self_attn.q_proj.weight"] = bf(256, 128)
+        t[p + "self_attn.kv_a_proj_with_mqa.weight"] = bf(72, 128)          # 72 rows: an edge tile
+        t[p + "self_attn.o_proj.weight"] = bf(128, 200)                      # 200 columns: an edge tile
+        t[p + "input_layernorm.weight"] = bf(128)
+        t[p + "mlp.gate.weight"] = bf(4, 128)
+        t[p + "mlp.experts.0.down_proj.weight"] = torch.zeros(128, 256, dtype=torch.bfloat16)   # all-zero tiles
+        t[p + "mlp.gate.e_score_correction_bias"] = torch.randn(4, generator=g)
+    shard_of = {k: ("model-00001-of-00002.safetensors" if "layers.1." not in k else "model-00002-of-00002.safetensors") for k in t}
+    os.makedirs(root, exist_ok=True)
+    for shard in sorted(set(shard_of.values())):
+        save_file({k: v for k, v in t.items() if shard_of[k] == shard}, os.path.join(root, shard))
+    with open(os.path.join(root, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": shard_of}, f)
+    with open(os.path.join(root, "config.json"), "w") as f:
+        json.dump({"model_type": "deepseek_v3", "hidden_size": 128}, f)
+    return t, shard_of
+
+
+def _padded_quant(w):
+    rows, cols = w.shape
+    wp = torch.nn.functional.pad(w.float(), (0, -cols % 128, 0, -rows % 128))
+    q, s = T.quant_block_fp32_scale(wp, (128, 128), amax_floor=None, zero_scale_to_one=True)
+    return q[:rows, :cols].contiguous(), s
+
+
+@pytest.mark.parametrize("with_reference", [False, True])
+def test_bf16_cast_fp8_cli(tmp_path, with_reference):
+    """tools/convert_fp8/bf16_cast_fp8.py drop-in: which tensors are quantised (by name rule, or by a reference FP8
+    checkpoint's `_scale_inv` keys), `<weight>_scale_inv` fp32 next to the weight in the same shard, index and side
+    files; codes and scales against the CPU oracle's divide form on zero-completed edge tiles."""
+    say("bf16_cast_fp8 cli", with_reference)
+    src, dst, ref = str(tmp_path / "bf16"), str(tmp_path / "fp8"), str(tmp_path / "ref")
+    t, shard_of = _bf16_ckpt(src)
+    cmd = [sys.executable, "-m", "gcore_lowp.bf16_cast_fp8", "--input-bf16-hf-path", src, "--output-fp8-hf-path", dst]
+    if with_reference:
+        # a reference FP8 checkpoint in which only q_proj (layers 0, 1) and layer 0's o_proj are FP8
+        os.makedirs(ref)
+        chosen = [k for k in t if k.endswith("q_proj.weight")] + ["model.layers.0.self_attn.o_proj.weight"]
+        rt = {}
+        for k, v in t.items():
+            rt[k] = v.to(E4M3) if k in chosen else v
+            if k in chosen:
+                rt[k + "_scale_inv"] = torch.ones(-(-v.shape[0] // 128), -(-v.shape[1] // 128))
+        rt["model.layers.1.self_attn.o_proj.weight"] = t["model.layers.1.self_attn.o_proj.weight"].to(E4M3)   # FP8, no scale: skipped
+        save_file(rt, os.path.join(ref, "model.safetensors"))
+        with open(os.path.join(ref, "model.safetensors.index.json"), "w") as f:
+            json.dump({"metadata": {}, "weight_map": {k: "model.safetensors" for k in rt}}, f)
+        with open(os.path.join(ref, "config.json"), "w") as f:
+            json.dump({"model_type": "deepseek_v3", "from": "reference"}, f)
+        cmd += ["--input-fp8-hf-path", ref]
+    else:
+        chosen = [k for k in t if k.endswith("_proj.weight")]
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-3000:]
+    with open(os.path.join(dst, "model.safetensors.index.json")) as f:
+        wm = json.load(f)["weight_map"]
+    assert set(wm) == set(t) | {k + "_scale_inv" for k in chosen}
+    for k in t:
+        assert wm[k] == shard_of[k]
+        with safe_open(os.path.join(dst, wm[k]), framework="pt", device="cpu") as f:
+            got = f.get_tensor(k)
+            if k in chosen:
+                q, s = _padded_quant(t[k])
+                assert wm[k + "_scale_inv"] == shard_of[k]
+                gs = f.get_tensor(k + "_scale_inv")
+                assert got.dtype == E4M3 and same(got, q), k
+                assert gs.dtype == torch.float32 and same(gs, s), k
+            else:
+                assert same(got, t[k]), k
+                assert k + "_scale_inv" not in f.keys()
+    with open(os.path.join(dst, "config.json")) as f:
+        cfg = json.load(f)
+    if with_reference:
+        assert cfg.get("from") == "reference" and "quantization_config" not in cfg
+        with open(os.path.join(dst, "weight_with_scale_inv_map.index.json")) as f:
+            assert set(json.load(f)["weight_with_scale_inv_map"]) == set(chosen)
+    else:
+        assert cfg["quantization_config"] == {"activation_scheme": "dynamic", "fmt": "e4m3", "quant_method": "fp8",
+                                              "weight_block_size": [128, 128], "modules_to_not_convert": ["lm_head"]}
