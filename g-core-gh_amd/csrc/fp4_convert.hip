@@ -38,6 +38,24 @@ __device__ __forceinline__ uint32_t tile_max_u32(uint32_t m, uint32_t (*lds)[16]
     return r;
 }
 
+// Same reduction for both tiles of the super tile at once: every lane gets its own tile's maximum and
+// the other tile's, from one barrier.  The caller must put a barrier before it uses `lds` again.
+__device__ __forceinline__ void tile_max_both_u32(uint32_t m, uint32_t (*lds)[16], int t, uint32_t &own, uint32_t &other)
+{
+    m = row16_max_u32(m);
+    const int row = t >> 4;
+    if ((t & 15) == 0) lds[row & 1][row >> 1] = m;
+    __syncthreads();
+    const int half = row & 1;
+    own = 0; other = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t a = lds[half][i], b = lds[half ^ 1][i];
+        own = a > own ? a : own;
+        other = b > other ? b : other;
+    }
+}
+
 struct Geometry {
     int64_t row0;        // first row of this lane in pass 0
     int64_t colb;        // byte column of this lane's 4 packed bytes
@@ -49,7 +67,9 @@ struct Geometry {
 __device__ __forceinline__ Geometry geometry(int64_t super, int64_t supers_c, int64_t cols, int t)
 {
     Geometry g;
-    const int64_t sr = super / supers_c, sc = super - sr * supers_c;
+    // the launchers keep the number of super tiles below 2^31: a 32-bit division instead of the
+    // ~150 scalar instructions of a 64-bit one
+    const int64_t sr = (uint32_t)super / (uint32_t)supers_c, sc = super - sr * supers_c;
     const int lane32 = t & 31;
     const int64_t col = sc * 256 + lane32 * 8;      // logical column of the lane's first element
     g.row0 = sr * 128 + (t >> 5);
@@ -166,10 +186,14 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
         mbits = prod > mbits ? prod : mbits;
         edge |= (sb[p] < 2u || sb[p] > 252u) ? 1u : 0u;
     }
-    // Every thread of the workgroup must take the same number of barriers, so both slow
-    // decisions (edge scale bytes, tile scale outside the fast range) are made for the
-    // super tile as a whole.
-    bool slow_tile = __syncthreads_or((int)edge) != 0;
+    // Every thread of the workgroup must take the same number of barriers, so both slow decisions
+    // (edge scale bytes, tile scale outside the fast range) are made for the super tile as a whole -- by
+    // every lane for both tiles, from one reduction: an edge byte travels as the key 0xFFFFFFFF (products
+    // are finite positive floats, so that pattern is free), and the scale of the other tile is derived
+    // redundantly instead of being voted on.
+    uint32_t key, key_other;
+    tile_max_both_u32(edge ? 0xFFFFFFFFu : mbits, lds, t, key, key_other);
+    bool slow_tile = key == 0xFFFFFFFFu || key_other == 0xFFFFFFFFu;
     BlockScale bs;
     // Each element is +-{0, .5, 1, 2, 4} * 2^e (even codes and 0.5) or +-{1, 2, 4} * 1.5 * 2^e (codes
     // 1.5, 3, 6), so its quotient by the tile scale is a power-of-two multiple of one of two numbers,
@@ -178,49 +202,58 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
     // them correctly rounded.
     float c1 = 1.0f, c3 = 1.5f;
     if (!slow_tile) {
-        const uint32_t key = tile_max_u32(mbits, lds, t);
+        auto out_of_range = [&](const BlockScale &b) -> bool {
+            if (MODE == LP_SCALE_POW2) return b.exp2 < -100 || b.exp2 > 100;
+            if (MODE == LP_SCALE_DIV) return !b.fast;
+            return !(b.div >= 0x1p-100f && b.div <= 0x1p100f);
+        };
         bs = derive_scale<MODE>(u2f(key), amax_floor, zero_rule);
-        bool bad;
+        slow_tile = out_of_range(bs) || out_of_range(derive_scale<MODE>(u2f(key_other), amax_floor, zero_rule));
         if (MODE == LP_SCALE_POW2) {
-            bad = bs.exp2 < -100 || bs.exp2 > 100;
             c1 = ldexpf(1.0f, -bs.exp2);
             c3 = ldexpf(1.5f, -bs.exp2);
         } else if (MODE == LP_SCALE_DIV) {
-            bad = !bs.fast;
             c1 = bs.recip;
             c3 = 1.5f / bs.div;
         } else {
-            bad = !(bs.div >= 0x1p-100f && bs.div <= 0x1p100f);
             c1 = bs.div;
             c3 = 1.5f * bs.div;
         }
-        slow_tile = __syncthreads_or((int)bad) != 0;
     }
 
     if (!slow_tile) {
         if (g.active && (t & 15) == 0 && (t >> 5) == 0) store_scale(scale_out, scale_dtype, g.tile, bs.stored);
         if (!g.active) return;
+        // All 8 elements of a pass share one scale byte sb, so their codes are eight numbers per pass:
+        //   magnitude 0 .5 1 1.5 2 3 4 6  ->  e4m3(0, t1/2, t1, t3, 2 t1, 2 t3, 4 t1, 4 t3),  t = c * 2^(sb-127).
+        // Four conversions build that table in two registers and byte permutes look the nibbles up: no
+        // decode, no multiply per element (a conversion costs about 3 plain VALU instructions, measured).
+        // The factors are formed by adding to the exponent field.  c1 and c3 are normal here (exponent
+        // field cf, c3's at most cf + 1), so t1/2 .. 4 t3 are normal floats for sb in [129 - cf, 378 - cf],
+        // and clamping sb to that range changes no result: a non-zero block has 2^(sb-127) <= 2 amax,
+        // i.e. sb <= 264 - cf, so above the range every element is zero (and zero maps to table entry 0);
+        // below it every quotient is under 2^-120 in magnitude and becomes a signed zero with the clamped
+        // factor as with the true one.
+        const uint32_t c1b = f2u(c1), c3b = f2u(c3);
+        const int cf = (int)(c1b >> 23);
+        const int sb_lo = 129 - cf, sb_hi = 378 - cf;
+        const uint32_t c1adj = c1b - (127u << 23), c3adj = c3b - (127u << 23);
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int64_t r = g.row0 + p * kRowsPerPass;
-            const int e = (int)sb[p] - 127;
-            // an all-zero block may carry any exponent: keep the factors finite so that 0 * t stays 0
-            const float t1 = fminf(ldexpf(c1, e), 3.0e38f), t3 = fminf(ldexpf(c3, e), 3.0e38f);
-            // decode again rather than keep decoded values alive across the reduction: the empty asm
-            // hides the value from common-subexpression elimination so the register footprint stays small
+            int sbe = (int)sb[p];
+            sbe = sbe < sb_lo ? sb_lo : (sbe > sb_hi ? sb_hi : sbe);
+            const uint32_t t1 = c1adj + ((uint32_t)sbe << 23), t3 = c3adj + ((uint32_t)sbe << 23);
+            const uint32_t tab_lo = cvt4(0.0f, u2f(t1 - (1u << 23)), u2f(t1), u2f(t3));
+            const uint32_t tab_hi = cvt4(u2f(t1 + (1u << 23)), u2f(t3 + (1u << 23)), u2f(t1 + (2u << 23)), u2f(t3 + (2u << 23)));
             uint32_t wp = w[p];
-            asm volatile("" : "+v"(wp));
-            const uint32_t mant = wp & 0x11111111u;
-            const uint32_t expnz = ((wp >> 1) | (wp >> 2)) & 0x11111111u;
-            const uint32_t odd = mant & expnz;                  // nibbles holding 1.5, 3 or 6
-            const uint32_t oddmask = (odd << 4) - odd;          // 0xF on those nibbles
-            float fe[8], fo[8];
-            fp4_decode8(wp & ~oddmask, fe);                     // the other elements, as they are
-            fp4_decode8((wp & oddmask) ^ odd, fo);              // 1.5, 3, 6 with the mantissa bit cleared: 1, 2, 4
-            float v[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = __builtin_fmaf(fo[j], t3, fe[j] * t1);
-            u32x2 out = {cvt4(v[0], v[1], v[2], v[3]), cvt4(v[4], v[5], v[6], v[7])};
+            asm volatile("" : "+v"(wp));                       // keep the packed word, not values derived before the barrier
+            // even elements sit in the low nibbles of the four bytes, odd elements in the high nibbles
+            uint32_t ce = __builtin_amdgcn_perm(tab_hi, tab_lo, wp & 0x07070707u);
+            uint32_t co = __builtin_amdgcn_perm(tab_hi, tab_lo, (wp >> 4) & 0x07070707u);
+            ce |= (wp & 0x08080808u) << 4;                     // signs (zero magnitudes carry none, see fp4_pos_zero)
+            co |= wp & 0x80808080u;
+            u32x2 out = {__builtin_amdgcn_perm(co, ce, 0x05010400u), __builtin_amdgcn_perm(co, ce, 0x07030602u)};
             __builtin_nontemporal_store(out, (u32x2 *)(q + r * cols + (g.colb << 1)));
             if (WRITE_BF16) {
                 const float s = u2f(sb[p] << 23);            // sb in 2..252: a normal power of two
@@ -234,6 +267,7 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
         return;
     }
 
+    __syncthreads();                                          // the reduction below writes `lds` again
     // Slow tile: scale bytes at the edge of the e8m0 range (bf16 rounding,
     // overflow to inf, NaN).  Literal arithmetic with software casts; inputs
     // are read again from memory so that the fast path keeps its registers.

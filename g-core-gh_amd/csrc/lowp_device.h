@@ -110,7 +110,11 @@ __device__ __forceinline__ float clamp448(float y) { return __builtin_amdgcn_fme
 // four floats -> four e4m3fn bytes (element 0 in the low byte)
 __device__ __forceinline__ uint32_t cvt4(float a, float b, float c, float d)
 {
-    int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    // the first conversion keeps the other half of its destination and the second one overwrites that half:
+    // starting from an undefined register (an asm output) saves the move that a zero would cost
+    int w;
+    asm volatile("" : "=v"(w));
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
     w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
     return (uint32_t)w;
 }

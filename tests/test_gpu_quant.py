@@ -272,6 +272,34 @@ def test_fp4_fused_amax_parity(G):
         assert bits_equal(hq2, hq) and bits_equal(hs2, hs)
 
 
+def test_fp4_fused_other_scale_modes(G):
+    """The fused FP4 -> FP8 kernel with the power-of-two and the multiply-by-reciprocal scale rules: bytes equal
+    FP4 -> bf16 (exact) followed by the oracle's quantiser of that rule; wide scale ranges put blocks far below the
+    tile maximum (signed zeros) next to blocks at it."""
+    from gcore_lowp import _abi as A
+    from gcore_lowp import ops
+    for (rows, cols), seed, (lo, hi) in [((256, 384), 11, (117, 127)), ((128, 640), 12, (2, 252)), ((128, 512), 13, (90, 150)),
+                                         ((2048, 7168), 14, (117, 127))]:
+        p, s = I.fp4_expert(rows, cols, seed, lo, hi)
+        if seed == 11:
+            p.view(torch.uint8)[:128, :64] = 0x80          # a tile of zeros
+        w = T.cast_e2m1fn_to_bf16(p, s)
+        say("fp4 fused, power-of-two scales", rows, cols, lo, hi)
+        rq, rs = T.quant_fp8_e4m3_scale_e8m0(w, (128, 128))
+        hq, hs = ops.fp4_to_fp8_amax(p.view(torch.uint8).cuda(), s.cuda(), scale_mode=A.SCALE_POW2, scale_dtype=torch.float8_e8m0fnu,
+                                     amax_floor=0.0)
+        assert bits_equal(hs, rs) and bits_equal(hq, rq)
+        say("fp4 fused, 448/amax multiply form", rows, cols, lo, hi)
+        rq, rs = T.quantize_fp8_blockwise(w, (128, 128), scale_dtype=torch.float32)
+        hq, hs = ops.fp4_to_fp8_amax(p.view(torch.uint8).cuda(), s.cuda(), scale_mode=A.SCALE_MUL, scale_dtype=torch.float32,
+                                     amax_floor=0.0)
+        finite = torch.isfinite(rs)
+        assert bits_equal(hs[finite], rs[finite])
+        a, b = u8(hq), u8(rq)
+        ok = (b & 0x7F) != 0x7F
+        assert torch.equal(a[ok], b[ok])
+
+
 def test_full_size_round_trip_properties(G):
     """Benchmark config 1 at full size: [4096, 4096] bf16, N(0, 0.02) + 0.1 % outliers."""
     x = I.weight_like(4096, 4096, 100).cuda()
