@@ -19,7 +19,8 @@ def cast_e2m1fn_to_bf16(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     assert in_dim % 32 == 0
     assert scale.size(0) == out_dim and scale.size(1) == in_dim // 32
     sc = scale if scale.dtype in (torch.float32, torch.bfloat16, ops.E8M0) else scale.float()
-    return ops.dequant_block(x.view(torch.uint8), sc, fp4=True, fp4_neg_zero=False, out_dtype=torch.bfloat16)
+    return ops.dequant_block(x.view(torch.uint8), sc, fp4=True, fp4_neg_zero=False, out_dtype=torch.bfloat16,
+                             block=(1, 32))
 
 
 def cast_e4m3fn_to_bf16(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
@@ -31,7 +32,7 @@ def cast_e4m3fn_to_bf16(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     assert out_dim % 128 == 0 and in_dim % 128 == 0
     assert scale.size() == (out_dim // 128, in_dim // 128)
     sc = scale if scale.dtype in (torch.float32, torch.bfloat16, ops.E8M0) else scale.float()
-    return ops.dequant_block(x.view(torch.uint8), sc, fp4=False, out_dtype=torch.bfloat16)
+    return ops.dequant_block(x.view(torch.uint8), sc, fp4=False, out_dtype=torch.bfloat16, block=(128, 128))
 
 
 # ---------------------------------------------------------------------------------------------

@@ -73,14 +73,15 @@ def _block_from_shapes(rows, cols, scales, what):
 
 
 def dequant_block(codes: torch.Tensor, scales: torch.Tensor, *, fp4: bool, fp4_neg_zero: bool = True,
-                  out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
-    """e4m3fn [..., M, N] or packed e2m1 [..., M, N/2] times block scales -> out_dtype [..., M, N]."""
+                  out_dtype: torch.dtype = torch.bfloat16, block: tuple[int, int] | None = None) -> torch.Tensor:
+    """e4m3fn [..., M, N] or packed e2m1 [..., M, N/2] times block scales -> out_dtype [..., M, N].  The block is
+    the ratio of the two shapes unless the caller's format fixes it (`block`; then an empty tensor is fine too)."""
     cg, home = A.to_device(codes)
     sg = scales.to(cg.device).contiguous()
     cg = cg.contiguous()
     m = cg.shape[-2]
     n = cg.shape[-1] * (2 if fp4 else 1)
-    bm, bn = _block_from_shapes(m, n, sg, "Weight")
+    bm, bn = block if block is not None else _block_from_shapes(m, n, sg, "Weight")
     lead = tuple(cg.shape[:-2])
     if tuple(sg.shape[:-2]) != lead:
         raise ValueError(f"leading dims of codes {lead} and scales {tuple(sg.shape[:-2])} differ")
