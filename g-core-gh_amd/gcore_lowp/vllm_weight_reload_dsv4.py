@@ -21,7 +21,8 @@ from .eager_quant_kernels import quant_fp4_e2m1_scale_e8m0_packed, quant_fp8_e4m
 
 __all__ = ["DSV4_EXPERT_WEIGHT_RE", "DSV4_VLLM_LOAD_RENAMES", "apply_shared_expert_alias", "base_reload_name_variants",
            "candidate_param_names_for_reflection", "get_module_from_param_name", "iter_model_aware_quantized_weights",
-           "map_checkpoint_key_to_vllm_param_name", "module_from_param_name", "with_model_prefix_variants"]
+           "loaded_name_candidates", "map_checkpoint_key_to_vllm_param_name", "module_from_param_name",
+           "with_model_prefix_variants"]
 
 _MEGA_MOE_CLS = "DeepseekV4MegaMoEExperts"
 _LAYER = r"^(layers\.\d+)\."
@@ -90,6 +91,21 @@ def with_model_prefix_variants(names: Iterable[str]) -> list[str]:
         if not n.startswith("model."):
             out.append(f"model.{n}")
     return _unique(out)
+
+
+def loaded_name_candidates(name: str) -> set[str]:
+    """Names under which vLLM's `load_weights` may report that checkpoint key `name` was loaded (:843-861): every
+    variant with and without the `model.` prefix, and for a `.scale` key also `.weight_scale` / `.weight_scale_inv`."""
+    base = base_reload_name_variants(name)
+    out = set(with_model_prefix_variants(base))
+    for b in base:
+        if b.endswith(".scale"):
+            stem = b[: -len(".scale")]
+            for alias in (f"{stem}.weight_scale", f"{stem}.weight_scale_inv"):
+                out.add(alias)
+                if not alias.startswith("model."):
+                    out.add(f"model.{alias}")
+    return out
 
 
 def candidate_param_names_for_reflection(model: nn.Module, name: str) -> list[str]:

@@ -126,3 +126,40 @@ def test_routing(expert_dtype):
 def test_scale_key_in_bucket_is_an_error():
     with pytest.raises(RuntimeError, match="expects bf16 weight keys"):
         R.iter_model_aware_quantized_weights(_Model(), [("layers.0.attn.wq_b.scale", torch.ones(1))], expert_dtype="fp8")
+
+
+def test_reference_alias_cases():
+    """The alias expectations of tests/test_gpatch_v4/test_vllm_weight_reload.py:217-339."""
+    c = R.loaded_name_candidates("layers.0.attn.wq_b.scale")
+    assert {"layers.0.attn.wq_b.weight_scale_inv", "model.layers.0.attn.wq_b.scale", "model.layers.0.attn.wq_b.weight_scale_inv"} <= c
+    assert "model.embed_tokens.weight" in R.loaded_name_candidates("embed.weight")
+    assert "model.lm_head.weight" in R.loaded_name_candidates("head.weight")
+    c = R.loaded_name_candidates("model.layers.0.attn.wq_b.scale")
+    assert {"layers.0.attn.wq_b.weight_scale_inv", "model.layers.0.attn.wq_b.weight_scale_inv"} <= c
+    assert "model.model.layers.0.attn.wq_b.scale" not in c
+    for key in ("layers.0.attn.wq_a.weight", "layers.0.attn.wkv.weight"):
+        assert "model.layers.0.attn.fused_wqa_wkv.weight" in R.loaded_name_candidates(key)
+    for key in ("layers.0.attn.wq_a.scale", "layers.0.attn.wkv.scale"):
+        assert "model.layers.0.attn.fused_wqa_wkv.weight_scale_inv" in R.loaded_name_candidates(key)
+    fused = "model.layers.2.attn.mla_attn.compressor.fused_wkv_wgate.weight"
+    assert fused in R.loaded_name_candidates("layers.2.attn.compressor.wkv.weight")
+    assert fused in R.loaded_name_candidates("layers.2.attn.compressor.wgate.weight")
+    assert "model.layers.2.attn.mla_attn.compressor.norm.weight" in R.loaded_name_candidates("layers.2.attn.compressor.norm.weight")
+    assert "model.layers.2.attn.mla_attn.compressor.ape" in R.loaded_name_candidates("layers.2.attn.compressor.ape")
+    ifused = "model.layers.2.attn.indexer.compressor.fused_wkv_wgate.weight"
+    assert ifused in R.loaded_name_candidates("layers.2.attn.indexer.compressor.wkv.weight")
+    assert ifused in R.loaded_name_candidates("layers.2.attn.indexer.compressor.wgate.weight")
+    m = nn.Module()
+    assert "model.layers.0.ffn.experts.w13_weight" in R.candidate_param_names_for_reflection(m, "layers.0.ffn.experts.3.w1.weight")
+    assert "model.layers.0.ffn.experts.w2_weight" in R.candidate_param_names_for_reflection(m, "layers.0.ffn.experts.3.w2.weight")
+    assert "model.layers.0.ffn.experts.w13_weight" in R.candidate_param_names_for_reflection(m, "layers.0.ffn.experts.3.w3.weight")
+    gate_up = "model.layers.0.ffn.shared_experts.gate_up_proj.weight"
+    assert gate_up in R.candidate_param_names_for_reflection(m, "layers.0.ffn.shared_experts.w1.weight")
+    assert gate_up in R.candidate_param_names_for_reflection(m, "layers.0.ffn.shared_experts.w3.weight")
+    assert "model.layers.0.ffn.shared_experts.down_proj.weight" in R.candidate_param_names_for_reflection(m, "layers.0.ffn.shared_experts.w2.weight")
+    assert gate_up + "_scale_inv" in R.candidate_param_names_for_reflection(m, "layers.0.ffn.shared_experts.w1.scale")
+    # the loader mapping keeps the shard names of the fused gate_up projection
+    assert R.map_checkpoint_key_to_vllm_param_name(m, "layers.0.ffn.shared_experts.w1.scale") == \
+        "model.layers.0.ffn.shared_experts.w1.weight_scale_inv"
+    assert R.map_checkpoint_key_to_vllm_param_name(m, "layers.0.ffn.shared_experts.w3.scale") == \
+        "model.layers.0.ffn.shared_experts.w3.weight_scale_inv"
