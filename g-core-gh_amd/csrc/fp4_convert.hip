@@ -7,11 +7,11 @@
 //                (exact), then quantised like a 128 x 128 bf16 tile
 //                (scale from amax); the bf16 tensor is written only on request.
 //
-// One 256-thread workgroup owns a 128-row x 256-column "super tile" (two scale
+// One workgroup (256 or 512 threads) owns a 128-row x 256-column "super tile" (two scale
 // tiles side by side) so that every row segment it touches is a full 128-byte
 // line of packed input and 256 bytes of output.  Lane l of a 32-lane half wave
 // owns 4 packed bytes (8 elements); lanes 0-15 belong to the left tile, 16-31
-// to the right one.  The packed tile lives in 16 VGPRs per lane, so HBM is
+// to the right one.  The packed tile lives in 16 (8) VGPRs per lane, so HBM is
 // read exactly once.
 #include "lowp_device.h"
 
@@ -19,41 +19,41 @@ using namespace lowp;
 
 namespace {
 
-constexpr int kRowsPerPass = 8;     // 256 threads / 32 lanes per row
-constexpr int kPasses = 16;         // 128 rows
+// Threads per workgroup (NT, a template parameter of everything below): 32 lanes cover a row of the super tile, so
+// a pass covers NT / 32 rows and a lane makes 128 / (NT / 32) passes.  Measured on config 5: the re-basing kernel
+// is 3-5 % faster with 512 threads than with 256, the fused kernel is indifferent (its per-tile set-up weighs
+// more when a lane has fewer passes; with 1024 threads both lose 10-20 %).
+constexpr int kRebaseThreads = 512;
+constexpr int kAmaxThreads = 256;
 
-// Max over one 128 x 128 tile.  `half` (0/1) selects the tile inside the
-// super tile; the 16 lanes of a DPP row all belong to the same half.
-__device__ __forceinline__ uint32_t tile_max_u32(uint32_t m, uint32_t (*lds)[16], int t)
-{
-    m = row16_max_u32(m);
-    const int row = t >> 4;              // 16 DPP rows in the workgroup; row & 1 = half
-    if ((t & 15) == 0) lds[row & 1][row >> 1] = m;
-    __syncthreads();
-    const int half = row & 1;
-    uint32_t r = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { uint32_t o = lds[half][i]; r = o > r ? o : r; }
-    __syncthreads();
-    return r;
-}
-
-// Same reduction for both tiles of the super tile at once: every lane gets its own tile's maximum and
-// the other tile's, from one barrier.  The caller must put a barrier before it uses `lds` again.
+// Maxima over the two 128 x 128 tiles of the super tile: every lane gets its own tile's and the other tile's,
+// from one barrier.  The 16 lanes of a DPP row all belong to one tile and the rows of a wave alternate between
+// the tiles, so a wave reduces to one value per tile (DPP within rows, one cross-lane exchange between rows r and
+// r + 2), the workgroup's waves meet in `lds`, and a second DPP reduction over one entry per lane finishes.
+// The caller must put a barrier before it uses `lds` again.
+template <int NT>
 __device__ __forceinline__ void tile_max_both_u32(uint32_t m, uint32_t (*lds)[16], int t, uint32_t &own, uint32_t &other)
 {
     m = row16_max_u32(m);
-    const int row = t >> 4;
-    if ((t & 15) == 0) lds[row & 1][row >> 1] = m;
+    const uint32_t o = (uint32_t)__shfl_xor((int)m, 32);
+    m = o > m ? o : m;
+    const int half = (t >> 4) & 1;
+    if ((t & 47) == 0) lds[half][t >> 6] = m;          // lanes 0 and 16 of every wave
     __syncthreads();
-    const int half = row & 1;
-    own = 0; other = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t a = lds[half][i], b = lds[half ^ 1][i];
-        own = a > own ? a : own;
-        other = b > other ? b : other;
-    }
+    const int e = t & 15;
+    const uint32_t a = e < NT / 64 ? lds[half][e] : 0u, b = e < NT / 64 ? lds[half ^ 1][e] : 0u;
+    own = row16_max_u32(a);
+    other = row16_max_u32(b);
+}
+
+// Max over the lane's own tile; leaves `lds` free for the next use.
+template <int NT>
+__device__ __forceinline__ uint32_t tile_max_u32(uint32_t m, uint32_t (*lds)[16], int t)
+{
+    uint32_t own, other;
+    tile_max_both_u32<NT>(m, lds, t, own, other);
+    __syncthreads();
+    return own;
 }
 
 struct Geometry {
@@ -85,10 +85,12 @@ __device__ __forceinline__ Geometry geometry(int64_t super, int64_t supers_c, in
 // that neighbours sharing scale cache lines sit behind the same L2.
 __device__ __forceinline__ int64_t xcd_remap(int64_t b, int64_t per_xcd) { return (b & 7) * per_xcd + (b >> 3); }
 
-__global__ __launch_bounds__(256) void fp4_rebase(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scale,
+template <int NT>
+__global__ __launch_bounds__(NT) void fp4_rebase(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scale,
                                                   int64_t cols, int64_t supers_c, int64_t n_supers, int64_t per_xcd,
                                                   uint8_t *__restrict__ q, void *__restrict__ scale_out, int scale_dtype)
 {
+    constexpr int kRowsPerPass = NT / 32, kPasses = 128 / kRowsPerPass;
     __shared__ uint32_t lds[2][16];
     const int64_t super = xcd_remap(blockIdx.x, per_xcd);
     if (super >= n_supers) return;
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(256) void fp4_rebase(const uint8_t *__restrict__ pa
     uint32_t S = 0;
 #pragma unroll
     for (int p = 0; p < kPasses; ++p) S = sb[p] > S ? sb[p] : S;
-    S = tile_max_u32(S, lds, t);
+    S = tile_max_u32<NT>(S, lds, t);
 
     const bool nan_tile = S == 0xFFu;
     if (g.active && (t & 15) == 0 && (t >> 5) == 0) {
@@ -146,12 +148,13 @@ __global__ __launch_bounds__(256) void fp4_rebase(const uint8_t *__restrict__ pa
 
 // ---------------------------------------------------------------- fused amax
 
-template <int MODE, bool WRITE_BF16>
-__global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scale,
+template <int MODE, bool WRITE_BF16, int NT>
+__global__ __launch_bounds__(NT) void fp4_amax(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scale,
                                                 int64_t cols, int64_t supers_c, int64_t n_supers, int64_t per_xcd,
                                                 float amax_floor, int zero_rule, uint8_t *__restrict__ q,
                                                 void *__restrict__ scale_out, int scale_dtype, uint16_t *__restrict__ bf16_out)
 {
+    constexpr int kRowsPerPass = NT / 32, kPasses = 128 / kRowsPerPass;
     __shared__ uint32_t lds[2][16];
     const int64_t super = xcd_remap(blockIdx.x, per_xcd);
     if (super >= n_supers) return;
@@ -192,7 +195,7 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
     // are finite positive floats, so that pattern is free), and the scale of the other tile is derived
     // redundantly instead of being voted on.
     uint32_t key, key_other;
-    tile_max_both_u32(edge ? 0xFFFFFFFFu : mbits, lds, t, key, key_other);
+    tile_max_both_u32<NT>(edge ? 0xFFFFFFFFu : mbits, lds, t, key, key_other);
     bool slow_tile = key == 0xFFFFFFFFu || key_other == 0xFFFFFFFFu;
     BlockScale bs;
     // Each element is +-{0, .5, 1, 2, 4} * 2^e (even codes and 0.5) or +-{1, 2, 4} * 1.5 * 2^e (codes
@@ -284,7 +287,7 @@ __global__ __launch_bounds__(256) void fp4_amax(const uint8_t *__restrict__ pack
             }
         }
     }
-    m2 = tile_max_u32(m2, lds, t);
+    m2 = tile_max_u32<NT>(m2, lds, t);
     const bool has_nan = m2 > 0x7F800000u;
     const float amax = u2f(has_nan ? 0x7FC00000u : m2);
     bs = derive_scale<MODE>(amax, amax_floor, zero_rule);
@@ -335,7 +338,7 @@ extern "C" int lp_fp4_to_fp8_rebase(const void *packed, const void *scale, int64
     const int64_t supers_c = (cols + 255) / 256, n_supers = (rows / 128) * supers_c;
     const int64_t per_xcd = (n_supers + 7) / 8;
     LP_REQUIRE(per_xcd * 8 <= 0x7FFFFFFF, "lp_fp4_to_fp8_rebase: too many tiles");
-    hipLaunchKernelGGL(fp4_rebase, dim3((unsigned)(per_xcd * 8)), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)packed,
+    hipLaunchKernelGGL(fp4_rebase<kRebaseThreads>, dim3((unsigned)(per_xcd * 8)), dim3(kRebaseThreads), 0, (hipStream_t)stream, (const uint8_t *)packed,
                        (const uint8_t *)scale, cols, supers_c, n_supers, per_xcd, (uint8_t *)q_out, scale_out, scale_dtype);
     return check_launch("lp_fp4_to_fp8_rebase");
 }
@@ -354,16 +357,16 @@ extern "C" int lp_fp4_to_fp8_amax(const void *packed, const void *scale, int64_t
     const int64_t supers_c = (cols + 255) / 256, n_supers = (rows / 128) * supers_c;
     const int64_t per_xcd = (n_supers + 7) / 8;
     LP_REQUIRE(per_xcd * 8 <= 0x7FFFFFFF, "lp_fp4_to_fp8_amax: too many tiles");
-    dim3 grid((unsigned)(per_xcd * 8)), block(256);
+    dim3 grid((unsigned)(per_xcd * 8)), block(kAmaxThreads);
     hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(MODE)                                                                                                   \
     do {                                                                                                               \
         if (bf16_out)                                                                                                  \
-            hipLaunchKernelGGL((fp4_amax<MODE, true>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
+            hipLaunchKernelGGL((fp4_amax<MODE, true, kAmaxThreads>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
                                cols, supers_c, n_supers, per_xcd, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,   \
                                scale_dtype, (uint16_t *)bf16_out);                                                      \
         else                                                                                                           \
-            hipLaunchKernelGGL((fp4_amax<MODE, false>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
+            hipLaunchKernelGGL((fp4_amax<MODE, false, kAmaxThreads>), grid, block, 0, st, (const uint8_t *)packed, (const uint8_t *)scale, \
                                cols, supers_c, n_supers, per_xcd, amax_floor, zero_rule, (uint8_t *)q_out, scale_out,   \
                                scale_dtype, (uint16_t *)bf16_out);                                                      \
     } while (0)
