@@ -377,7 +377,15 @@ def main():
             by = touched * N4 * K4 + Mt * K4 + Mt * N4 * 2
             res4[name] = {"ms": ms4, "tflops": fl / ms4 / 1e9, "mfma_frac": fl / ms4 / 1e9 / FP8_PEAK_TFLOPS,
                           "hbm_floor_GB": by / 1e9, "hbm_frac_of_floor": by / ms4 / 1e6 / HBM_PEAK_GBS}
-            del x4q, x4s, w4q, w4s, c4
+            # the same problem with power-of-two (e8m0) scales, which the matrix cores apply themselves: the codes
+            # in place are kept (timing does not depend on their values), only the scale tables change type
+            x4s8 = torch.randint(118, 128, (Mt, K4 // 128), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+            w4s8 = torch.randint(110, 120, (E4 * N4 // 128, K4 // 128), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+            fn8 = lambda: chk(L.lp_gemm_fp8_grouped(x4q.data_ptr(), x4s8.data_ptr(), w4q.data_ptr(), w4s8.data_ptr(), A.E8M0,  # noqa: E731
+                                                    offs_d.data_ptr(), E4, Mt, N4, K4, c4.data_ptr(), A.BF16, stream()))
+            ms48, _ = time_launches([fn8], 5, 2)
+            res4[name + "_e8m0_scales"] = {"ms": ms48, "tflops": fl / ms48 / 1e9, "mfma_frac": fl / ms48 / 1e9 / FP8_PEAK_TFLOPS}
+            del x4q, x4s, w4q, w4s, c4, x4s8, w4s8
             torch.cuda.empty_cache()
         extras["c4_grouped_gemm"] = res4
 
