@@ -354,7 +354,10 @@ def main():
         offs_d = offs.to(dev)
         Mt = int(offs[-1])
         res4 = {"m_splits_max": int(m_splits.max()), "m_splits_min": int(m_splits.min()),
-                "m_splits_zero": int((m_splits == 0).sum()), "rows": Mt}
+                "m_splits_zero": int((m_splits == 0).sum()), "rows": Mt,
+                "m_splits_histogram": {f"<={hi}": int(((m_splits > lo) & (m_splits <= hi)).sum())
+                                       for lo, hi in ((-1, 0), (0, 64), (64, 128), (128, 256), (256, 512), (512, 1024),
+                                                      (1024, 2048), (2048, 4096), (4096, 8192))}}
         for name, (N4, K4) in (("gate_up", (4096, 7168)), ("down", (7168, 2048))):
             x4 = randn(Mt, K4)
             x4q = torch.empty(Mt, K4, dtype=torch.uint8, device=dev)
