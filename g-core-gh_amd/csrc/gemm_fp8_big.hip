@@ -490,34 +490,41 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
 {
     constexpr int NT = TM * 2;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB>::LDS_BYTES];
-    __shared__ int scan[NT];
+    __shared__ int wave_total[NT / 64];
     __shared__ int found_e, found_first;
     int64_t gmt, tn;
     const bool in_range = gemm::tile_coords(blockIdx.x, max_mtiles, tiles_n, gmt, tn, true, gridDim.x);
     const int t = threadIdx.x;
     if (t == 0) found_e = -1;
-    __syncthreads();
     auto tiles_of = [](int rows) -> int {
         if (PART == 1) return rows / TM;
         if (PART == 2) rows %= 256;
         return (rows + TM - 1) / TM;
     };
+    // Which expert owns row tile gmt: a prefix sum over the experts' tile counts, NT experts at a time -- inside a
+    // wave by shuffles, across the waves through their totals (two barriers per NT experts).
     int base = 0;
     for (int e0 = 0; e0 < E; e0 += NT) {
         const int e = e0 + t;
-        int cnt = 0;
-        if (e < E) cnt = tiles_of(m_offsets[e + 1] - m_offsets[e]);
-        scan[t] = cnt;
-        __syncthreads();
-        for (int off = 1; off < NT; off <<= 1) {
-            int v = t >= off ? scan[t - off] : 0;
-            __syncthreads();
-            scan[t] += v;
-            __syncthreads();
+        const int cnt = e < E ? tiles_of(m_offsets[e + 1] - m_offsets[e]) : 0;
+        int incl = cnt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off);
+            if ((t & 63) >= off) incl += up;
         }
-        const int incl = base + scan[t], excl = incl - cnt;
-        if (in_range && e < E && gmt >= excl && gmt < incl) { found_e = e; found_first = excl; }
-        base += scan[NT - 1];
+        if ((t & 63) == 63) wave_total[t >> 6] = incl;
+        __syncthreads();                                       // also orders found_e = -1 before the write below
+        int before = base, all = 0;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) {
+            const int v = wave_total[w];
+            if (w < (t >> 6)) before += v;
+            all += v;
+        }
+        incl += before;
+        if (in_range && e < E && gmt >= incl - cnt && gmt < incl) { found_e = e; found_first = incl - cnt; }
+        base += all;
         __syncthreads();
     }
     if (!in_range || found_e < 0) return;
