@@ -270,10 +270,12 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ w
     }
 }
 
-// how many K ranges to use: aim at >= 2 workgroups per CU (256 CUs)
+// how many K ranges to use: aim at >= 2 workgroups per CU (256 CUs).  Only for few tiles: from about 96 tiles on
+// the hand-scheduled 128 x 128 kernel (which splits K inside the workgroup) is ahead of this kernel pair
+// (measured at K = 7168: 64 tiles 26 us against 37, 96 tiles 44 against 37, 192 tiles 63 against 37).
 int choose_splits(int64_t tiles, int64_t kblocks)
 {
-    if (tiles >= 256 || kblocks < 8) return 1;
+    if (tiles > 80 || kblocks < 8) return 1;
     int64_t s = (512 + tiles - 1) / tiles;
     if (s > kblocks / 4) s = kblocks / 4;     // keep >= 4 K steps per range
     if (s > 16) s = 16;
@@ -489,7 +491,10 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     static const bool force_small = getenv("LP_GEMM_FORCE_SMALL") != nullptr;
     static const char *force_tn = getenv("LP_GEMM_TN");
     const int esz = out_dtype == LP_BF16 ? 2 : 4, ssz = scale_dtype == LP_F32 ? 4 : 1;
-    if (!force_small && M >= 192 && tiles_m * tiles_n >= 800) {
+    // From 800 tiles of 128 x 128 on, and already above the 512 that fit the chip at once when the 256-row tiles
+    // still fit one round (576 tiles at K = 7168: 126 us as 128-tiles in two rounds, ~105 us as 144 big tiles).
+    const int64_t small_tiles = tiles_m * tiles_n, big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    if (!force_small && M >= 192 && (small_tiles >= 800 || (small_tiles > 512 && big_tiles <= 256))) {
         if (force_tn) return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, atoi(force_tn), st);
         const int64_t bm = (M + 255) / 256, bn = (N + 255) / 256, tiles = bm * bn;
         const int64_t full = tiles / 256, rem = tiles % 256;

@@ -631,9 +631,11 @@ int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *B
     const int64_t tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
-    // About one tile per CU or fewer: split K inside the workgroup (needs whole scale groups of 512 in each half)
+    // At most one tile per CU: split K inside the workgroup (needs whole scale groups of 512 in each half).  With
+    // more tiles than CUs the 512-thread workgroups would need a second round where 256-thread ones share the CUs
+    // (288 tiles at K = 7168: 90 us with the split against 60 without).
     static const char *dual_env = getenv("LP_GEMM_MID_DUAL");        // tuning aid: 0 / 1 forces it off / on
-    const bool dual = K % 1024 == 0 && (dual_env ? atoi(dual_env) != 0 : tiles_m * tiles_n <= 320);
+    const bool dual = K % 1024 == 0 && (dual_env ? atoi(dual_env) != 0 : tiles_m * tiles_n <= 256);
     static const char *deep_env = getenv("LP_GEMM_MID_STAGES");      // tuning aid: 4 forces the four-stage loop, 2 forbids it
     const bool four = deep_env ? atoi(deep_env) == 4 : false;
     if (four) {
@@ -667,7 +669,7 @@ int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *B
     // With two K blocks per stage a workgroup keeps twice the bytes in flight but owns the CU's LDS alone:
     // better while there is at most about one tile per CU, worse when two workgroups could share a CU.
     static const char *force = getenv("LP_GEMM_MID_KSUB");           // tuning aid
-    const bool deep = force ? atoi(force) == 2 : tiles_m * tiles_n <= 320;
+    const bool deep = force ? atoi(force) == 2 : tiles_m * tiles_n <= 256;
     if (deep)
         hipLaunchKernelGGL((gemm_asm<128, 128, 2>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
                            (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
