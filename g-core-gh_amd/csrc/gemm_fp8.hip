@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ w
 // (measured at K = 7168: 64 tiles 26 us against 37, 96 tiles 44 against 37, 192 tiles 63 against 37).
 int choose_splits(int64_t tiles, int64_t kblocks)
 {
-    if (tiles > 80 || kblocks < 8) return 1;
+    if (tiles > 80 || kblocks < 32) return 1;                 // short K: the second launch costs more than the split gains
     int64_t s = (512 + tiles - 1) / tiles;
     if (s > kblocks / 4) s = kblocks / 4;     // keep >= 4 K steps per range
     if (s > 16) s = 16;
@@ -366,7 +366,8 @@ extern "C" int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 
 static int64_t split_bytes(int64_t M, int64_t N, int64_t K)
 {
-    if (M <= 64) {
+    static const bool skinny = getenv("LP_GEMM_SKINNY") != nullptr && getenv("LP_GEMM_NO_SKINNY") == nullptr;
+    if (M <= 64 && skinny) {
         int sp, per;
         gemm::skinny_plan(N, K, sp, per);
         if (per <= gemm::kSkinnyBlocks) return gemm::skinny_workspace_bytes(N, sp);
@@ -397,7 +398,7 @@ static int launch_small(const void *Aq, const void *As, const void *Bq, const vo
                         int64_t N, int64_t K, void *C, int64_t ldc, int out_dtype, hipStream_t st)
 {
     static const char *mid_min = getenv("LP_GEMM_MID_MIN_M");       // tuning aid
-    if (M >= (mid_min ? atoi(mid_min) : 64) && gemm::mid_asm_ok(As, Bs, scale_dtype, M, N, K))
+    if (M >= (mid_min ? atoi(mid_min) : 1) && gemm::mid_asm_ok(As, Bs, scale_dtype, M, N, K))
         return gemm::launch_mid_asm(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, ldc, out_dtype, st);
     const int64_t tiles_m = (M + TM - 1) / TM, tiles_n = N / TN;
     const int64_t grid = padded_grid(tiles_m, tiles_n);
@@ -451,7 +452,9 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
         return lp_gemm_fp8_block(Aq, fa, Bq, fb, LP_F32, M, N, K, C, out_dtype, (char *)workspace + sc_bytes,
                                  workspace_bytes - sc_bytes, stream);
     }
-    static const bool no_skinny = getenv("LP_GEMM_NO_SKINNY") != nullptr;       // tuning aid
+    // The K-split weight-streaming kernel pair is opt-in (LP_GEMM_SKINNY=1): on every decode shape measured since
+    // the single-launch kernels above and the 128-row tile kernel exist it is level with them or behind (two launches).
+    static const bool no_skinny = getenv("LP_GEMM_SKINNY") == nullptr || getenv("LP_GEMM_NO_SKINNY") != nullptr;
     static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;           // tuning aid
     if (!no_thin && gemm::thin_ok(M, N, K)) return gemm::launch_thin(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, st);
     if (M <= 64 && !no_skinny) {

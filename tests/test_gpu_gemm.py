@@ -341,3 +341,32 @@ def test_grouped_linear_backward(G, m_splits):
     out2 = lin(x2, (wq, ws), m_splits)
     out2.backward(g)
     assert torch.equal(out2, out) and torch.equal(x2.grad, x.grad)
+
+
+def test_gemm_skinny_pair_opt_in():
+    """The K-split weight-streaming kernel pair is no longer chosen by default; LP_GEMM_SKINNY=1 selects it (the
+    switch is read once per process, hence the child process).  Decode shapes with caller workspace, against the
+    fp32 dequantise-then-matmul reference, to the path's tolerance."""
+    import os
+    import subprocess
+    import sys
+    say("gemm skinny pair (LP_GEMM_SKINNY=1, child process)")
+    code = r'''
+import sys, torch
+import gcore_lowp as G
+torch.manual_seed(3)
+for (M, N, K) in ((8, 2048, 7168), (33, 4096, 14336), (64, 1536, 3584), (16, 4096, 7168)):
+    a = torch.randn(M, K, device="cuda"); b = torch.randn(N, K, device="cuda") * 0.02
+    aq, as_ = G.quant_1d(a); bq, bs = G.quant_2d(b)
+    print("[case] skinny", M, N, K, flush=True)
+    c = G.gemm_fp8_block_scaling_impl(aq, as_, bq, bs)
+    ref = (aq.float() * as_.repeat_interleave(128, 1)) @ (bq.float() * bs.repeat_interleave(128, 0).repeat_interleave(128, 1)).t()
+    err = (c.float() - ref).abs().max().item() / ref.abs().max().item()
+    cos = torch.nn.functional.cosine_similarity(c.float().flatten(), ref.flatten(), dim=0).item()
+    assert err <= 2e-2 and cos >= 0.9999, (M, N, K, err, cos)
+print("ok")
+'''
+    env = dict(os.environ, LP_GEMM_SKINNY="1", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    env.pop("LP_GEMM_NO_SKINNY", None)
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=200)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-1500:], r.stderr[-1500:])
