@@ -214,6 +214,28 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
         [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies)
 
+// Index arithmetic of the staged bf16 epilogue for a wave tile of 64 rows x COLS columns (COLS = 128, 96 or 64).
+// A row of the staging region holds COLS bf16 plus 16 bytes of padding (rows then start 4 banks apart: the 8-byte
+// writes of 16 rows spread over the banks instead of hitting the same ones).  Written per accumulator block
+// (mb, nb) by lane (l16, lq): row mb * 16 + l16, columns nb * 16 + 4 lq .. + 3.  Read back in 16-byte chunks of 8
+// columns: LPR lanes cover a row, 64 / LPR rows per pass.  The same formulas are restated on the host and checked to
+// cover every element exactly once and to stay inside the region.
+template <int COLS>
+struct StagedEpilogue {
+    static constexpr int PITCH = COLS * 2 + 16;
+    static constexpr int WAVE_BYTES = 64 * PITCH;
+    static constexpr int CHUNKS = COLS / 8;                       // 16-byte chunks per row
+    static constexpr int LPR = CHUNKS > 8 ? 16 : 8;               // lanes per row when reading (a power of two >= CHUNKS)
+    static constexpr int PASSES = 64 / (64 / LPR);
+    __host__ __device__ static constexpr int write_offset(int mb, int nb, int l16, int lq)
+    {
+        return (mb * 16 + l16) * PITCH + (nb * 16 + 4 * lq) * 2;
+    }
+    __host__ __device__ static constexpr int read_row(int pass, int lane) { return pass * (64 / LPR) + lane / LPR; }
+    __host__ __device__ static constexpr int read_chunk(int lane) { return lane % LPR; }
+    __host__ __device__ static constexpr int read_offset(int row, int chunk) { return row * PITCH + chunk * 16; }
+};
+
 template <int TM, int TN, int KSUB, int NST = 2>
 struct AsmTile {
     static constexpr int WAVES = TM / 64 * 2, NBW = TN / 32;
@@ -231,7 +253,11 @@ struct AsmTile {
 // BROW: the weights carry an e8m0 scale per row and K block ([N, K/128] bytes) instead of per 128 rows; the matrix
 // instruction takes a scale per operand row anyway, so the loop only fetches them differently (hardware-scaled
 // 128 x 128 loop: waves 2 and 3 copy the weight-scale dwords of a group while waves 0 and 1 copy the activations').
-template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false>
+// STAGED: bf16 results leave through LDS, so that a store instruction writes 16 bytes per lane and whole runs of a row
+// (4 rows x 256 contiguous bytes for a 128-column wave tile) instead of 16 rows x 32 bytes.  Each wave turns its own
+// 64-row sub-tile in a region of its own (the stage memory, free after the loop), so only the barrier that ends the
+// loop's use of that memory is needed.  Used by the dense kernels only.
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
@@ -416,6 +442,36 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             for (int r = 0; r < 16; ++r) accs[nb][r] += o[r];
         }
     }
+    if constexpr (STAGED) {
+        static_assert(!DUAL, "the staged epilogue shares no LDS with the K-split reduction");
+        using E = StagedEpilogue<TN / 2>;
+        static_assert(WAVES * E::WAVE_BYTES <= T::LDS_BYTES, "the waves' staging regions must fit the tile's LDS");
+        if (out_dtype == LP_BF16) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this wave's last fragment reads
+            __syncthreads();                                          // every wave is done with the stage memory
+            uint8_t *stage = smem + wave * E::WAVE_BYTES;
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) {
+#pragma unroll
+                for (int nb = 0; nb < NBW; ++nb) {
+                    const u32x2 o = {pack_bf16(accs[nb][mb * 4], accs[nb][mb * 4 + 1]), pack_bf16(accs[nb][mb * 4 + 2], accs[nb][mb * 4 + 3])};
+                    *(u32x2 *)(stage + E::write_offset(mb, nb, l16, lq)) = o;
+                }
+            }
+            __syncthreads();
+            const int64_t row_base = m0 + wm * 64;
+#pragma unroll
+            for (int p = 0; p < E::PASSES; ++p) {
+                const int row = E::read_row(p, lane), chunk = E::read_chunk(lane);
+                const int64_t n = wcol0 + chunk * 8;
+                if (chunk < E::CHUNKS && row_base + row < M && n < N) {
+                    const u32x4 v = *(const u32x4 *)(stage + E::read_offset(row, chunk));
+                    *(u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n) = v;
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
         if (arow[mb] >= M) continue;
@@ -445,7 +501,7 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
     __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<TM, TN, KSUB, NST>::LDS_BYTES];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<TM, TN, KSUB, HWS, false, NST>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+    tile_asm<TM, TN, KSUB, HWS, false, NST, false, true>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
 }
 
 // 128 x 128 tile with the K split inside the workgroup (see tile_asm): 8 waves, two sets of LDS stages.
