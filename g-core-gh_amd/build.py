@@ -61,6 +61,18 @@ def _generate():
         subprocess.check_call([sys.executable, gen])
 
 
+def _audit_asm_operands():
+    """The hand-scheduled GEMM loops keep their addresses in asm operands: fail the build if the compiler placed
+    one of them in a register a loop writes (csrc/check_asm_operands.py)."""
+    sys.path.insert(0, CSRC)
+    try:
+        import check_asm_operands
+    finally:
+        sys.path.pop(0)
+    if check_asm_operands.audit(quiet=True) != 0:
+        raise RuntimeError("gemm_fp8_big.hip: an asm operand shares a register with the loop it feeds; not linking")
+
+
 def build(force: bool = False) -> str:
     _generate()
     os.makedirs(OBJ, exist_ok=True)
@@ -68,6 +80,7 @@ def build(force: bool = False) -> str:
     with ThreadPoolExecutor(max_workers=min(8, len(sources()))) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), sources()))
     if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
+        _audit_asm_operands()
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:

@@ -200,7 +200,7 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
 // expert's row range), weight rows n0 .. n0 + TN - 1 of the matrix at Bq / Bs.  Waves are laid out
 // (TM / 64) x 2; a wave owns 64 rows x TN / 2 columns.
 #define LP_ASM_CLOBBERS                                                                                                   \
-    "memory", "scc", "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43",    \
+    "memory", "scc", "m0", "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43",    \
         "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59",   \
         "v60", "v61", "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75",   \
         "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91",   \
@@ -256,7 +256,16 @@ struct AsmTile {
 // STAGED: bf16 results leave through LDS, so that a store instruction writes 16 bytes per lane and whole runs of a row
 // (4 rows x 256 contiguous bytes for a 128-column wave tile) instead of 16 rows x 32 bytes.  Each wave turns its own
 // 64-row sub-tile in a region of its own (the stage memory, free after the loop), so only the barrier that ends the
-// loop's use of that memory is needed.  Used by the dense kernels only.
+// loop's use of that memory is needed.  Not used with DUAL (its reduction owns the LDS at that point).
+//
+// Register contract of the asm statements: the loops name v30 .. v255, s40 .. s77 and m0 literally and keep their
+// operands (addresses, offsets, counts) live to the end.  Accumulator outputs are therefore early-clobber ("=&"):
+// without it the compiler may hand an operand the same register as an output -- the loop zeroes and accumulates into
+// it and then loads from a wild offset.  m0 is on the clobber list so that no m0 set-up of the compiler's is assumed
+// to survive the loop (clang warns about reserved registers on a clobber list; that is the intent here).
+// check_asm_operands.py verifies both on the generated assembly at build time.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
@@ -349,8 +358,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
         asm volatile(
 #include "gemm_big_hw_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
-              "={v[192:207]}"(acc4), "={v[208:223]}"(acc5), "={v[224:239]}"(acc6), "={v[240:255]}"(acc7)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -359,7 +368,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid_hwrow_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS, [sdst] "s"(sdst), [srdb] "v"(srdb)
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -367,7 +376,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid4_hw_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -375,7 +384,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid4_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -383,7 +392,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid_hw_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -391,8 +400,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
         asm volatile(
 #include "gemm_big_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
-              "={v[192:207]}"(acc4), "={v[208:223]}"(acc5), "={v[224:239]}"(acc6), "={v[240:255]}"(acc7)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -401,8 +410,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5;
         asm volatile(
 #include "gemm_big192_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3),
-              "={v[192:207]}"(acc4), "={v[208:223]}"(acc5)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5)
             : LP_ASM_INPUTS, [bsptr2] "s"(bs2_u), [sel1] "s"(sel1), [sel2] "s"(sel2)
             : LP_ASM_CLOBBERS, "v224", "v225", "v226", "v227", "v228", "v229", "v230", "v231", "s64", "s65", "s66", "s67",
               "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77");
@@ -411,7 +420,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -419,7 +428,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
 #include "gemm_mid2_loop.inc"
-            : "={v[128:143]}"(acc0), "={v[144:159]}"(acc1), "={v[160:175]}"(acc2), "={v[176:191]}"(acc3)
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
             : LP_ASM_INPUTS
             : LP_ASM_CLOBBERS);
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -491,6 +500,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     }
 }
 
+#pragma clang diagnostic pop
 
 template <int TM, int TN, int KSUB, bool HWS = false, int NST = 2>
 __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
@@ -526,7 +536,7 @@ __global__ __launch_bounds__(256) void gemm_asm_rowscale(const uint8_t *__restri
     __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<128, 128, 1>::LDS_BYTES + 4096];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<128, 128, 1, true, false, 2, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
+    tile_asm<128, 128, 1, true, false, 2, true, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
@@ -589,7 +599,7 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
     const int64_t first = PART == 2 ? row_begin + (row_end - row_begin) / 256 * 256 : row_begin;
     const int64_t kblocks = K / KB;
     const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
-    tile_asm<TM, TN, KSUB, HWS>(smem, Aq, As, Bq + (int64_t)e * N * K, bs_e, first + (gmt - found_first) * TM, row_end,
+    tile_asm<TM, TN, KSUB, HWS, false, 2, false, true>(smem, Aq, As, Bq + (int64_t)e * N * K, bs_e, first + (gmt - found_first) * TM, row_end,
                                 tn * TN, N, K, C, N, out_dtype);
 }
 

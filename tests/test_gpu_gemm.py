@@ -288,11 +288,15 @@ def test_gemm_rowscale(G, shape):
     b = I.act_like(N, K, 4) * 0.05
     aq, a_s = T.quant_fp8_e4m3_scale_e8m0(a, (1, 128))
     bq, b_s = T.quant_fp8_e4m3_scale_e8m0(b, (1, 128))
-    out = torch.empty(M, N, dtype=torch.float32, device="cuda")
-    G.gemm_fp8_rowscale(aq.view(torch.uint8).cuda(), a_s.view(torch.uint8).cuda(), bq.view(torch.uint8).cuda(),
-                        b_s.view(torch.uint8).cuda(), M, N, K, out)
     ref = (T.dequant_act_f32(aq.cuda(), a_s.float().cuda()) @ T.dequant_act_f32(bq.cuda(), b_s.float().cuda()).T)
-    check(out, ref, f"rowscale {shape}")
+    outs = {}
+    for dt in (torch.float32, torch.bfloat16):           # bf16 leaves through the LDS-staged epilogue
+        out = torch.full((M, N), float("nan"), dtype=dt, device="cuda")
+        G.gemm_fp8_rowscale(aq.view(torch.uint8).cuda(), a_s.view(torch.uint8).cuda(), bq.view(torch.uint8).cuda(),
+                            b_s.view(torch.uint8).cuda(), M, N, K, out)
+        check(out, ref, f"rowscale {shape} {dt}")
+        outs[dt] = out
+    assert torch.equal(outs[torch.bfloat16], outs[torch.float32].to(torch.bfloat16)), "bf16 output is the rounded fp32 output"
 
 
 @pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200], [2048, 1024, 0, 4096]],
