@@ -10,9 +10,10 @@
 // One workgroup (256 threads) = 128 rows x 128 columns.  A thread owns 8 consecutive rows x 8 consecutive columns
 // (16 lanes cover the 256 bytes of a row, all 8 row loads are issued before anything else); the column amax goes
 // thread -> the 4 lanes of a wave that share the columns (two shuffles) -> the 4 waves (1 KB of LDS, one barrier);
-// every thread then holds the scales of its 8 columns, quantises, and writes, per column, its 8 codes (8 consecutive
-// rows = 8 contiguous bytes of the transposed output) directly: the 16 threads that share a column fill its 128-byte
-// line between them, so no transposing pass through LDS is needed.
+// every thread then holds the scales of its 8 columns and quantises; per column its 8 codes (8 consecutive rows = 8
+// contiguous bytes of the transposed output) go to a 16 KB LDS tile [column][row], swizzled so that neither side has
+// bank conflicts, and leave from there as whole 128-byte lines, 16 bytes per lane (measured 5-13 % faster than letting
+// the 16 threads of 4 waves that share a line store 8 bytes each).  A block that is padding only loads nothing.
 #include "lowp_device.h"
 
 using namespace lowp;
@@ -30,12 +31,13 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     // which expert owns padded block `blk`: thread t counts the blocks of experts t, t + 256, ..., a prefix sum over the
     // workgroup (wave shuffles, then the four wave totals through LDS) finds the one whose range holds blk
     __shared__ int wave_total[4];
-    __shared__ int hit_e, hit_pb;
+    __shared__ int hit_e, hit_pb, hit_rb, hit_re;
     if (t == 0) hit_e = -1;
     int64_t pb = 0;
     for (int e0 = 0; e0 < E; e0 += 256) {
         const int ee = e0 + t;
-        const int cnt = ee < E ? (m_offsets[ee + 1] - m_offsets[ee] + pad_rows - 1) / pad_rows * (pad_rows >> 7) : 0;
+        const int rb = ee < E ? m_offsets[ee] : 0, re = ee < E ? m_offsets[ee + 1] : 0;
+        const int cnt = (re - rb + pad_rows - 1) / pad_rows * (pad_rows >> 7);
         int incl = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -51,15 +53,14 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
             chunk += wave_total[w];
         }
         const int64_t end = pb + before + incl;           // blocks up to and including this expert
-        if (cnt > 0 && blk >= end - cnt && blk < end) { hit_e = ee; hit_pb = (int)(end - cnt); }
+        if (cnt > 0 && blk >= end - cnt && blk < end) { hit_e = ee; hit_pb = (int)(end - cnt); hit_rb = rb; hit_re = re; }
         pb += chunk;
         __syncthreads();
         if (hit_e >= 0 || blk < pb) break;                // uniform: both read after the barrier
     }
     if (hit_e < 0) return;
-    const int e = hit_e;
     pb = hit_pb;
-    const int r_begin = m_offsets[e], r_end = m_offsets[e + 1];
+    const int r_begin = hit_rb, r_end = hit_re;
     const int nblk = (r_end - r_begin + pad_rows - 1) / pad_rows * (pad_rows >> 7);
     const int lb = (int)(blk - pb);                      // block inside the expert
     const int64_t r0 = (int64_t)r_begin + (int64_t)lb * 128;
@@ -67,13 +68,17 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
 
     // ---- loads: row rg * 8 + i, columns c0 + 8 cc .. + 7; rows past the expert's end repeat its last row and
     // are zeroed afterwards (no branch between the loads)
-    float v[8][8];
+    // The loaded words stay as they are; bf16 pairs are unpacked where they are used (32 registers instead of 64 live
+    // across the barrier: five workgroups per CU instead of four).
+    constexpr int W = IS_BF16 ? 4 : 8;
+    uint32_t rw[8][W];
     {
-        u32x4 raw[8][IS_BF16 ? 1 : 2];
+        u32x4 raw[8][IS_BF16 ? 1 : 2] = {};
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
+            if (valid == 0) break;                        // uniform over the workgroup
             const int row = rg * 8 + i;
-            const int64_t r = valid > 0 ? r0 + (row < valid ? row : valid - 1) : r_begin;
+            const int64_t r = r0 + (row < valid ? row : valid - 1);
             if (IS_BF16) {
                 raw[i][0] = __builtin_nontemporal_load((const u32x4 *)((const uint16_t *)x + r * cols + c0 + cc * 8));
             } else {
@@ -86,14 +91,13 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
         for (int i = 0; i < 8; ++i) {
             const bool live = rg * 8 + i < valid;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                uint32_t b;
-                if (IS_BF16) b = (j & 1) ? raw[i][0][j >> 1] & 0xFFFF0000u : raw[i][0][j >> 1] << 16;
-                else b = raw[i][(j >> 2) & (IS_BF16 ? 0 : 1)][j & 3];
-                v[i][j] = u2f(live ? b : 0u);
-            }
+            for (int k = 0; k < W; ++k) rw[i][k] = live ? raw[i][k >> 2][k & 3] : 0u;
         }
     }
+    auto elem = [&](int i, int j) -> float {
+        if (IS_BF16) return u2f((j & 1) ? rw[i][(j >> 1) & 3] & 0xFFFF0000u : rw[i][(j >> 1) & 3] << 16);
+        return u2f(rw[i][j & (W - 1)]);
+    };
     // ---- column maxima of |x| as integers on the sign-cleared bits (inf / NaN sort above every finite value)
     uint32_t m[8];
 #pragma unroll
@@ -101,7 +105,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
         uint32_t a = 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t b = f2u(v[i][j]) & 0x7FFFFFFFu;
+            const uint32_t b = f2u(elem(i, j)) & 0x7FFFFFFFu;
             a = b > a ? b : a;
         }
         // lanes l, l ^ 16, l ^ 32, l ^ 48 hold the same columns
@@ -115,6 +119,14 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
         wave_max[wave][cc][1] = u32x4{m[4], m[5], m[6], m[7]};
     }
     __syncthreads();
+    if (IS_BF16) {
+        // opaque to the compiler: what was unpacked for the maxima is not kept, the codes unpack again from these words
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) asm volatile("" : "+v"(rw[i][k]));
+        }
+    }
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
         const u32x4 a = wave_max[w][cc][0], b = wave_max[w][cc][1];
@@ -127,6 +139,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     // ---- scales, codes, stores
     const int64_t P = (int64_t)nblk * 128;
     const int64_t base = cols * pb * 128;                // codes of the experts before this one
+    __shared__ __attribute__((aligned(16))) u32x2 turned[128 * 16];      // [column][16 groups of 8 rows], groups XOR-swizzled by column chunk
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const bool special = m[j] >= 0x7F800000u;        // inf or NaN in the block: literal arithmetic
@@ -139,20 +152,28 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
             lo = hi = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                lo |= (uint32_t)quant_slow<LP_SCALE_POW2>(v[i][j], bs) << (8 * i);
-                hi |= (uint32_t)quant_slow<LP_SCALE_POW2>(v[4 + i][j], bs) << (8 * i);
+                lo |= (uint32_t)quant_slow<LP_SCALE_POW2>(elem(i, j), bs) << (8 * i);
+                hi |= (uint32_t)quant_slow<LP_SCALE_POW2>(elem(4 + i, j), bs) << (8 * i);
             }
         } else {
             const float f = u2f((uint32_t)(127 - bs.exp2) << 23);        // 2^-e, exact: |e| <= 126 for finite amax
             const bool tiny = bs.exp2 < -126 || bs.exp2 > 126;
             float y[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) y[i] = clamp448(tiny ? ldexpf(v[i][j], -bs.exp2) : v[i][j] * f);
+            for (int i = 0; i < 8; ++i) y[i] = clamp448(tiny ? ldexpf(elem(i, j), -bs.exp2) : elem(i, j) * f);
             lo = cvt4(y[0], y[1], y[2], y[3]);
             hi = cvt4(y[4], y[5], y[6], y[7]);
         }
-        // plain store: the 16 threads that share this 128-byte line sit in 4 waves, and L2 puts the pieces together
-        *(u32x2 *)(qT + base + c * P + (int64_t)lb * 128 + rg * 8) = u32x2{lo, hi};
+        turned[(cc * 8 + j) * 16 + (rg ^ cc)] = u32x2{lo, hi};
+    }
+    // 8 lanes write the 128 bytes of a column's line, 16 bytes each: a store instruction of a wave covers 8 whole lines
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int col = p * 32 + (t >> 3), pair = t & 7, sw = (col >> 3) & 15;
+        const u32x4 raw = *(const u32x4 *)&turned[col * 16 + ((pair ^ (sw >> 1)) << 1)];
+        const u32x4 out = (sw & 1) ? u32x4{raw[2], raw[3], raw[0], raw[1]} : raw;
+        *(u32x4 *)(qT + base + (c0 + col) * P + (int64_t)lb * 128 + pair * 16) = out;
     }
 }
 
