@@ -256,7 +256,7 @@ struct AsmTile {
 // STAGED: bf16 results leave through LDS, so that a store instruction writes 16 bytes per lane and whole runs of a row
 // (4 rows x 256 contiguous bytes for a 128-column wave tile) instead of 16 rows x 32 bytes.  Each wave turns its own
 // 64-row sub-tile in a region of its own (the stage memory, free after the loop), so only the barrier that ends the
-// loop's use of that memory is needed.  Not used with DUAL (its reduction owns the LDS at that point).
+// loop's use of that memory is needed.  With DUAL it follows the reduction, in the first K half's stage memory.
 //
 // Register contract of the asm statements: the loops name v30 .. v255, s40 .. s77 and m0 literally and keep their
 // operands (addresses, offsets, counts) live to the end.  Accumulator outputs are therefore early-clobber ("=&"):
@@ -452,12 +452,16 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         }
     }
     if constexpr (STAGED) {
-        static_assert(!DUAL, "the staged epilogue shares no LDS with the K-split reduction");
         using E = StagedEpilogue<TN / 2>;
         static_assert(WAVES * E::WAVE_BYTES <= T::LDS_BYTES, "the waves' staging regions must fit the tile's LDS");
         if (out_dtype == LP_BF16) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this wave's last fragment reads
-            __syncthreads();                                          // every wave is done with the stage memory
+            // DUAL: only the first K half's waves are left; they stage in their own half's stage memory, which every
+            // one of them left before the reduction's barriers (the reduction itself used the other half's), so no
+            // barrier is needed -- and none is wanted, the other four waves have ended.
+            if constexpr (!DUAL) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // this wave's last fragment reads
+                __syncthreads();                                      // every wave is done with the stage memory
+            }
             uint8_t *stage = smem + wave * E::WAVE_BYTES;
 #pragma unroll
             for (int mb = 0; mb < 4; ++mb) {
@@ -467,7 +471,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
                     *(u32x2 *)(stage + E::write_offset(mb, nb, l16, lq)) = o;
                 }
             }
-            __syncthreads();
+            if constexpr (DUAL) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave reads back only what it wrote
+            else __syncthreads();
             const int64_t row_base = m0 + wm * 64;
 #pragma unroll
             for (int p = 0; p < E::PASSES; ++p) {
@@ -524,7 +529,7 @@ __global__ __launch_bounds__(512) void gemm_asm_dual(const uint8_t *__restrict__
     __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * AsmTile<128, 128, KSUB>::LDS_BYTES];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<128, 128, KSUB, HWS, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
+    tile_asm<128, 128, KSUB, HWS, true, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
 // 128 x 128 tiles, e8m0 scales per row and K block on both operands (the weight-gradient GEMM of the grouped linear).

@@ -89,6 +89,25 @@ def test_gemm_dense(G, shape, pow2):
     check(out, ref_gemm(xq, xs, wq, ws), f"dense {shape}")
 
 
+@pytest.mark.parametrize("shape", [(2048, 2048, 7168), (300, 2048, 1024), (129, 1280, 2560), (1000, 4096, 512), (513, 18432, 1024),
+                                   (2048, 18432, 512), (777, 4224, 1536), (257, 19200, 512), (64, 24576, 1536), (16, 4096, 2048)],
+                         ids=lambda s: "M%d_N%d_K%d" % s)
+@pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
+def test_gemm_bf16_output_is_the_rounded_fp32_output(G, shape, pow2):
+    """Every kernel rounds the same fp32 accumulators whichever way the result leaves (directly or as whole row runs
+    through LDS): the bf16 output equals the fp32 output rounded to nearest-even, element for element, and rows or
+    columns outside the problem are not written.  Shapes cover the K split inside a workgroup (<= 256 tiles), the
+    256-row kernels with ragged M and N and the decode kernels."""
+    M, N, K = shape
+    xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + N + K + 7, pow2=pow2)
+    say("gemm bf16 vs fp32 output", shape, "pow2" if pow2 else "f32")
+    args = (xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+    wide = G.gemm_fp8_block_scaling_impl(*args, out_dtype=torch.float32)
+    narrow = G.gemm_fp8_block_scaling_impl(*args)
+    assert narrow.dtype == torch.bfloat16 and wide.dtype == torch.float32
+    assert torch.equal(narrow, wide.to(torch.bfloat16)), (narrow.float() - wide).abs().max().item()
+
+
 def test_gemm_small_exact_vs_c_oracle(G, corc):
     """Small case against the double-precision scalar oracle, fp32 output: catches scale indexing
     (As[i, kb], Bs[j // 128, kb]) with distinct scales per block."""
