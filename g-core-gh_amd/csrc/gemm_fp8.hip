@@ -504,6 +504,7 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
         int64_t n_big = N;                                   // columns given to the big kernel
         if (full >= 1 && rem > 0 && rem < 160) n_big = (full * 256 / bm) * 256;
         if (n_big > N) n_big = N;
+        if (n_big > 0 && n_big < N && gemm::launch_mixed(Aq, As, Bq, Bs, scale_dtype, M, N, K, n_big, C, N, out_dtype, st, &rc)) return rc;
         if (n_big > 0) {
             rc = gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, n_big, K, C, N, out_dtype, 256, st);
             if (rc) return rc;

@@ -532,6 +532,32 @@ __global__ __launch_bounds__(512) void gemm_asm_dual(const uint8_t *__restrict__
     tile_asm<128, 128, KSUB, HWS, true, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
+// One launch for a problem split by columns: 256 x 256 tiles on weight rows [0, n_big) and K-split 128 x 128 tiles on the
+// rest (what gemm_asm<256, 256, 1> followed by gemm_asm_dual would do in two launches).  The big tiles come first in the
+// grid; a CU that has finished its last big tile goes on with the small ones, so the launch gap and the uneven end
+// of the big tiles' last round are not waited for.  grid_big is a multiple of 8, so both parts keep their XCD mapping.
+template <bool HWS>
+__global__ __launch_bounds__(512) void gemm_asm_mixed(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                      const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
+                                                      int64_t N, int64_t K, int64_t n_big, int64_t grid_big, void *__restrict__ C,
+                                                      int64_t ldc, int out_dtype)
+{
+    constexpr int LDS_BIG = AsmTile<256, 256, 1>::LDS_BYTES, LDS_DUAL = 2 * AsmTile<128, 128, 1>::LDS_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BIG > LDS_DUAL ? LDS_BIG : LDS_DUAL];
+    int64_t tm, tn;
+    if ((int64_t)blockIdx.x < grid_big) {
+        if (!gemm::tile_coords(blockIdx.x, (M + 255) / 256, n_big / 256, tm, tn)) return;
+        tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 256, M, tn * 256, n_big, K, C, ldc, out_dtype);
+    } else {
+        const int64_t n_small = N - n_big;
+        if (!gemm::tile_coords(blockIdx.x - grid_big, (M + 127) / 128, n_small / 128, tm, tn)) return;
+        const char *bs = (const char *)Bs + (n_big / 128) * (K / KB) * (HWS ? 1 : 4);
+        char *c = (char *)C + n_big * (out_dtype == LP_BF16 ? 2 : 4);
+        tile_asm<128, 128, 1, HWS, true, 2, false, true>(smem, Aq, As, Bq + n_big * K, (const float *)bs, tm * 128, M, tn * 128,
+                                                         n_small, K, c, ldc, out_dtype);
+    }
+}
+
 // 128 x 128 tiles, e8m0 scales per row and K block on both operands (the weight-gradient GEMM of the grouped linear).
 __global__ __launch_bounds__(256) void gemm_asm_rowscale(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
@@ -687,6 +713,32 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
     if (scale_dtype == LP_F32) GO(LP_F32);
     GO(LP_E8M0);
 #undef GO
+}
+
+// Columns [0, n_big) on 256 x 256 tiles and [n_big, N) on K-split 128 x 128 tiles in one launch; false when the shape does
+// not fit both loops (the caller then launches the two kernels one after the other).
+bool launch_mixed(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
+                  int64_t n_big, void *C, int64_t ldc, int out_dtype, hipStream_t st, int *rc)
+{
+    static const bool off = getenv("LP_GEMM_NO_ASM") != nullptr || getenv("LP_GEMM_NO_MID") != nullptr ||
+                            (getenv("LP_GEMM_MIXED") && atoi(getenv("LP_GEMM_MIXED")) == 0);
+    const int64_t n_small = N - n_big;
+    if (off || (scale_dtype != LP_F32 && scale_dtype != LP_E8M0) || n_big <= 0 || n_small <= 0 || n_big % 256 || n_small % 128 ||
+        K % 1024 || !asm_shape_ok(As, Bs, M, N, K, scale_dtype))
+        return false;
+    const int64_t small_tiles = ((M + 127) / 128) * (n_small / 128);
+    if (small_tiles > 256) return false;                               // the K split pays up to one tile per CU
+    const int64_t grid_big = gemm::padded_grid((M + 255) / 256, n_big / 256);
+    const int64_t grid = grid_big + gemm::padded_grid((M + 127) / 128, n_small / 128);
+    if (grid > 0x7FFFFFFF) return false;
+    if (scale_dtype == LP_E8M0)
+        hipLaunchKernelGGL((gemm_asm_mixed<true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, n_big, grid_big, C, ldc, out_dtype);
+    else
+        hipLaunchKernelGGL((gemm_asm_mixed<false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, n_big, grid_big, C, ldc, out_dtype);
+    *rc = check_launch("lp_gemm_fp8_block(asm mixed)");
+    return true;
 }
 
 // 128 x 128 tiles on the hand-scheduled loop: two workgroups share a CU, so one computes while the other waits.
