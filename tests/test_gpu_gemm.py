@@ -71,6 +71,8 @@ DENSE_SHAPES = [
     # between the 256 x 256 and the 128 x 128 kernel (576 tiles on 256 CUs)
     (333, 8320, 512), (200, 16384, 256), (2048, 4224, 384), (256, 32768, 128), (1000, 9216, 640),
     (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536), (32, 128, 7168), (48, 16384, 2048), (64, 2048, 7168),
+    # the column split in one launch (256 x 256 tiles, then K-split 128 x 128 tiles): K a multiple of 1024, ragged M
+    (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024),
     # at most 16 rows: one workgroup per 16 weight rows over the whole of K (ragged K-block runs, M < 16, one K block)
     (16, 4096, 7168), (1, 4096, 7168), (5, 3072, 2048), (16, 7168, 2560), (13, 18432, 128), (16, 3200, 6528),
     # 17 to 64 rows: the same cut with separate rings for weights and activations (2, 3, 4 row groups)
@@ -90,14 +92,15 @@ def test_gemm_dense(G, shape, pow2):
 
 
 @pytest.mark.parametrize("shape", [(2048, 2048, 7168), (300, 2048, 1024), (129, 1280, 2560), (1000, 4096, 512), (513, 18432, 1024),
-                                   (2048, 18432, 512), (777, 4224, 1536), (257, 19200, 512), (64, 24576, 1536), (16, 4096, 2048)],
+                                   (2048, 18432, 512), (777, 4224, 1536), (257, 19200, 512), (64, 24576, 1536), (16, 4096, 2048),
+                                   (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024)],
                          ids=lambda s: "M%d_N%d_K%d" % s)
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_gemm_bf16_output_is_the_rounded_fp32_output(G, shape, pow2):
     """Every kernel rounds the same fp32 accumulators whichever way the result leaves (directly or as whole row runs
     through LDS): the bf16 output equals the fp32 output rounded to nearest-even, element for element, and rows or
     columns outside the problem are not written.  Shapes cover the K split inside a workgroup (<= 256 tiles), the
-    256-row kernels with ragged M and N and the decode kernels."""
+    256-row kernels with ragged M and N, the single-launch column split and the decode kernels."""
     M, N, K = shape
     xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + N + K + 7, pow2=pow2)
     say("gemm bf16 vs fp32 output", shape, "pow2" if pow2 else "f32")
