@@ -396,3 +396,42 @@ print("ok")
     env.pop("LP_GEMM_NO_SKINNY", None)
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=200)
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-1500:], r.stderr[-1500:])
+
+
+def test_gemm_column_split_one_launch_equals_two_launches(G):
+    """The single-launch column split (256 x 256 tiles, then K-split 128 x 128 tiles) gives bit for bit what the two
+    launches it replaces give; LP_GEMM_MIXED=0 restores those (the switch is read once per process, hence the child
+    process, which prints a digest of every output)."""
+    import hashlib
+    import os
+    import subprocess
+    import sys
+    say("gemm column split: one launch against two (LP_GEMM_MIXED=0 in a child process)")
+    shapes = ((2048, 18432, 1024), (1900, 18432, 2048))
+
+    def digests():
+        out = []
+        for (M, N, K) in shapes:
+            for pow2 in (False, True):
+                xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + K, pow2=pow2)
+                c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+                out.append(hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest())
+        return out
+
+    code = (
+        "import sys, hashlib, torch\n"
+        "import gcore_lowp as G\n"
+        "sys.path.insert(0, %r)\n"
+        "from tests import test_gpu_gemm as t\n"
+        "for (M, N, K) in %r:\n"
+        "    for pow2 in (False, True):\n"
+        "        xq, xs, wq, ws = t.quantized_problem(M, N, K, seed=M + K, pow2=pow2)\n"
+        "        print('[case] two launches', M, N, K, pow2, flush=True)\n"
+        "        c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())\n"
+        "        print('md5', hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest(), flush=True)\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), shapes)
+    env = dict(os.environ, LP_GEMM_MIXED="0", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
+    theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
+    assert len(theirs) == 2 * len(shapes) and theirs == digests(), (theirs, r.stdout[-800:])
