@@ -179,6 +179,9 @@ def test_gemm_grouped(G, case):
     ref = T.grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits)
     check(out, ref, f"grouped {case[:3]}")
     assert (out.float().cpu() - ref).abs().max().item() < 1.0
+    # whichever way the results leave the kernel (directly, or as row runs through LDS): the same rounded accumulators
+    wide = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda(), out_dtype=torch.float32)
+    assert wide.dtype == torch.float32 and torch.equal(out, wide.to(torch.bfloat16))
     say("deepgemm-style call")
     m_indices = torch.repeat_interleave(torch.arange(E), torch.tensor(m_splits)).to(torch.int32)
     out2 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
