@@ -69,7 +69,8 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     // ---- loads: row rg * 8 + i, columns c0 + 8 cc .. + 7; rows past the expert's end repeat its last row and
     // are zeroed afterwards (no branch between the loads)
     // The loaded words stay as they are; bf16 pairs are unpacked where they are used (32 registers instead of 64 live
-    // across the barrier: five workgroups per CU instead of four).
+    // across the barrier); with the other waves' maxima read one wave at a time below, a thread needs 69 registers and
+    // seven workgroups share a CU (96 and five with those reads unrolled, 123 and four with floats kept).
     constexpr int W = IS_BF16 ? 4 : 8;
     uint32_t rw[8][W];
     {
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
             for (int k = 0; k < W; ++k) asm volatile("" : "+v"(rw[i][k]));
         }
     }
-#pragma unroll
+#pragma unroll 1                         // one wave's maxima at a time: unrolled, the 32 loaded registers set the kernel's peak
     for (int w = 0; w < 4; ++w) {
         const u32x4 a = wave_max[w][cc][0], b = wave_max[w][cc][1];
 #pragma unroll
