@@ -58,6 +58,7 @@ def main():
         sys.exit("bench.py: no GPU visible")
     import gcore_lowp  # noqa: F401  (fails loudly if the HIP library is missing)
     from gcore_lowp import _abi as A
+    from tests._inputs import zipf_m_splits        # the grouped problem's rows per expert: one recipe for tests and bench
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -347,10 +348,7 @@ def main():
 
         # -------------------------------------------------------------- config 4: grouped MoE GEMM
         E4, tokens, topk = 256, 8192, 8
-        cpu_gen = torch.Generator().manual_seed(4321)
-        pop = torch.arange(1, E4 + 1, dtype=torch.float64) ** -1.1
-        choice = torch.multinomial(pop.expand(tokens, E4), topk, replacement=False, generator=cpu_gen)
-        m_splits = torch.bincount(choice.flatten(), minlength=E4)
+        m_splits = zipf_m_splits(E4, tokens, topk, seed=4321)
         offs = torch.zeros(E4 + 1, dtype=torch.int32)
         offs[1:] = torch.cumsum(m_splits, 0)
         offs_d = offs.to(dev)

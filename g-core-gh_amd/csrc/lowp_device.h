@@ -31,10 +31,13 @@ __device__ __forceinline__ BlockScale derive_scale(float amax, float amax_floor,
     BlockScale b;
     b.stored = 1.0f; b.div = 1.0f; b.recip = 1.0f; b.exp2 = 0; b.fast = true;
     if (MODE == LP_SCALE_POW2) {
-        float safe = amax < 1.17549435e-38f ? 1.17549435e-38f : amax;
+        // amax_floor = 0: the all-zero rule of the eager quantiser; a positive floor (the round_sf branch of the
+        // 1 x 128 / 128 x 128 test quantisers) replaces it, a floored block is never "all zero"
+        const float a = amax < amax_floor ? amax_floor : amax;
+        float safe = a < 1.17549435e-38f ? 1.17549435e-38f : a;
         float r = safe / kE4M3Max;
         int e = ceil_log2_exact(r);
-        if (!(amax > 0.0f)) e = 0;
+        if (!(a > 0.0f)) e = 0;
         b.exp2 = e;
         b.stored = ldexpf(1.0f, e);
     } else if (MODE == LP_SCALE_RCP_POW2) {

@@ -43,21 +43,24 @@ def quantize_fp8_blockwise(weight: torch.Tensor, block_size: tuple[int, int], *,
 
 def _div_quant(x, block, *, round_sf, amax_floor, zero_rule):
     if round_sf:
-        # pow2 scale with a floor on amax: same as the POW2 mode whenever amax >= floor
-        raise NotImplementedError("round_sf=True with an amax floor: use quant_fp8_e4m3_scale_e8m0")
+        # s = 2^ceil(log2(max(amax, floor) / 448)) as an fp32 tensor; a floored block has no all-zero rule
+        # (tests/test_gfused/test_deepseek_tilekernels_quant.py:32-35,51-54)
+        q, s, _ = ops.quant_fp8_block(x, block, scale_mode=A.SCALE_POW2, scale_dtype=torch.float32,
+                                      amax_floor=amax_floor, zero_rule=A.ZERO_NONE)
+        return q, s
     q, s, _ = ops.quant_fp8_block(x, block, scale_mode=A.SCALE_DIV, scale_dtype=torch.float32,
                                   amax_floor=amax_floor, zero_rule=zero_rule)
     return q, s
 
 
 def quant_1d(x: torch.Tensor, block_size: int = 128, *, round_sf: bool = False):
-    """Row-wise 1 x block_size activation quant, s = max(amax, 1e-12)/448.
+    """Row-wise 1 x block_size activation quant, s = max(amax, 1e-12)/448 (round_sf: rounded up to a power of two).
     Returns (e4m3fn [M, K], fp32 scale [M, K/block_size])."""
     return _div_quant(x, (1, block_size), round_sf=round_sf, amax_floor=1e-12, zero_rule=A.ZERO_NONE)
 
 
 def quant_2d(w: torch.Tensor, block_size: tuple[int, int] = (128, 128), *, round_sf: bool = False):
-    """bm x bn weight quant, s = max(amax, 1e-12)/448.
+    """bm x bn weight quant, s = max(amax, 1e-12)/448 (round_sf: rounded up to a power of two).
     Returns (e4m3fn [N, K], fp32 scale [N/bm, K/bn])."""
     return _div_quant(w, tuple(block_size), round_sf=round_sf, amax_floor=1e-12, zero_rule=A.ZERO_NONE)
 

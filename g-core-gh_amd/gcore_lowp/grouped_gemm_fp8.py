@@ -24,10 +24,21 @@ def _scale_arg(s, dev):
     return s.to(torch.float32).contiguous(), A.F32
 
 
+def _check_offsets(m_offsets: torch.Tensor, E: int, dev, what: str) -> torch.Tensor:
+    """The kernels read m_offsets as E + 1 int32 values in device memory: give them exactly that."""
+    assert isinstance(m_offsets, torch.Tensor) and m_offsets.dim() == 1 and m_offsets.numel() == E + 1, \
+        f"{what}: m_offsets must hold E + 1 = {E + 1} values"
+    assert not m_offsets.dtype.is_floating_point, f"{what}: m_offsets must be an integer tensor"
+    return m_offsets.to(device=dev, dtype=torch.int32).contiguous()
+
+
 def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor | None = None,
-                     out_dtype=torch.bfloat16) -> torch.Tensor:
+                     out_dtype=torch.bfloat16, total_rows: int | None = None, validate: bool = False) -> torch.Tensor:
     """xq [M,K] e4m3fn, xs [M,K/128], wq [E,N,K] e4m3fn, ws [E,N/128,K/128],
-    m_offsets int32 [E+1] on the GPU (rows of expert e: m_offsets[e]..m_offsets[e+1]-1)."""
+    m_offsets integer [E+1] (rows of expert e: m_offsets[e]..m_offsets[e+1]-1, non-decreasing from 0, last <= M).
+    Rows at or beyond m_offsets[E] belong to no expert: a freshly allocated `out` has them zeroed, a caller's `out`
+    keeps them.  total_rows: m_offsets[E] when the caller knows it on the host (saves reading it back);
+    validate: check the offsets on the host (one device read-back)."""
     M, K = xq.shape
     E, N, K2 = wq.shape
     assert K == K2 and K % 128 == 0 and N % 128 == 0
@@ -38,11 +49,18 @@ def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor 
     sb, cb = _scale_arg(ws, dev)
     if ca != cb:
         sa, sb, ca = sa.to(torch.float32), sb.to(torch.float32), A.F32
+    offs = _check_offsets(m_offsets, E, dev, "grouped_gemm_fp8")
+    if validate:
+        o = offs.cpu()
+        if int(o[0]) != 0 or bool((o[1:] < o[:-1]).any()) or int(o[-1]) > M:
+            raise ValueError(f"grouped_gemm_fp8: m_offsets must start at 0, never decrease and end at or below M = {M}")
     if out is None:
-        out = torch.zeros((M, N), dtype=out_dtype, device=dev)
+        out = torch.empty((M, N), dtype=out_dtype, device=dev)
+        if total_rows is None:
+            total_rows = int(offs[-1].item()) if E > 0 else 0
+        if total_rows < M:
+            out[total_rows:].zero_()
     assert out.is_contiguous() and tuple(out.shape) == (M, N) and out.dtype in (torch.bfloat16, torch.float32)
-    offs = m_offsets.to(device=dev, dtype=torch.int32).contiguous()
-    assert offs.numel() == E + 1
     with torch.cuda.device(dev):
         A.check(A.lib().lp_gemm_fp8_grouped(
             xq.contiguous().data_ptr(), sa.data_ptr(), wq.contiguous().data_ptr(), sb.data_ptr(), ca,
@@ -51,16 +69,29 @@ def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor 
     return out
 
 
+def offsets_from_m_indices(m_indices: torch.Tensor, E: int) -> torch.Tensor:
+    """Row ranges [E + 1] from a DeepGEMM-style contiguous layout: m_indices[r] = expert of row r, non-decreasing
+    over the real rows, -1 on the padding rows that close an expert's (aligned) segment.  A padding row is attached to
+    the expert whose segment it closes (leading ones to expert 0), so every real row keeps its own expert's range;
+    no value is read back to the host."""
+    idx = m_indices.to(torch.int64)
+    owner = torch.cummax(idx, 0).values.clamp(min=0) if idx.numel() else idx
+    counts = torch.bincount(owner, minlength=E)[:E]
+    offs = torch.zeros(E + 1, dtype=torch.int32, device=m_indices.device)
+    offs[1:] = torch.cumsum(counts, 0).to(torch.int32)
+    return offs
+
+
 def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs, rhs, out: torch.Tensor, m_indices: torch.Tensor) -> None:
     """lhs = (x_fp8 [M,K], x_scale [M,K/128]); rhs = (w_fp8 [E,N,K], w_scale [E,N/128,K/128]);
-    m_indices int32 [M], non-decreasing expert id per row; writes `out` [M,N] bf16 in place."""
+    m_indices int32 [M], non-decreasing expert id per row, -1 = padding row; writes `out` [M,N] bf16 in place.
+    DeepGEMM skips padding rows; here they are computed with the weights of the expert whose segment they close, so
+    their rows of `out` hold unspecified (finite-input dependent) values instead of staying untouched -- every real
+    row is the same either way."""
     xq, xs = lhs
     wq, ws = rhs
-    E = wq.shape[0]
-    counts = torch.bincount(m_indices.to(torch.int64).clamp(min=0), minlength=E)[:E]
-    offs = torch.zeros(E + 1, dtype=torch.int32, device=xq.device)
-    offs[1:] = torch.cumsum(counts, 0).to(torch.int32)
-    grouped_gemm_fp8(xq, xs, wq, ws, offs, out=out)
+    assert m_indices.dim() == 1 and m_indices.numel() == xq.shape[0], (tuple(m_indices.shape), xq.shape[0])
+    grouped_gemm_fp8(xq, xs, wq, ws, offsets_from_m_indices(m_indices.to(xq.device), wq.shape[0]), out=out)
 
 
 def choose_colwise_pad(m_splits) -> int:
@@ -78,6 +109,8 @@ def quant_fp8_colwise_t(x: torch.Tensor, m_offsets: torch.Tensor, m_splits, pad_
     pad_rows None: choose_colwise_pad(m_splits)."""
     assert x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
     rows, cols = x.shape
+    assert all(int(m) >= 0 for m in m_splits) and sum(int(m) for m in m_splits) <= rows, "m_splits must fit the rows of x"
+    m_offsets = _check_offsets(m_offsets, len(m_splits), x.device, "quant_fp8_colwise_t")
     if pad_rows is None:
         pad_rows = choose_colwise_pad(m_splits)
     nblk = [(int(m) + pad_rows - 1) // pad_rows * (pad_rows // 128) for m in m_splits]
@@ -126,7 +159,7 @@ class _GroupedGemmFp8(torch.autograd.Function):
         from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
         xq, xs = quant_fp8_e4m3_scale_e8m0(x, block_size=(1, 128))
         offs = _offsets(m_splits, x.device)
-        out = grouped_gemm_fp8(xq, xs, wq, ws, offs, out_dtype=out_dtype)
+        out = grouped_gemm_fp8(xq, xs, wq, ws, offs, out_dtype=out_dtype, total_rows=sum(m_splits))
         ctx.need_wgrad = weight is not None and weight.requires_grad
         ctx.need_dgrad = inp.requires_grad
         saved = [wq.view(torch.uint8), ws.view(torch.uint8), offs]
@@ -149,7 +182,8 @@ class _GroupedGemmFp8(torch.autograd.Function):
             dyq, dys = quant_fp8_e4m3_scale_e8m0(dy, block_size=(1, 128))
             wt = wq.transpose(1, 2).contiguous().view(ops.E4M3)
             wst = ws.transpose(1, 2).contiguous().view(ops.E8M0)
-            dgrad = grouped_gemm_fp8(dyq, dys, wt, wst, offs, out_dtype=ctx.out_dtype).view(ctx.inp_shape)
+            dgrad = grouped_gemm_fp8(dyq, dys, wt, wst, offs, out_dtype=ctx.out_dtype,
+                                     total_rows=sum(ctx.m_splits)).view(ctx.inp_shape)
         if ctx.need_wgrad:
             xtq, xts = ctx.saved_tensors[3:5]
             dtq, dts, nblk = quant_fp8_colwise_t(dy, offs, ctx.m_splits, ctx.pad_rows)       # padded like X^T in the forward
@@ -179,6 +213,7 @@ class MyTeGroupedLinearFp8(torch.nn.Module):
     def forward(self, inp: torch.Tensor, weight, m_splits: list) -> torch.Tensor:
         assert len(m_splits) == self.num_gemms, (len(m_splits), self.num_gemms)
         m_splits = [int(x) for x in m_splits]
+        assert all(m >= 0 for m in m_splits), "m_splits must not be negative"
         if hasattr(weight, "_data") and hasattr(weight, "_scale"):
             wq, ws = weight._data, weight._scale
         elif isinstance(weight, (tuple, list)):

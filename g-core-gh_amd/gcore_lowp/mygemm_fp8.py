@@ -13,17 +13,13 @@ from . import ops
 
 __all__ = ["gemm_fp8_block_scaling_impl", "gemm_impl"]
 
-_workspace: dict = {}
-
-
 def _get_workspace(dev: torch.device, nbytes: int) -> torch.Tensor | None:
+    """Scratch for the K-split kernels: a fresh tensor per call.  The caching allocator hands the block back to
+    the stream that used it last, so two GEMMs on different streams never share partial sums (a cached buffer
+    per device would) and a block that is still being read is not given to another stream."""
     if nbytes <= 0:
         return None
-    ws = _workspace.get(dev)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-        _workspace[dev] = ws
-    return ws
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
 
 
 def _scale_arg(s: torch.Tensor, dev) -> tuple[torch.Tensor, int]:
@@ -96,3 +92,53 @@ def gemm_impl(A_, B_, block_M=128, block_N=128, block_K=64, dtype=torch.bfloat16
         A.check(A.lib().lp_gemm_nt(a.data_ptr(), b.data_ptr(), _NT_CODES[dtype], M, N, K, C.data_ptr(),
                                    _NT_CODES[out_dtype], A.stream_ptr()))
     return C.to(home)
+
+
+class _GemmProfiler:
+    """`kernel.get_profiler(...).do_bench()` of the tile compiler's kernel objects: average latency in ms."""
+
+    def __init__(self, kernel):
+        self._k = kernel
+
+    def do_bench(self, warmup: int = 5, rep: int = 20) -> float:
+        k = self._k
+        dev = A.require_gpu()
+        g = torch.Generator(device=dev).manual_seed(0)
+        # small integers (exact in e4m3 and bf16), like the reference's TensorSupplyType.Integer
+        a = torch.randint(-3, 4, (k.M, k.K), generator=g, device=dev).to(torch.float32).to(k.dtype)
+        b = torch.randint(-3, 4, (k.N, k.K), generator=g, device=dev).to(torch.float32).to(k.dtype)
+        for _ in range(max(warmup, 1)):
+            k(a, b)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(max(rep, 1)):
+            k(a, b)
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop) / max(rep, 1)
+
+
+class _CompiledGemm:
+    """What `gemm_impl.compile(M=, N=, K=, ...)` returns in the reference (tests/test_gfused/test_my_gemm_fp8.py:141-163):
+    a callable fixed to one shape and dtype pair, with a profiler.  Nothing is compiled here; the shape is checked
+    when the object is called."""
+
+    def __init__(self, M, N, K, block_M=128, block_N=128, block_K=64, dtype=torch.bfloat16, out_dtype=torch.bfloat16,
+                 accum_dtype=torch.float32):
+        if dtype not in (torch.float8_e4m3fn, torch.bfloat16):
+            raise TypeError(f"gemm_impl: operands must be float8_e4m3fn or bfloat16, got {dtype}")
+        if out_dtype not in _NT_CODES:
+            raise TypeError(f"gemm_impl: unsupported out_dtype {out_dtype}")
+        self.M, self.N, self.K = int(M), int(N), int(K)
+        self.dtype, self.out_dtype, self.accum_dtype = dtype, out_dtype, accum_dtype
+        self.blocks = (block_M, block_N, block_K)
+
+    def __call__(self, A_, B_):
+        assert tuple(A_.shape) == (self.M, self.K) and tuple(B_.shape) == (self.N, self.K), (A_.shape, B_.shape)
+        return gemm_impl(A_, B_, *self.blocks, dtype=self.dtype, out_dtype=self.out_dtype, accum_dtype=self.accum_dtype)
+
+    def get_profiler(self, tensor_supply_type=None):
+        return _GemmProfiler(self)
+
+
+gemm_impl.compile = _CompiledGemm

@@ -139,7 +139,8 @@ def fp4_to_fp8_amax(x: torch.Tensor, scale: torch.Tensor, *, scale_mode: int = A
 def selftest(which: int) -> int:
     dev = A.require_gpu()
     out = torch.zeros(1, dtype=torch.int64, device=dev)
-    A.check(A.lib().lp_selftest(which, out.data_ptr(), A.stream_ptr()))
+    with torch.cuda.device(dev):
+        A.check(A.lib().lp_selftest(which, out.data_ptr(), A.stream_ptr()))
     return int(out.item())
 
 
@@ -147,5 +148,6 @@ def debug_cast(kind: int, x: torch.Tensor) -> torch.Tensor:
     dev = A.require_gpu()
     xg = x.to(dev, torch.float32).contiguous()
     out = torch.empty(xg.shape, dtype=torch.int16 if kind == 3 else torch.uint8, device=dev)
-    A.check(A.lib().lp_debug_cast(kind, xg.data_ptr(), out.data_ptr(), xg.numel(), A.stream_ptr()))
+    with torch.cuda.device(dev):
+        A.check(A.lib().lp_debug_cast(kind, xg.data_ptr(), out.data_ptr(), xg.numel(), A.stream_ptr()))
     return out.cpu()

@@ -39,8 +39,9 @@ enum lp_dtype {
 
 /* How the per-block scale is derived from the block's amax. */
 enum lp_scale_mode {
-    /* s = 2^ceil(log2(max(amax, FLT_MIN)/448)), q = cast(clamp(x / s));
-     * gpatch_v4/kernel/quantize/eager_quant_kernels.py:132-181 */
+    /* s = 2^ceil(log2(max(amax, amax_floor, FLT_MIN)/448)), q = cast(clamp(x / s)); with amax_floor = 0 an
+     * all-zero block gets s = 1: gpatch_v4/kernel/quantize/eager_quant_kernels.py:132-181; with a positive
+     * floor (1e-12) it is the round_sf branch of tests/test_gfused/test_deepseek_tilekernels_quant.py:22-58 */
     LP_SCALE_POW2 = 0,
     /* s = max(amax, amax_floor)/448, q = cast(clamp(x / s));
      * tests/test_gfused/test_te_gemm_fp8.py:82-101,

@@ -229,10 +229,13 @@ int64_t orc_quant_fp8_block(const float *x, int64_t rows, int64_t cols, int bm, 
             if (saw_nan) amax = NAN;
             float s = 1.0f, f = 1.0f;
             if (mode == ORC_SCALE_POW2) {
-                float safe = amax < FLT_MIN ? FLT_MIN : amax;       /* clamp(min=tiny) */
+                /* amax_floor > 0: the round_sf branch of tests/test_gfused/test_deepseek_tilekernels_quant.py:22-58
+                 * (amax.clamp(min=1e-12) first, no all-zero rule); amax_floor = 0: eager_quant_kernels.py:168-171 */
+                float a = amax < amax_floor ? amax_floor : amax;
+                float safe = a < FLT_MIN ? FLT_MIN : a;             /* clamp(min=tiny) */
                 float r = safe / 448.0f;
                 s = ldexpf(1.0f, orc_pow2_exponent(r, log2_kind));
-                if (!(amax > 0.0f)) s = 1.0f;                        /* where(max_abs > 0, s, 1) */
+                if (!(a > 0.0f)) s = 1.0f;                           /* where(max_abs > 0, s, 1) */
             } else if (mode == ORC_SCALE_RCP || mode == ORC_SCALE_RCP_POW2) {
                 /* gpatch_v4/kernel/quantize/qat.py:155-161: amax = max(amax, floor); s = amax * fl32(1/448),
                  * or 2^ceil(log2 s) built on the bits of s (qat.py:98-113) when the scale is rounded */

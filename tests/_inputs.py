@@ -58,3 +58,14 @@ def edge_tiles():
     stripe[17 + 29 * 3, 3 * 32 + 31] = -1792.0
     tiles.append(stripe)
     return torch.cat(tiles, dim=1).to(torch.bfloat16)
+
+
+def zipf_m_splits(experts=256, tokens=8192, topk=8, seed=4321, exponent=1.1):
+    """Rows per expert of the grouped-GEMM benchmark problem: expert popularity ~ rank^-exponent, every token picks
+    `topk` distinct experts (seeded, without replacement), rows are then sorted by expert.  Returns an int64 tensor
+    [experts] summing to tokens * topk."""
+    g = torch.Generator().manual_seed(seed)
+    pop = torch.arange(1, experts + 1, dtype=torch.float64) ** -exponent
+    choice = torch.multinomial(pop.expand(tokens, experts), topk, replacement=False, generator=g)
+    return torch.bincount(choice.flatten(), minlength=experts)
+

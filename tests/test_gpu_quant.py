@@ -68,6 +68,8 @@ def test_software_casts_match_oracle(G, corc):
 def _ref(name, x, block):
     if name == "pow2":
         return T.quant_fp8_e4m3_scale_e8m0(x, block)
+    if name == "pow2_floor":
+        return T.quant_block_pow2_scale(x, block, amax_floor=1e-12)
     if name == "div_floor":
         return T.quant_block_fp32_scale(x, block, amax_floor=1e-12)
     if name == "div_zero1":
@@ -79,6 +81,9 @@ def _hip(G, name, x, block):
     from gcore_lowp import _abi as A, ops
     if name == "pow2":
         return G.quant_fp8_e4m3_scale_e8m0(x, block)
+    if name == "pow2_floor":
+        # the round_sf branch of the reference's test quantisers, through the drop-ins that carry that flag
+        return G.quant_1d(x, block[1], round_sf=True) if block[0] == 1 else G.quant_2d(x, block, round_sf=True)
     if name == "div_floor":
         q, s, _ = ops.quant_fp8_block(x, block, scale_mode=A.SCALE_DIV, scale_dtype=torch.float32, amax_floor=1e-12)
         return q, s
@@ -105,7 +110,7 @@ def _inputs_for(block):
     return xs
 
 
-@pytest.mark.parametrize("name", ["pow2", "div_floor", "div_zero1", "mul"])
+@pytest.mark.parametrize("name", ["pow2", "pow2_floor", "div_floor", "div_zero1", "mul"])
 @pytest.mark.parametrize("block", [(128, 128), (1, 128), (2, 2), (64, 32)])
 def test_quant_parity(G, corc, name, block):
     for label, x in _inputs_for(block).items():
@@ -119,7 +124,7 @@ def test_quant_parity(G, corc, name, block):
         assert bits_equal(hs, rs), f"scales differ: {name} {block} {label}"
         assert bits_equal(hq, rq), f"codes differ: {name} {block} {label}: {(u8(hq) != u8(rq)).sum().item()} bytes"
         # and against the scalar C oracle
-        kw = {"pow2": dict(mode=0), "div_floor": dict(mode=1, amax_floor=1e-12),
+        kw = {"pow2": dict(mode=0), "pow2_floor": dict(mode=0, amax_floor=1e-12), "div_floor": dict(mode=1, amax_floor=1e-12),
               "div_zero1": dict(mode=1, zero_rule=2), "mul": dict(mode=2)}[name]
         cq, cs, csb, _ = corc.quant_fp8_block(x.float().numpy(), block[0], block[1], **kw)
         assert np.array_equal(u8(hq).numpy(), cq)

@@ -22,6 +22,7 @@ def _bits(t):
 
 MODES = [
     ("pow2", dict(mode=0, amax_floor=0.0, zero_rule=0)),
+    ("pow2_floor", dict(mode=0, amax_floor=1e-12, zero_rule=0)),
     ("div_floor", dict(mode=1, amax_floor=1e-12, zero_rule=0)),
     ("div_zero1", dict(mode=1, amax_floor=0.0, zero_rule=2)),
     ("mul", dict(mode=2, amax_floor=0.0, zero_rule=0)),
@@ -32,6 +33,8 @@ def _torch_quant(name, x, block):
     if name == "pow2":
         q, s = T.quant_fp8_e4m3_scale_e8m0(x, block)
         return q, s.float()
+    if name == "pow2_floor":
+        return T.quant_block_pow2_scale(x, block, amax_floor=1e-12)
     if name == "div_floor":
         return T.quant_block_fp32_scale(x, block, amax_floor=1e-12)
     if name == "div_zero1":
@@ -54,6 +57,27 @@ def test_c_and_torch_oracles_agree(corc, name, kw, block):
         assert nan == 0
         assert np.array_equal(q, _u8(tq)), name
         assert np.array_equal(s.view(np.uint32), _bits(ts.float()).view(np.uint32)), name
+
+
+def test_pow2_with_amax_floor_closed_forms(corc):
+    """round_sf branch (tests/test_gfused/test_deepseek_tilekernels_quant.py:32-35): an all-zero block is floored to
+    amax = 1e-12, so its scale is 2^ceil(log2(1e-12 / 448)) = 2^-48 (1e-12/448 = 2.23e-15 lies in (2^-49, 2^-48]),
+    never 1; any block whose amax exceeds the floor gets exactly the scale of the unfloored power-of-two mode."""
+    x = I.weight_like(256, 256, 21).float()
+    x[:128, :128] = 0
+    for orc in ("c", "torch"):
+        if orc == "c":
+            q, s, _, _ = corc.quant_fp8_block(x.numpy(), 128, 128, mode=0, amax_floor=1e-12)
+            q0, s0, _, _ = corc.quant_fp8_block(x.numpy(), 128, 128, mode=0, amax_floor=0.0)
+        else:
+            tq, ts = T.quant_block_pow2_scale(x, (128, 128), amax_floor=1e-12)
+            tq0, ts0 = T.quant_fp8_e4m3_scale_e8m0(x, (128, 128))
+            q, s, q0, s0 = _u8(tq), ts.numpy().reshape(2, 2), _u8(tq0), ts0.float().numpy()
+        s, s0 = np.asarray(s, dtype=np.float32).reshape(2, 2), np.asarray(s0, dtype=np.float32).reshape(2, 2)
+        assert s[0, 0] == np.float32(2.0 ** -48) and s0[0, 0] == 1.0, orc
+        assert (q[:128, :128] == 0).all()
+        mask = np.ones((2, 2), bool); mask[0, 0] = False
+        assert np.array_equal(s[mask], s0[mask]) and np.array_equal(q[128:], q0[128:]) and np.array_equal(q[:, 128:], q0[:, 128:])
 
 
 def test_pow2_exact_equals_libm_on_bf16_grid(corc):
