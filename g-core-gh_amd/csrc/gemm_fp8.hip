@@ -15,6 +15,7 @@
 //
 // The same tile routine serves the dense, split-K (skinny M) and grouped
 // (per-expert row ranges) entry points.
+#include <pthread.h>
 #include <stdlib.h>
 
 #include "gemm_common.h"
@@ -540,3 +541,59 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
                            (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
     return check_launch("lp_gemm_fp8_grouped");
 }
+
+// ---------------------------------------------------------------------------------------------
+// lp_gemm_fp8_block for callers that cannot allocate device memory: the K-split partial sums go to a buffer that is
+// part of the library's device image instead of a caller workspace.  Each GPU the process uses holds its own copy
+// of the array at its own address; in host code the array's name is only a handle for hipGetSymbolAddress, so the
+// device address is looked up once per device (with that device current) and everything below uses that pointer.
+constexpr int64_t kStaticScratchBytes = 32ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+extern "C" int64_t lp_gemm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];            // device address of `scratch` per device ordinal, nullptr = not looked up yet
+pthread_mutex_t g_scratch_lock = PTHREAD_MUTEX_INITIALIZER;
+
+int static_scratch(void **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(LP_ERR_HIP, "lp_gemm_fp8_block_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block_static: device ordinal %d out of range", dev);
+    pthread_mutex_lock(&g_scratch_lock);
+    void *p = g_scratch_ptr[dev];
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e == hipSuccess && p) g_scratch_ptr[dev] = p;
+    }
+    pthread_mutex_unlock(&g_scratch_lock);
+    if (e != hipSuccess || !p)
+        return fail(LP_ERR_HIP, "lp_gemm_fp8_block_static: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    *out = p;
+    return LP_OK;
+}
+}  // namespace
+
+extern "C" int lp_gemm_fp8_block_static(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                                        int64_t M, int64_t N, int64_t K, void *C, int out_dtype, lp_stream_t stream)
+{
+    int rc = check_gemm_args("lp_gemm_fp8_block_static", Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    // Only the K-split pair uses scratch (fp32 partial tiles, every one of them written before the reduction reads
+    // it, so the buffer's previous contents never matter and nothing is cleared).
+    const int64_t need = split_bytes(M, N, K);
+    LP_REQUIRE(need <= kStaticScratchBytes,
+               "lp_gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of K-split scratch, the built-in buffer holds %lld; "
+               "call lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes()",
+               (long long)M, (long long)N, (long long)K, (long long)need, (long long)kStaticScratchBytes);
+    void *ws = nullptr;
+    if (need > 0) {
+        rc = static_scratch(&ws);
+        if (rc) return rc;
+    }
+    return lp_gemm_fp8_block(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, ws, need, stream);
+}
+

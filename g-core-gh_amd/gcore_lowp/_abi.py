@@ -39,6 +39,8 @@ PROTOTYPES = {
     "lp_fp4_to_fp8_rebase": (_i32, [_p, _p, _i64, _i64, _p, _p, _i32, _p]),
     "lp_fp4_to_fp8_amax": (_i32, [_p, _p, _i64, _i64, _i32, _f32, _i32, _p, _p, _i32, _p, _p]),
     "lp_gemm_fp8_block": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p, _i64, _p]),
+    "lp_gemm_fp8_block_static": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
+    "lp_gemm_static_scratch_bytes": (_i64, []),
     "lp_gemm_nt": (_i32, [_p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_gemm_fp8_rowscale": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_quant_fp8_colwise_t": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _i64, _i32, _p, _p, _i32, _p]),

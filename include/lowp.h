@@ -226,6 +226,22 @@ int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void
 int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * lp_gemm_fp8_block without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the K-split partial sums go to a buffer of
+ * lp_gemm_static_scratch_bytes() = 32 MiB that is part of the library's device image (every GPU the process uses
+ * holds one copy until the process ends).  Same kernels, same summation order and therefore the same bits as
+ * lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes(M, N, K).  The call allocates and frees nothing.
+ * Shapes whose K split needs more than the buffer are rejected with LP_ERR_INVALID and a message naming both
+ * sizes (shapes that need no scratch always pass).  All calls on one GPU share that GPU's buffer: calls that can
+ * overlap on one GPU (different streams, or threads) race on it -- serialise them or use lp_gemm_fp8_block.
+ * Nothing has to be cleared between calls: every partial tile is written before it is read.
+ * No counterpart in the reference (its GEMM is a JIT kernel without scratch, gfused/mygemm_fp8.py:44-97).
+ */
+int lp_gemm_fp8_block_static(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                             int64_t M, int64_t N, int64_t K, void *C, int out_dtype, lp_stream_t stream);
+int64_t lp_gemm_static_scratch_bytes(void);
+
+/*
  * Unscaled C = A B^T with fp32 accumulation.  A [M,K], B [N,K], both of
  * in_dtype (LP_E4M3 or LP_BF16); C [M,N] of out_dtype (LP_E4M3, LP_BF16, LP_F32).
  * K must be a multiple of 128 (LP_E4M3) or 64 (LP_BF16), N a multiple of 16; M is free.

@@ -82,6 +82,25 @@ def test_host_side_validation(lib):
     assert L.lp_gemm_fp8_rowscale(None, None, None, None, lib.E8M0, 0, 128, 128, None, lib.BF16, None) == 0
     assert L.lp_quant_fp8_block(None, lib.BF16, 0, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, None, None, lib.F32, None, None) == 0
     assert L.lp_gemm_fp8_block(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None, 0, None) == 0
+    assert L.lp_gemm_fp8_block_static(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None) == 0
+
+
+def test_static_scratch_entry_rejects_oversized_split(lib):
+    """The entry point that brings its own K-split scratch refuses, before anything is launched or looked up on the
+    device, a shape whose partial sums do not fit the built-in buffer, and names both sizes."""
+    import ctypes
+    L = lib.lib()
+    cap = L.lp_gemm_static_scratch_bytes()
+    assert cap == 32 << 20
+    buf = ctypes.create_string_buffer(64)
+    one = ctypes.cast(ctypes.addressof(buf) + (-ctypes.addressof(buf)) % 16, ctypes.c_void_p)
+    M, N, K = 1280, 1024, 7168                          # 80 tiles x 7 K ranges of fp32 partials
+    need = 7 * M * N * 4
+    assert cap < need <= L.lp_gemm_workspace_bytes(M, N, K)      # the latter also counts the tuning aid's scale copies
+    rc = L.lp_gemm_fp8_block_static(one, one, one, one, lib.F32, M, N, K, one, lib.BF16, None)
+    assert rc == -1 and str(need) in lib.last_error() and str(cap) in lib.last_error()
+    rc = L.lp_gemm_fp8_block_static(one, one, one, one, lib.F32, 64, 100, 128, one, lib.BF16, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
 
 
 def test_wrappers_keep_reference_exceptions(lib):
