@@ -17,6 +17,10 @@ Kernel durations are measured with HIP events on the stream the kernels are
 launched on (torch's current stream); launches are replayed from a HIP graph
 where possible so that host launch cost does not leak into device time, and
 bandwidth kernels rotate over buffer sets larger than the 256 MB Infinity Cache.
+After the W warm-up launches every timed region is preceded by untimed replays
+of its graph until the GPU has been busy for 40 ms, then exactly K launches are
+timed in one region: the first tens of milliseconds after an idle stretch run
+up to 15 % slower, which a short timed region would report as the kernel's time.
 """
 from __future__ import annotations
 
@@ -30,6 +34,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "g-core-gh_amd"))
 
+SETTLE_MS = 40.0             # untimed graph replays before every timed region (see time_launches)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 # Bytes per launch of the headline GEMM kernel between its L2s and the memory side (Infinity Cache / HBM): reads from
@@ -42,10 +47,12 @@ GEMM_MIXED_TRAFFIC_BYTES = 528.4e6   # gemm_asm_mixed on the whole problem; same
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: deep,copy,c2q,c1,c3,c5,c4 (default: all)")
+    ap.add_argument("--only-gemm", action="store_true", help="extras: only the skinny and the grouped GEMM (counter runs)")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches (for counter-collection runs)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget of the CPU baseline sample")
     args = ap.parse_args()
@@ -85,8 +92,19 @@ def main():
                             fns[i % len(fns)]()
                 torch.cuda.current_stream().wait_stream(side)
                 torch.cuda.synchronize()
-                g.replay()                     # one untimed replay
-                torch.cuda.synchronize()
+                # untimed replays until the GPU has worked for SETTLE_MS without a pause: after an idle stretch the
+                # first ~30 ms of back-to-back GEMM launches run measurably slower (clocks still rising; six replays
+                # of 5 ms went 288, 268, 257, 252, 249, 244 us per launch), and a timed region that short would
+                # measure the ramp instead of the kernel
+                spent, n_rep = 0.0, 0
+                while n_rep < 1 or (spent < SETTLE_MS and n_rep < 64):
+                    s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    s0.record()
+                    g.replay()
+                    s1.record()
+                    torch.cuda.synchronize()
+                    spent += s0.elapsed_time(s1)
+                    n_rep += 1
             except Exception as e:             # capture unsupported: time eager launches
                 print(f"[bench] graph capture failed ({e}); timing eager launches", file=sys.stderr)
                 g = None
@@ -117,6 +135,10 @@ def main():
                                  q.data_ptr(), s.data_ptr(), A.F32, None, stream()))
 
     extras = {}
+    only = set(filter(None, ("c3,c4" if args.only_gemm else args.only).split(",")))
+
+    def want(section):
+        return not args.no_extras and (not only or section in only)
 
     # ------------------------------------------------------------------ config 2: dense GEMM (headline)
     M, N, K = 2048, 18432, 7168
@@ -145,9 +167,8 @@ def main():
     flops = 2.0 * M * N * K
     tflops = flops / (ms * 1e-3) / 1e12
     headline = {"ms": ms, "tflops": tflops}
-    # The call above is one launch (gemm_asm_mixed): 256 x 256 tiles on the first 16384 weight rows (two full rounds of
-    # 256 tiles), then K-split 128 x 128 tiles on the remaining 2048.  Beside it, the 256 x 256-tile kernel alone on the
-    # part of the problem it covers:
+    # The call above is one launch of gemm_asm_wide: 256 x 288 tiles, 8 x 64 = 512 of them, exactly two rounds on the 256
+    # CUs.  Beside it, the 256 x 256-tile kernel on the 16384 weight rows that make two full rounds of its tiles:
     N_BIG = 16384
     c_big = torch.empty(M, N_BIG, dtype=torch.bfloat16, device=dev)
 
@@ -180,7 +201,53 @@ def main():
     del bq, b_s, c, a_bf, a_s8, b_s8
     torch.cuda.empty_cache()
 
-    if not args.no_extras:
+    if want("deep"):
+        # -------------------------------------------------------------- a deep-K problem (K = 18432) on 256 x 256 tiles:
+        # what the loop reaches when the K steps dominate; and the unscaled NT GEMM at the reference's benchmark shape
+        # (tests/test_gfused/test_my_gemm_fp8.py:137: 4096^3, fp8 in, fp8 out, 0.575 ms on its hardware)
+        Md, Nd, Kd = 4096, 7168, 18432
+        ad = randn(Md, Kd)
+        adq = torch.empty(Md, Kd, dtype=torch.uint8, device=dev)
+        ads = torch.empty(Md, Kd // 128, dtype=torch.float32, device=dev)
+        quant_into(ad, 1, 128, adq, ads)
+        ads8 = torch.empty(Md, Kd // 128, dtype=torch.uint8, device=dev)
+        chk(L.lp_quant_fp8_block(ad.data_ptr(), A.BF16, Md, Kd, 1, 128, A.SCALE_POW2, 0.0, 0, adq.data_ptr(), ads8.data_ptr(),
+                                 A.E8M0, None, stream()))
+        del ad
+        wdq, wds, wds8 = [], [], []
+        for _ in range(2):
+            w = randn(Nd, Kd, std=0.02)
+            q = torch.empty(Nd, Kd, dtype=torch.uint8, device=dev)
+            sc = torch.empty(Nd // 128, Kd // 128, dtype=torch.float32, device=dev)
+            quant_into(w, 128, 128, q, sc)
+            wdq.append(q)
+            wds.append(sc)
+            wds8.append(torch.randint(118, 124, (Nd // 128, Kd // 128), dtype=torch.uint8, device=dev))
+            del w
+        cd = torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev)
+        fl_d = 2.0 * Md * Nd * Kd
+        for label, sa, sbs, code in (("fp32_scales", ads, wds, A.F32), ("e8m0_scales", ads8, wds8, A.E8M0)):
+            fns = [(lambda i=i: chk(L.lp_gemm_fp8_block(adq.data_ptr(), sa.data_ptr(), wdq[i].data_ptr(), sbs[i].data_ptr(), code,
+                                                        Md, Nd, Kd, cd.data_ptr(), A.BF16, None, 0, stream()))) for i in range(2)]
+            ms_d, _ = time_launches(fns, 10, 3)
+            extras[f"deep_k_gemm_4096x7168x18432_{label}"] = {"ms": ms_d, "tflops": fl_d / ms_d / 1e9,
+                                                              "mfma_frac": fl_d / ms_d / 1e9 / FP8_PEAK_TFLOPS}
+        del adq, ads, ads8, wdq, wds, wds8, cd
+        torch.cuda.empty_cache()
+        n4 = 4096
+        a_nt = torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).float().to(E4M3)
+        b_nt = [torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).float().to(E4M3) for _ in range(4)]
+        c_nt = torch.empty(n4, n4, dtype=torch.uint8, device=dev)
+        fns = [(lambda i=i: chk(L.lp_gemm_nt(a_nt.data_ptr(), b_nt[i].data_ptr(), A.E4M3, n4, n4, n4, c_nt.data_ptr(), A.E4M3, stream())))
+               for i in range(4)]
+        ms_nt, _ = time_launches(fns, 12, 4)
+        extras["gemm_impl_fp8_4096x4096x4096"] = {"ms": ms_nt, "tflops": 2.0 * n4 ** 3 / ms_nt / 1e9,
+                                                  "mfma_frac": 2.0 * n4 ** 3 / ms_nt / 1e9 / FP8_PEAK_TFLOPS,
+                                                  "reference_ms_on_its_hardware": 0.575}
+        del a_nt, b_nt, c_nt
+        torch.cuda.empty_cache()
+
+    if want("copy"):
         # -------------------------------------------------------------- calibration: a plain device copy of known size
         # (what a streaming read+write kernel reaches on this box; also the reference kernel for scaling the
         # FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this script)
@@ -194,6 +261,7 @@ def main():
                                                    "bytes": 4 * n, "kernel": "torch elementwise copy (bf16)"}
             del src, dst
             torch.cuda.empty_cache()
+    if want("c2q"):
         # -------------------------------------------------------------- config 2 operand: weight quantisation at full size
         w_big = randn(N, K, std=0.02)
         wq_big = torch.empty(N, K, dtype=torch.uint8, device=dev)
@@ -203,6 +271,7 @@ def main():
                                              "bytes": N * K * 3}
         del w_big, wq_big, ws_big
         torch.cuda.empty_cache()
+    if want("c1"):
         # -------------------------------------------------------------- config 1: 128x128 quant / dequant
         R = C = 4096
         sets = 12                                   # 12 x (32 + 16 MiB) > 256 MB
@@ -226,6 +295,7 @@ def main():
         del xs, qs, ss, outs
         torch.cuda.empty_cache()
 
+    if want("c3"):
         # -------------------------------------------------------------- config 3: skinny GEMM
         M3, N3, K3 = 64, 4096, 7168
         sets = 12                                   # 12 x 29 MB of weights > 256 MB
@@ -255,6 +325,7 @@ def main():
         del w3q, w3s
         torch.cuda.empty_cache()
 
+    if want("c5"):
         # -------------------------------------------------------------- config 5: FP4 -> FP8 (fused), whole MoE layer
         E_total, chunk = 256, 256                    # experts per launch: the whole layer, one launch per tensor kind
         shapes = [(2048, 7168), (2048, 7168), (7168, 2048)]
@@ -346,6 +417,7 @@ def main():
         del bufs, bouts
         torch.cuda.empty_cache()
 
+    if want("c4"):
         # -------------------------------------------------------------- config 4: grouped MoE GEMM
         E4, tokens, topk = 256, 8192, 8
         m_splits = zipf_m_splits(E4, tokens, topk, seed=4321)
@@ -474,10 +546,9 @@ def main():
                    "M": M, "N": N, "K": K, "operands": "pre-quantised, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_MIXED_TRAFFIC_BYTES,
-                     "kernel": "gemm_asm_mixed<false>: the whole problem in one launch (512 tiles of 256x256 on weight rows "
-                               "0..16383, then 256 K-split tiles of 128x128 on rows 16384..18431)",
+                     "kernel": "gemm_asm_wide<false>: the whole problem in one launch, 512 tiles of 256x288 (two full rounds of 256 CUs)",
                      "launch_ms": ms, "flops_per_launch": flops, "wall_ms_per_step": wall_ms,
-                     "big_tiles_alone": {"kernel": "gemm_asm<256,256,1>: M=2048, weight rows 0..16383 of 18432, K=7168 (512 tiles)",
+                     "tiles_256x256_alone": {"kernel": "gemm_asm<256,256,1>: M=2048, weight rows 0..16383 of 18432, K=7168 (512 tiles)",
                                          "launch_ms": big_ms, "flops_per_launch": big_flops, "tflops": big_tflops,
                                          "frac": big_tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_BIG_TRAFFIC_BYTES}},
         "cpu_baseline": cpu,

@@ -63,10 +63,10 @@ def declared_registers(hip_path: str) -> dict[str, set[tuple[str, int]]]:
     """Per loop file: the registers its asm statement in the .hip source declares as outputs or clobbers."""
     with open(hip_path) as f:
         src = f.read()
-    macro = re.search(r"#define LP_ASM_CLOBBERS(.*?)\n#define", src, re.S).group(1)
+    macros = {m.group(1): m.group(2) for m in re.finditer(r"#define (LP_ASM_CLOBBERS\w*)\b(.*?)(?=\n#define)", src, re.S)}
     out = {}
     for m in re.finditer(r'#include "(\w+_loop\.inc)"(.*?)\);', src, re.S):
-        text = m.group(2).replace("LP_ASM_CLOBBERS", macro)
+        text = re.sub(r"LP_ASM_CLOBBERS\w*", lambda k: macros[k.group(0)], m.group(2))
         regs = set()
         for q in re.findall(r'"=&\{(v\[\d+:\d+\])\}"', text):
             regs |= _regs(q)

@@ -500,6 +500,7 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     const int64_t small_tiles = tiles_m * tiles_n, big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
     if (!force_small && M >= 192 && (small_tiles >= 800 || (small_tiles > 512 && big_tiles <= 256))) {
         if (force_tn) return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, atoi(force_tn), st);
+        if (gemm::launch_wide(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, st, &rc)) return rc;
         const int64_t bm = (M + 255) / 256, bn = (N + 255) / 256, tiles = bm * bn;
         const int64_t full = tiles / 256, rem = tiles % 256;
         int64_t n_big = N;                                   // columns given to the big kernel

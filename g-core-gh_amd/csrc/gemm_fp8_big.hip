@@ -208,6 +208,21 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120",   \
         "v121", "v122", "v123", "v124", "v125", "v126", "v127", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47",   \
         "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63"
+#define LP_ASM_CLOBBERS_WIDE                                                                                              \
+    "memory", "scc", "m0", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32",  \
+        "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49",   \
+        "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v64", "v65", "v66",   \
+        "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83",   \
+        "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100",  \
+        "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "s40", "s41", "s42", "s43",     \
+        "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60",   \
+        "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77",   \
+        "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86"
+#define LP_ASM_INPUTS_WIDE                                                                                                \
+    [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
+        [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
+        [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
+        [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride)
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
@@ -225,14 +240,14 @@ struct StagedEpilogue {
     static constexpr int PITCH = COLS * 2 + 16;
     static constexpr int WAVE_BYTES = 64 * PITCH;
     static constexpr int CHUNKS = COLS / 8;                       // 16-byte chunks per row
-    static constexpr int LPR = CHUNKS > 8 ? 16 : 8;               // lanes per row when reading (a power of two >= CHUNKS)
-    static constexpr int PASSES = 64 / (64 / LPR);
+    static constexpr int PASSES = CHUNKS;                         // 64 rows x CHUNKS chunks, 64 chunks per pass
     __host__ __device__ static constexpr int write_offset(int mb, int nb, int l16, int lq)
     {
         return (mb * 16 + l16) * PITCH + (nb * 16 + 4 * lq) * 2;
     }
-    __host__ __device__ static constexpr int read_row(int pass, int lane) { return pass * (64 / LPR) + lane / LPR; }
-    __host__ __device__ static constexpr int read_chunk(int lane) { return lane % LPR; }
+    // chunks are read back in row-major order: consecutive lanes take consecutive chunks of a row and go on with the next row
+    __host__ __device__ static constexpr int read_row(int pass, int lane) { return (pass * 64 + lane) / CHUNKS; }
+    __host__ __device__ static constexpr int read_chunk(int pass, int lane) { return (pass * 64 + lane) % CHUNKS; }
     __host__ __device__ static constexpr int read_offset(int row, int chunk) { return row * PITCH + chunk * 16; }
 };
 
@@ -241,7 +256,9 @@ struct AsmTile {
     static constexpr int WAVES = TM / 64 * 2, NBW = TN / 32;
     static constexpr int A_BYTES = TM * KB, B_BYTES = TN * KB;                   // one K block of 128
     static constexpr int B_LDS = NST * KSUB * A_BYTES, S_LDS = NST * KSUB * (A_BYTES + B_BYTES);
-    static constexpr int LDS_BYTES = S_LDS + 2 * TM * 16;                        // NST stages of KSUB K blocks + scale groups
+    static constexpr int LOOP_BYTES = S_LDS + 2 * TM * 16;                       // NST stages of KSUB K blocks + scale groups
+    static constexpr int STAGING = WAVES * StagedEpilogue<TN / 2>::WAVE_BYTES;  // the waves' bf16 staging regions after the loop
+    static constexpr int LDS_BYTES = LOOP_BYTES > STAGING ? LOOP_BYTES : STAGING;
 };
 
 // HWS: e8m0 scales applied by the matrix cores (v_mfma_scale_*); As / Bs then point at bytes.
@@ -336,6 +353,12 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t sel1 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 32) >> 7) != (wcol0 >> 7)));
     const uint32_t sel2 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 64) >> 7) != (wcol0 >> 7)));
     (void)bs2_u; (void)sel1; (void)sel2;
+    // 256 x 288 tile: first 16-column block of this wave that lies in the second weight-scale block, whether this wave has
+    // a fifth weight copy (36 blocks of 8 rows over 8 waves), distance between a wave's weight copies (64 rows)
+    const uint32_t splitnb = __builtin_amdgcn_readfirstlane((uint32_t)(((((wcol0 >> 7) + 1) << 7) - wcol0) >> 4));
+    const uint32_t bextra = __builtin_amdgcn_readfirstlane(wave < (TN / 8) % WAVES ? 1u : 0u);
+    const uint32_t bstride = __builtin_amdgcn_readfirstlane((uint32_t)(8 * WAVES * K));
+    (void)splitnb; (void)bextra; (void)bstride;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
     // Layout: activation stages, weight stages, scale groups.
@@ -354,7 +377,29 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     (void)sdst; (void)srdb;
 
     f32x16v accs[NBW];
-    if constexpr (HWS && NBW == 8) {
+    if constexpr (TN == 288) {
+        static_assert(TM == 256 && KSUB == 1 && !DUAL && NST == 2 && !BROW, "the 288-column tile exists for the 256-row kernel only");
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7, acc8;
+        if constexpr (HWS) {
+            asm volatile(
+#include "gemm_wide_hw_loop.inc"
+                : "=&{v[112:127]}"(acc0), "=&{v[128:143]}"(acc1), "=&{v[144:159]}"(acc2), "=&{v[160:175]}"(acc3),
+                  "=&{v[176:191]}"(acc4), "=&{v[192:207]}"(acc5), "=&{v[208:223]}"(acc6), "=&{v[224:239]}"(acc7),
+                  "=&{v[240:255]}"(acc8)
+                : LP_ASM_INPUTS_WIDE
+                : LP_ASM_CLOBBERS_WIDE);
+        } else {
+            asm volatile(
+#include "gemm_wide_loop.inc"
+                : "=&{v[112:127]}"(acc0), "=&{v[128:143]}"(acc1), "=&{v[144:159]}"(acc2), "=&{v[160:175]}"(acc3),
+                  "=&{v[176:191]}"(acc4), "=&{v[192:207]}"(acc5), "=&{v[208:223]}"(acc6), "=&{v[224:239]}"(acc7),
+                  "=&{v[240:255]}"(acc8)
+                : LP_ASM_INPUTS_WIDE
+                : LP_ASM_CLOBBERS_WIDE);
+        }
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4;
+        accs[5] = acc5; accs[6] = acc6; accs[7] = acc7; accs[8] = acc8;
+    } else if constexpr (HWS && NBW == 8) {
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
         asm volatile(
 #include "gemm_big_hw_loop.inc"
@@ -476,9 +521,9 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             const int64_t row_base = m0 + wm * 64;
 #pragma unroll
             for (int p = 0; p < E::PASSES; ++p) {
-                const int row = E::read_row(p, lane), chunk = E::read_chunk(lane);
+                const int row = E::read_row(p, lane), chunk = E::read_chunk(p, lane);
                 const int64_t n = wcol0 + chunk * 8;
-                if (chunk < E::CHUNKS && row_base + row < M && n < N) {
+                if (row_base + row < M && n < N) {
                     const u32x4 v = *(const u32x4 *)(stage + E::read_offset(row, chunk));
                     *(u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n) = v;
                 }
@@ -517,6 +562,19 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
     tile_asm<TM, TN, KSUB, HWS, false, NST, false, true>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+}
+
+// 256 x 288 tiles: N = 18432 is 64 of them, so a 2048-row problem is 512 tiles, exactly two rounds on 256 CUs.
+template <bool HWS>
+__global__ __launch_bounds__(512) void gemm_asm_wide(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                     const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
+                                                     int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                     void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<256, 288, 1>::LDS_BYTES];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    tile_asm<256, 288, 1, HWS, false, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 256, M, tn * 288, N, K, C, ldc, out_dtype);
 }
 
 // 128 x 128 tile with the K split inside the workgroup (see tile_asm): 8 waves, two sets of LDS stages.
@@ -713,6 +771,30 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
     if (scale_dtype == LP_F32) GO(LP_F32);
     GO(LP_E8M0);
 #undef GO
+}
+
+// 256 x 288 tiles when they divide N and fill the last round of tiles better than 256 x 256 tiles would; false when
+// the shape does not fit (the caller goes on with the other kernels).
+bool launch_wide(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
+                 void *C, int64_t ldc, int out_dtype, hipStream_t st, int *rc)
+{
+    static const bool off = getenv("LP_GEMM_NO_ASM") != nullptr || (getenv("LP_GEMM_WIDE") && atoi(getenv("LP_GEMM_WIDE")) == 0);
+    static const bool force = getenv("LP_GEMM_WIDE") && atoi(getenv("LP_GEMM_WIDE")) == 1;             // tuning aid
+    if (off || (scale_dtype != LP_F32 && scale_dtype != LP_E8M0) || N % 288 || !asm_shape_ok(As, Bs, M, N, K, scale_dtype)) return false;
+    const int64_t tiles_m = (M + 255) / 256, wide = tiles_m * (N / 288), big = tiles_m * ((N + 255) / 256);
+    // fraction of CU slots used over whole rounds of 256 tiles
+    const double fill_wide = (double)wide / (double)((wide + 255) / 256 * 256), fill_big = (double)big / (double)((big + 255) / 256 * 256);
+    if (!force && !(fill_wide >= 0.9 && fill_wide > fill_big + 0.05)) return false;
+    const int64_t grid = gemm::padded_grid(tiles_m, N / 288);
+    if (grid > 0x7FFFFFFF) return false;
+    if (scale_dtype == LP_E8M0)
+        hipLaunchKernelGGL((gemm_asm_wide<true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, N / 288, C, ldc, out_dtype);
+    else
+        hipLaunchKernelGGL((gemm_asm_wide<false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
+                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, N / 288, C, ldc, out_dtype);
+    *rc = check_launch("lp_gemm_fp8_block(asm 256x288)");
+    return true;
 }
 
 // Columns [0, n_big) on 256 x 256 tiles and [n_big, N) on K-split 128 x 128 tiles in one launch; false when the shape does

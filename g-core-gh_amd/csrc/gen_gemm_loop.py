@@ -35,12 +35,39 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
-    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, lines
+    global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR
     HW = hw
+    # wide: a wave owns 64 x 144 columns (nine 16-column blocks), e.g. the 256 x 288 tile that cuts 18432 weight rows
+    # into exactly 64 tile columns.  144 columns always straddle two weight-scale blocks, at a 16-column boundary known
+    # only at run time (s74 = first block that takes the second scale row): the folds read one set of scale products,
+    # which is switched to the second row's products when the loop reaches that block.  The accumulators take 144
+    # registers, so the plan below moves everything down; fragment read addresses and the scale buffer base are used
+    # straight from the asm operands, and the weight copies share one per-lane offset (the tile's weight rows are
+    # never clamped: N is a multiple of the tile width) with one scalar base per copy.
+    WIDE = wide
+    if wide:
+        assert tm == 256 and waves_m == 4 and waves_n == 2 and ksub == 1 and nstage == 2 and not brow and not early
+        ACC, P, AF, WFB = 112, 80, 48, (32, 40)
+        SAN, SC, SC2, SRD = 24, 28, 20, "v19"
+        WS1, WS2, WSCUR = "v20", "v21", "v22"            # hardware-scaled variant: weight-scale bytes of row 1, row 2, in use
+        RA0, RA1, RB0, RB1, SRD0 = "%[ard0]", "%[ard1]", "%[brd0]", "%[brd1]", "%[srd]"
+    else:
+        ACC, P, AF, WFB = 128, 96, 64, (48, 56)
+        SAN, SC, SC2, SRD = 40, 44, None, "v35"
+        WS1 = WS2 = WSCUR = "v36"
+        RA0, RA1, RB0, RB1, SRD0 = "v30", "v31", "v32", "v33", "v34"
+    # early: a stage is handed back in two parts.  Half way through a K step every wave holds the step's activation
+    # fragments in registers and has read the first half of its weight blocks, so after a barrier there the
+    # activation rows and the first half of each wave column's weight rows are requested for the step after the
+    # next; the other weight rows follow at the end of the step as before.  Every request then has about one and a
+    # half steps to land instead of one (the loop spends its waiting time at the end-of-step wait for the copies).
+    EARLY = early
+    assert not early or (nstage == 2 and ksub == 1 and not brow)
     NSTAGE = nstage
     BROW = brow                 # weight scales per row and K step (e8m0, hardware-scaled loop only) instead of per 128 rows
     assert not brow or (hw and tm == 128 and tn == 128)
@@ -54,8 +81,9 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False):
     NB = tn // waves_n // 16
     # a wave whose columns are not a multiple of 128 wide can straddle two weight-scale blocks: two scale rows
     # are loaded and each pair of 16-column blocks takes the one the set-up code selected for it
-    SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64
-    assert (tm // 8) % WAVES == 0 and (tn // 8) % WAVES == 0
+    SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64 and not wide
+    assert (tm // 8) % WAVES == 0 and ((tn // 8) % WAVES == 0 or wide)
+    assert not early or ((tn // 8 // WAVES) % 2 == 0 and (tn // waves_n // 16) % 2 == 0)
     lines = []
 
 
@@ -69,13 +97,13 @@ def b_lds(stage, sub):
     return (stage * KSUB + sub) * B_BYTES
 
 
-ACC, P, AF, SC, SAN = 128, 96, 64, 44, 40
 SCP = (44, 224, 228)        # scale products per pair of 16-column blocks when a wave straddles two weight-scale blocks
-WFB = (48, 56)
-RA0, RA1, RB0, RB1 = 30, 31, 32, 33
-SRD0, SRD = 34, 35
 SRDB0, SRDB = 37, 38        # row-scaled weights: LDS address of the lane's weight-scale dwords (half 0, half in use)
 WSN, WSC = 96, 100          # ... the dwords of this group / of the next one, one per 16-row block
+WB_EXTRA = ("s[42:43]", "s[78:79]", "s[80:81]", "s[82:83]", "s[84:85]")     # wide: weight base per copy (64 rows apart)
+
+_uid = 0
+
 
 def emit(s):
     lines.append(s)
@@ -85,22 +113,72 @@ def vr(base, n):
     return f"v[{base}:{base + n - 1}]"
 
 
-def dma(stage):
-    """Issue the global->LDS copies of one stage; the operand bases advance by one K block after each."""
+def dma(stage, part="all"):
+    """Issue the global->LDS copies of one stage; the operand bases advance by one K block after each.
+    part "mid": the activation rows and the weight copies with an even index (the first half of each wave
+    column's rows), then the activation base advances; part "end": the odd weight copies, then the weight base."""
     bbase = NSTAGE * KSUB * A_BYTES
     for sub in range(KSUB):
-        for i in range(A_BYTES // 1024 // WAVES):
-            emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
-            emit("s_nop 0")
-            emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
-        for i in range(B_BYTES // 1024 // WAVES):
+        if part in ("all", "mid"):
+            for i in range(A_BYTES // 1024 // WAVES):
+                emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
+                emit("s_nop 0")
+                emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
+        ncopies = -(-B_BYTES // 1024 // WAVES)
+        for i in range(ncopies):
+            if (part == "mid" and i % 2) or (part == "end" and i % 2 == 0):
+                continue
+            partial = WIDE and (i + 1) * WAVES * 1024 > B_BYTES       # only the first waves have rows left for this copy
+            if partial:
+                global _uid
+                _uid += 1
+                emit("s_cmp_eq_u32 s86, 0")
+                emit(f"s_cbranch_scc1 Lnobx{_uid}%=")
             emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + i * WAVES * 1024}")
             emit("s_nop 0")
-            emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
-        emit("s_add_u32 s40, s40, 128")
-        emit("s_addc_u32 s41, s41, 0")
-        emit("s_add_u32 s42, s42, 128")
-        emit("s_addc_u32 s43, s43, 0")
+            if WIDE:
+                emit(f"global_load_lds_dwordx4 %[boff0], {WB_EXTRA[i]}")
+            else:
+                emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
+            if partial:
+                emit(f"Lnobx{_uid}%=:")
+        if part in ("all", "mid"):
+            emit("s_add_u32 s40, s40, 128")
+            emit("s_addc_u32 s41, s41, 0")
+        if part in ("all", "end"):
+            for i in range(ncopies if WIDE else 1):
+                lo = int(WB_EXTRA[i][2:4])
+                emit(f"s_add_u32 s{lo}, s{lo}, 128")
+                emit(f"s_addc_u32 s{lo + 1}, s{lo + 1}, 0")
+
+
+def copies_per_part():
+    """Requests of one wave in the mid-step part and in the end-of-step part of a stage (early hand-back)."""
+    a, b = A_BYTES // 1024 // WAVES, B_BYTES // 1024 // WAVES
+    return a + (b + 1) // 2, b // 2
+
+
+def wait_copies(c, at_end, extra=""):
+    """Early hand-back: wait until the requests this point depends on have landed.  Requests return in order, so it
+    is enough to bound how many younger ones may still be out: in the steady state the two parts issued since
+    (one mid-step part and one end-of-step part).  On the last trip nothing is requested for steps past the end,
+    so fewer, or none, are younger (c = step within the trip, s50 = 1 on the last trip)."""
+    mid, end = copies_per_part()
+    steady = mid + end
+    if at_end:
+        last = {0: steady, 1: steady, 2: end, 3: 0}[c]
+    else:
+        last = {0: steady, 1: steady, 2: steady, 3: 0}[c]
+    tag = f"{'e' if at_end else 'm'}{c}"
+    if last != steady:
+        emit("s_cmp_eq_u32 s50, 1")
+        emit(f"s_cbranch_scc1 Lwl{tag}%=")
+    emit(f"s_waitcnt vmcnt({steady}){extra}")
+    if last != steady:
+        emit(f"s_branch Lwj{tag}%=")
+        emit(f"Lwl{tag}%=:")
+        emit(f"s_waitcnt vmcnt({last}){extra}")
+        emit(f"Lwj{tag}%=:")
 
 
 def scale_group_copy(tag):
@@ -128,19 +206,23 @@ def weight_scale_load():
         emit("s_load_dword s60, s[46:47], 0x0")          # four e8m0 bytes = four K steps
         emit("s_add_u32 s46, s46, 4")
         emit("s_addc_u32 s47, s47, 0")
+        if WIDE:
+            emit("s_load_dword s68, s[72:73], 0x0")
+            emit("s_add_u32 s72, s72, 4")
+            emit("s_addc_u32 s73, s73, 0")
         return
     emit("s_load_dwordx4 s[60:63], s[46:47], 0x0")
     emit("s_add_u32 s46, s46, 16")
     emit("s_addc_u32 s47, s47, 0")
-    if SPLIT:
+    if SPLIT or WIDE:
         emit("s_load_dwordx4 s[68:71], s[72:73], 0x0")
         emit("s_add_u32 s72, s72, 16")
         emit("s_addc_u32 s73, s73, 0")
 
 
 def read_frag(dst, addr0, addr1, off):
-    emit(f"ds_read_b128 {vr(dst, 4)}, v{addr0} offset:{off}")
-    emit(f"ds_read_b128 {vr(dst + 4, 4)}, v{addr1} offset:{off}")
+    emit(f"ds_read_b128 {vr(dst, 4)}, {addr0} offset:{off}")
+    emit(f"ds_read_b128 {vr(dst + 4, 4)}, {addr1} offset:{off}")
 
 
 def read_scales(col):
@@ -149,13 +231,21 @@ def read_scales(col):
     if HW:
         if col == 0:
             for mb in range(MB):
-                emit(f"ds_read_b32 v{SC + mb}, v{SRD} offset:{mb * 64}")
+                emit(f"ds_read_b32 v{SC + mb}, {SRD} offset:{mb * 64}")
             if BROW:
                 for nb in range(NB):
                     emit(f"ds_read_b32 v{WSC + nb}, v{SRDB} offset:{nb * 64}")
         return
     for mb in range(MB):
-        emit(f"ds_read_b32 v{SAN + mb}, v{SRD} offset:{mb * 256 + col * 4}")
+        emit(f"ds_read_b32 v{SAN + mb}, {SRD} offset:{mb * 256 + col * 4}")
+
+
+def par(c, nb):
+    """Which of the two weight-fragment / result buffers block nb of step c uses.  They alternate from block to block,
+    across step boundaries too: with an odd number of blocks the first block of the next step (whose fragment is read
+    while the last block of this step still computes) must not land in that block's buffer.  Four steps per trip
+    make the pattern repeat from trip to trip."""
+    return (c * NB + nb) & 1
 
 
 def mfma(nb, mb, c=0):
@@ -163,19 +253,19 @@ def mfma(nb, mb, c=0):
         # scales applied by the matrix core: byte c of the weight-scale register (uniform) and of the lane's
         # activation-scale register; accumulation in place
         acc = vr(ACC + 16 * nb + 4 * mb, 4)
-        wscale = f"v{WSN + nb}" if BROW else "v36"
-        emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, {wscale}, v{SAN + mb} "
+        wscale = f"v{WSN + nb}" if BROW else WSCUR
+        emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[par(c, nb)], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, {wscale}, v{SAN + mb} "
              f"op_sel:[{c & 1},{c & 1},0] op_sel_hi:[{c >> 1},{c >> 1},0]")
         return
-    emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * (nb & 1) + 4 * mb, 4)}, {vr(WFB[nb & 1], 8)}, {vr(AF + 8 * mb, 8)}, 0")
+    emit(f"v_mfma_f32_16x16x128_f8f6f4 {vr(P + 16 * par(c, nb) + 4 * mb, 4)}, {vr(WFB[par(c, nb)], 8)}, {vr(AF + 8 * mb, 8)}, 0")
 
 
-def fold(nb, mb):
+def fold(nb, mb, c=0):
     if HW:
         return
     sc = SCP[nb >> 1] if SPLIT else SC
     for r in range(4):
-        emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * (nb & 1) + 4 * mb + r}, v{sc + mb}")
+        emit(f"v_fmac_f32 v{ACC + 16 * nb + 4 * mb + r}, v{P + 16 * par(c, nb) + 4 * mb + r}, v{sc + mb}")
 
 
 def step(c):
@@ -205,6 +295,10 @@ def step(c):
     else:
         for mb in range(MB):
             emit(f"v_mul_f32 v{SC + mb}, s{56 + c}, v{SAN + mb}")
+            if WIDE:
+                emit(f"v_mul_f32 v{SC2 + mb}, s{64 + c}, v{SAN + mb}")
+    if HW and WIDE:
+        emit(f"v_mov_b32 {WSCUR}, {WS1}")
     if c == 0:
         # next group of scales: into the other half of the scale buffer
         emit("s_cmp_eq_u32 s50, 1")
@@ -216,18 +310,32 @@ def step(c):
     if c == 3:
         # the next step belongs to the next group
         emit(f"s_xor_b32 s55, s55, {SCL_HALF}")
-        emit(f"v_add_u32 v{SRD}, s55, v{SRD0}")
+        emit(f"v_add_u32 {SRD}, s55, {SRD0}")
         if BROW:
             emit(f"v_add_u32 v{SRDB}, s55, v{SRDB0}")
-    read_frag(WFB[1], RB0, RB1, boff + 2048)
+    read_frag(WFB[par(c, 1)], RB0, RB1, boff + 2048)
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
     for mb in range(MB):
         emit(f"s_waitcnt lgkmcnt({8 - 2 * mb})")
         mfma(0, mb, c)
     read_scales((c + 1) & 3)
     for nb in range(1, NB):
+        if HW and WIDE:
+            # from the first block in the second weight-scale block on, the matrix instructions take that row's bytes
+            emit(f"s_cmp_eq_u32 s74, {nb}")
+            emit(f"s_cbranch_scc0 Lsw{c}_{nb}%=")
+            emit(f"v_mov_b32 {WSCUR}, {WS2}")
+            emit(f"Lsw{c}_{nb}%=:")
+        # Early hand-back: the barrier sits in front of the first read of the second weight half (block NB / 2, read
+        # one block ahead), so that half is known to have landed before anyone reads it, and behind every wave's
+        # last read of the first half, so those rows and the activation rows can be requested again right after it.
+        handback = EARLY and nb == NB // 2 - 1
+        if handback:
+            assert nb + 1 < NB
+            wait_copies(c, False, " lgkmcnt(0)")
+            emit("s_barrier")
         if nb + 1 < NB:
-            read_frag(WFB[(nb + 1) & 1], RB0, RB1, boff + (nb + 1) * 2048)
+            read_frag(WFB[par(c, nb + 1)], RB0, RB1, boff + (nb + 1) * 2048)
         if nb == 1:
             pending = 4 if (not HW or c == 3) else 0                # scale reads issued after block 0
             if BROW and c == 3:
@@ -238,7 +346,9 @@ def step(c):
         if nb + 1 == NB:
             if flip:
                 # every wave has read all of this stage and its share of the next stage has landed
-                if NSTAGE == 2:
+                if EARLY:
+                    wait_copies(c, True, " lgkmcnt(0)")
+                elif NSTAGE == 2:
                     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
                 else:
                     # four stages: the copies of the two steps after the next one may stay in flight (the group's
@@ -259,10 +369,19 @@ def step(c):
                 emit("s_barrier")
             else:
                 emit("s_waitcnt lgkmcnt(0)")
-            read_frag(WFB[0], RB0, RB1, nboff)
+            read_frag(WFB[par(c + 1, 0)], RB0, RB1, nboff)
         for mb in range(MB):
             mfma(nb, mb, c)
-            fold(nb - 1, mb)
+            fold(nb - 1, mb, c)
+            if handback and mb == 0:
+                # the activation rows and the first weight half of the step after the next, into the rows just freed
+                cond = c + 1 + KSUB >= 4
+                if cond:
+                    emit("s_cmp_eq_u32 s50, 1")
+                    emit(f"s_cbranch_scc1 Lnodmam{c}%=")
+                dma(stage, "mid")
+                if cond:
+                    emit(f"Lnodmam{c}%=:")
             if nb + 1 == NB:
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
                 if mb == 0 and flip:
@@ -271,12 +390,20 @@ def step(c):
                     if cond:
                         emit("s_cmp_eq_u32 s50, 1")
                         emit(f"s_cbranch_scc1 Lnodma{c}%=")
-                    dma(stage)
+                    dma(stage, "end" if EARLY else "all")
                     if cond:
                         emit(f"Lnodma{c}%=:")
+        if WIDE and not HW:
+            # the folds of block nb follow (in the next block's shadow): if it is the first block in the second
+            # weight-scale block, they and all later ones use that row's products
+            emit(f"s_cmp_eq_u32 s74, {nb}")
+            emit(f"s_cbranch_scc0 Lsw{c}_{nb}%=")
+            for mb in range(MB):
+                emit(f"v_mov_b32 v{SC + mb}, v{SC2 + mb}")
+            emit(f"Lsw{c}_{nb}%=:")
     # fold of the last block: the 12 folds of mb 0..2 separate the last MFMA from the read of its result
     for mb in range(MB):
-        fold(NB - 1, mb)
+        fold(NB - 1, mb, c)
 
 
 def generate():
@@ -289,13 +416,22 @@ def generate():
         emit("s_mov_b64 s[72:73], %[bsptr2]")
         emit("s_mov_b32 s74, %[sel1]")
         emit("s_mov_b32 s75, %[sel2]")
+    if WIDE:
+        emit("s_mov_b64 s[72:73], %[bsptr2]")
+        emit("s_mov_b32 s74, %[splitnb]")
+        emit("s_mov_b32 s86, %[bextra]")
+        for i in range(1, len(WB_EXTRA)):                 # weight base of copy i: 64 rows further on
+            lo, prev = int(WB_EXTRA[i][2:4]), int(WB_EXTRA[i - 1][2:4])
+            emit(f"s_add_u32 s{lo}, s{prev}, %[bstride]")
+            emit(f"s_addc_u32 s{lo + 1}, s{prev + 1}, 0")
     emit("s_mov_b32 s48, %[m0base]")
     emit("s_mov_b32 s49, %[trips]")
     emit("s_mov_b32 s53, %[copies]")
     emit("s_mov_b32 s54, 0")
     emit("s_mov_b32 s55, 0")
     for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
-        emit(f"v_mov_b32 v{reg}, %[{name}]")
+        if not reg.startswith("%"):
+            emit(f"v_mov_b32 {reg}, %[{name}]")
     if BROW:
         emit("s_mov_b32 s51, %[sdst]")
         emit(f"v_mov_b32 v{SRDB0}, %[srdb]")
@@ -304,8 +440,19 @@ def generate():
         emit(f"v_mov_b32 v{ACC + r}, 0")
     scale_group_copy("a")
     weight_scale_load()
-    dma(0)
-    if NSTAGE == 2:
+    if EARLY:
+        # both stages are requested in the order of the steady state (mid part, end part), then stage 0 and the
+        # scale group (older) are waited for: what may stay out is exactly what the first waits of the loop allow
+        for st in range(2):
+            dma(st, "mid")
+            dma(st, "end")
+        emit(f"s_waitcnt vmcnt({sum(copies_per_part())}) lgkmcnt(0)")
+        emit("s_barrier")
+    else:
+        dma(0)
+    if EARLY:
+        pass
+    elif NSTAGE == 2:
         emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
         emit("s_barrier")
         dma(1)                               # K >= 512: there are at least four steps, which two stages hold at most
@@ -316,7 +463,7 @@ def generate():
         emit(f"s_waitcnt vmcnt({(NSTAGE - 1) * per}) lgkmcnt(0)")
         emit("s_barrier")
     for mb in range(MB):
-        emit(f"ds_read_b32 v{(SC if HW else SAN) + mb}, v{SRD} offset:{mb * (64 if HW else 256)}")
+        emit(f"ds_read_b32 v{(SC if HW else SAN) + mb}, {SRD} offset:{mb * (64 if HW else 256)}")
     if BROW:
         for nb in range(NB):
             emit(f"ds_read_b32 v{WSC + nb}, v{SRDB} offset:{nb * 64}")
@@ -334,10 +481,12 @@ def generate():
             for nb in range(NB):
                 emit(f"v_mov_b32 v{WSN + nb}, v{WSC + nb}")
         else:
-            emit("v_mov_b32 v36, s60")
+            emit(f"v_mov_b32 {WS1}, s60")
+            if WIDE:
+                emit(f"v_mov_b32 {WS2}, s68")
     emit("s_mov_b64 s[56:57], s[60:61]")
     emit("s_mov_b64 s[58:59], s[62:63]")
-    if SPLIT:
+    if SPLIT or WIDE:
         emit("s_mov_b64 s[64:65], s[68:69]")
         emit("s_mov_b64 s[66:67], s[70:71]")
     emit("s_sub_u32 s49, s49, 1")
@@ -358,7 +507,10 @@ def main():
     here = os.path.dirname(os.path.abspath(__file__))
     for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
-                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True)), ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
+                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True)),
+                      ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
+                      ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, False, True)),
+                      ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)

@@ -1,6 +1,6 @@
 """Index arithmetic of the GEMM's staged bf16 epilogue (StagedEpilogue in csrc/gemm_fp8_big.hip), restated on the
 host: what a wave writes into its staging region per accumulator block and what it reads back per pass must cover
-every element of the 64-row wave tile exactly once, at aligned offsets inside the region, for the three wave-tile
+every element of the 64-row wave tile exactly once, at aligned offsets inside the region, for the four wave-tile
 widths in use.  A mistake here would show on the GPU as wrong results at best and as an out-of-range access at
 worst, so it is checked where a mistake costs nothing."""
 import pytest
@@ -9,12 +9,12 @@ import pytest
 def layout(cols):
     pitch = cols * 2 + 16
     chunks = cols // 8
-    lpr = 16 if chunks > 8 else 8
-    return {"pitch": pitch, "wave_bytes": 64 * pitch, "chunks": chunks, "lpr": lpr, "passes": 64 // (64 // lpr)}
+    return {"pitch": pitch, "wave_bytes": 64 * pitch, "chunks": chunks, "passes": chunks}
 
 
 @pytest.mark.parametrize(("cols", "waves", "lds_bytes"), [(128, 8, 2 * (256 + 256) * 128 + 2 * 256 * 16),      # 256 x 256 tile
                                                           (96, 8, 2 * (256 + 192) * 128 + 2 * 256 * 16),       # 256 x 192 tile
+                                                          (144, 8, 8 * 64 * (144 * 2 + 16)),                   # 256 x 288 tile: LDS sized for it
                                                           (64, 4, 2 * (128 + 128) * 128 + 2 * 128 * 16)])      # 128 x 128 tile
 def test_staged_epilogue_mapping(cols, waves, lds_bytes):
     L = layout(cols)
@@ -32,9 +32,7 @@ def test_staged_epilogue_mapping(cols, waves, lds_bytes):
     seen = set()
     for p in range(L["passes"]):
         for lane in range(64):
-            row, chunk = p * (64 // L["lpr"]) + lane // L["lpr"], lane % L["lpr"]
-            if chunk >= L["chunks"]:
-                continue
+            row, chunk = (p * 64 + lane) // L["chunks"], (p * 64 + lane) % L["chunks"]
             off = row * L["pitch"] + chunk * 16
             assert off % 16 == 0 and off + 16 <= L["wave_bytes"] and 0 <= row < 64
             for j in range(8):
@@ -46,7 +44,7 @@ def test_staged_epilogue_mapping(cols, waves, lds_bytes):
 
 def test_staged_epilogue_bank_spread():
     """The 8-byte writes of one instruction (16 rows x 4 lanes) touch each LDS bank at most twice."""
-    for cols in (128, 96, 64):
+    for cols in (144, 128, 96, 64):
         L = layout(cols)
         for nb in range(cols // 16):
             hits = {}

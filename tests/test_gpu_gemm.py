@@ -71,8 +71,10 @@ DENSE_SHAPES = [
     # between the 256 x 256 and the 128 x 128 kernel (576 tiles on 256 CUs)
     (333, 8320, 512), (200, 16384, 256), (2048, 4224, 384), (256, 32768, 128), (1000, 9216, 640),
     (2048, 18432, 512), (4096, 4096, 1024), (1024, 16384, 1536), (32, 128, 7168), (48, 16384, 2048), (64, 2048, 7168),
+    # N = 18432 = 64 x 288: the 256 x 288 tile kernel (512 tiles for 2048 rows, two full rounds), ragged M
+    (2048, 18432, 1024), (1900, 18432, 2048),
     # the column split in one launch (256 x 256 tiles, then K-split 128 x 128 tiles): K a multiple of 1024, ragged M
-    (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024),
+    (3000, 12800, 1024), (2048, 9472, 1024), (1900, 9472, 2048),
     # at most 16 rows: one workgroup per 16 weight rows over the whole of K (ragged K-block runs, M < 16, one K block)
     (16, 4096, 7168), (1, 4096, 7168), (5, 3072, 2048), (16, 7168, 2560), (13, 18432, 128), (16, 3200, 6528),
     # 17 to 64 rows: the same cut with separate rings for weights and activations (2, 3, 4 row groups)
@@ -93,7 +95,7 @@ def test_gemm_dense(G, shape, pow2):
 
 @pytest.mark.parametrize("shape", [(2048, 2048, 7168), (300, 2048, 1024), (129, 1280, 2560), (1000, 4096, 512), (513, 18432, 1024),
                                    (2048, 18432, 512), (777, 4224, 1536), (257, 19200, 512), (64, 24576, 1536), (16, 4096, 2048),
-                                   (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024)],
+                                   (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024), (2048, 9472, 1024)],
                          ids=lambda s: "M%d_N%d_K%d" % s)
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_gemm_bf16_output_is_the_rounded_fp32_output(G, shape, pow2):
@@ -410,7 +412,7 @@ def test_gemm_column_split_one_launch_equals_two_launches(G):
     import subprocess
     import sys
     say("gemm column split: one launch against two (LP_GEMM_MIXED=0 in a child process)")
-    shapes = ((2048, 18432, 1024), (1900, 18432, 2048))
+    shapes = ((2048, 9472, 1024), (1900, 9472, 2048))          # 296 tiles of 256 x 256: one round and 40 left over
 
     def digests():
         out = []
@@ -438,3 +440,43 @@ def test_gemm_column_split_one_launch_equals_two_launches(G):
     assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
     theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
     assert len(theirs) == 2 * len(shapes) and theirs == digests(), (theirs, r.stdout[-800:])
+
+
+def test_gemm_wide_tile_forced_on_other_shapes(G):
+    """The 256 x 288 tile kernel is chosen by itself only where it fills whole rounds of CUs; LP_GEMM_WIDE=1 (read once
+    per process, hence the child) sends every prefill-sized problem whose N is a multiple of 288 to it: few tile
+    columns, ragged M, tile origins at all four offsets inside a weight-scale block, both scale types; with
+    power-of-two scales the result must equal the default kernels' bit for bit (same order of summation)."""
+    import hashlib
+    import os
+    import subprocess
+    import sys
+    say("gemm 256 x 288 tiles forced (LP_GEMM_WIDE=1 in a child process)")
+    shapes = ((2048, 4608, 512), (1000, 13824, 512), (333, 27648, 1024))
+    mine = []
+    for (M, N, K) in shapes:
+        xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + K, pow2=True)
+        c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+        mine.append(hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest())
+    code = (
+        "import sys, hashlib, torch\n"
+        "import gcore_lowp as G\n"
+        "sys.path.insert(0, %r)\n"
+        "from tests import test_gpu_gemm as t\n"
+        "for (M, N, K) in %r:\n"
+        "    for pow2 in (False, True):\n"
+        "        xq, xs, wq, ws = t.quantized_problem(M, N, K, seed=M + K, pow2=pow2)\n"
+        "        print('[case] 256 x 288 tiles', M, N, K, pow2, flush=True)\n"
+        "        c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())\n"
+        "        wide = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), out_dtype=torch.float32)\n"
+        "        assert torch.equal(c, wide.to(torch.bfloat16))\n"
+        "        t.check(c, t.ref_gemm(xq, xs, wq, ws), 'forced wide %%s' %% ((M, N, K),))\n"
+        "        if pow2:\n"
+        "            print('md5', hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest(), flush=True)\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), shapes)
+    env = dict(os.environ, LP_GEMM_WIDE="1", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
+    theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
+    assert theirs == mine, (theirs, mine, r.stdout[-800:])
+
