@@ -47,6 +47,17 @@ __device__ __forceinline__ bool tile_coords(int64_t b, int64_t tiles_m, int64_t 
     return true;
 }
 
+// Rows of expert e from the caller's offset table, made safe to use: both ends are clamped to [0, M_total] and a
+// decreasing pair is an empty expert, so a bad table cannot send a tile outside the operands.
+__device__ __forceinline__ int expert_rows(const int32_t *__restrict__ m_offsets, int e, int64_t M_total, int64_t &begin)
+{
+    int64_t a = m_offsets[e], b = m_offsets[e + 1];
+    a = a < 0 ? 0 : (a > M_total ? M_total : a);
+    b = b < 0 ? 0 : (b > M_total ? M_total : b);
+    begin = a;
+    return b > a ? (int)(b - a) : 0;
+}
+
 inline int64_t padded_grid(int64_t tiles_m, int64_t tiles_n)
 {
     const int64_t chunks = (tiles_m * tiles_n + CHUNK - 1) / CHUNK;

@@ -292,7 +292,7 @@ template <int SDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_grouped(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                     const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                     int scale_dtype, const int32_t *__restrict__ m_offsets, int E,
-                                                    int64_t N, int64_t K, int64_t max_mtiles, int64_t tiles_n,
+                                                    int64_t M_total, int64_t N, int64_t K, int64_t max_mtiles, int64_t tiles_n,
                                                     void *__restrict__ C, int out_dtype)
 {
     __shared__ Smem sm;
@@ -308,7 +308,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int e0 = 0; e0 < E; e0 += 256) {
         const int e = e0 + t;
         int cnt = 0;
-        if (e < E) cnt = (m_offsets[e + 1] - m_offsets[e] + TM - 1) / TM;
+        int64_t unused;
+        if (e < E) cnt = (lowp::gemm::expert_rows(m_offsets, e, M_total, unused) + TM - 1) / TM;
         scan[t] = cnt;
         __syncthreads();
         for (int off = 1; off < 256; off <<= 1) {
@@ -324,7 +325,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     if (!in_range || found_e < 0) return;
     const int e = found_e;
-    const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
+    int64_t row_begin;
+    const int64_t row_end = lowp::gemm::expert_rows(m_offsets, e, M_total, row_begin) + row_begin;
     const int64_t kblocks = K / TK;
     TileArgs ta;
     ta.Aq = Aq; ta.As = As; ta.scale_dtype = scale_dtype;
@@ -536,10 +538,10 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_grouped: problem too large");
     if (scale_dtype == LP_F32)
         hipLaunchKernelGGL(gemm_grouped<LP_F32>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, M_total, N, K, max_mtiles, tiles_n, C, out_dtype);
     else
         hipLaunchKernelGGL(gemm_grouped<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, N, K, max_mtiles, tiles_n, C, out_dtype);
+                           (const uint8_t *)Bq, Bs, scale_dtype, m_offsets, E, M_total, N, K, max_mtiles, tiles_n, C, out_dtype);
     return check_launch("lp_gemm_fp8_grouped");
 }
 

@@ -251,13 +251,14 @@ struct StagedEpilogue {
     __host__ __device__ static constexpr int read_offset(int row, int chunk) { return row * PITCH + chunk * 16; }
 };
 
-template <int TM, int TN, int KSUB, int NST = 2>
+// WN: waves side by side along N (2, or 4 for the flat 128 x 256 tile); a wave owns 64 rows x TN / WN columns.
+template <int TM, int TN, int KSUB, int NST = 2, int WN = 2>
 struct AsmTile {
-    static constexpr int WAVES = TM / 64 * 2, NBW = TN / 32;
+    static constexpr int WAVES = TM / 64 * WN, NBW = TN / WN / 16;
     static constexpr int A_BYTES = TM * KB, B_BYTES = TN * KB;                   // one K block of 128
     static constexpr int B_LDS = NST * KSUB * A_BYTES, S_LDS = NST * KSUB * (A_BYTES + B_BYTES);
     static constexpr int LOOP_BYTES = S_LDS + 2 * TM * 16;                       // NST stages of KSUB K blocks + scale groups
-    static constexpr int STAGING = WAVES * StagedEpilogue<TN / 2>::WAVE_BYTES;  // the waves' bf16 staging regions after the loop
+    static constexpr int STAGING = WAVES * StagedEpilogue<TN / WN>::WAVE_BYTES; // the waves' bf16 staging regions after the loop
     static constexpr int LDS_BYTES = LOOP_BYTES > STAGING ? LOOP_BYTES : STAGING;
 };
 
@@ -283,21 +284,23 @@ struct AsmTile {
 // check_asm_operands.py verifies both on the generated assembly at build time.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false>
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false, int WN = 2>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
 {
-    using T = AsmTile<TM, TN, KSUB, NST>;
+    using T = AsmTile<TM, TN, KSUB, NST, WN>;
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
+    static_assert(WN == 2 || (WN == 4 && TM == 128 && TN == 256 && KSUB == 1 && !DUAL && NST == 2 && !BROW), "four waves along N: the 128 x 256 tile");
     static_assert(!DUAL || (TM == 128 && TN == 128), "the K split inside a workgroup is built for the 128 x 128 tile");
     static_assert(NST == 2 || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "four stages: 128 x 128 tile only");
     static_assert(!BROW || (HWS && TM == 128 && TN == 128 && KSUB == 1 && !DUAL && NST == 2), "row-scaled weights: hardware-scaled 128 x 128 loop");
-    static_assert(TM / 8 / WAVES == 4 && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3), "copies per operand and wave");
+    static_assert((TM / 8 / WAVES == 4 || (WN == 4 && TM / 8 / WAVES == 2)) && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3),
+                  "copies per operand and wave");
     constexpr int NBC = TN / 8 / WAVES;                 // weight copies per wave and K block
     const int t = threadIdx.x, lane = t & 63, wave = DUAL ? (t >> 6) & (WAVES - 1) : t >> 6;
     const int kg = DUAL ? __builtin_amdgcn_readfirstlane(t >> 6) / WAVES : 0;                 // which half of K
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int l16 = lane & 15, lq = lane >> 4;
     const uint32_t kblocks = (uint32_t)(K / KB);
     const uint32_t trips = (DUAL ? kblocks / 2 : kblocks) / 4;
@@ -341,12 +344,12 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t copies = __builtin_amdgcn_readfirstlane(BROW || wave < TM / 64 ? 1u : 0u);
     // weight scale row(s) of this wave.  With TN / 2 = 128 or 64 columns per wave they lie in one scale block;
     // 96 columns can straddle two, and each pair of 16-column blocks is told which of the two rows it uses.
-    const int64_t wcol0 = n0 + wn * (TN / 2);
+    const int64_t wcol0 = n0 + wn * (TN / WN);
     const int64_t last_blk = (N >> 7) - 1;
     int64_t sblk = wcol0 >> 7;
     if (sblk > last_blk) sblk = last_blk;
     const uint64_t bs_u = uniform((const char *)Bs + sblk * kblocks * SS);
-    int64_t sblk2 = (wcol0 + TN / 2 - 1) >> 7;
+    int64_t sblk2 = (wcol0 + TN / WN - 1) >> 7;
     if (sblk2 > last_blk) sblk2 = last_blk;
     const uint64_t bs2_u = uniform((const char *)Bs + sblk2 * kblocks * SS);
     // pair p covers columns wcol0 + 32 p .. + 31 (within one scale block since wcol0 is a multiple of 32)
@@ -364,7 +367,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     // Layout: activation stages, weight stages, scale groups.
     const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
     const uint32_t m0base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
-    const int arow_l = wm * 64 + l16, brow_l = wn * (TN / 2) + l16;
+    const int arow_l = wm * 64 + l16, brow_l = wn * (TN / WN) + l16;
     const uint32_t ard0 = lds0 + arow_l * KB + swz(arow_l, 2 * lq) * 16;
     const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
     const uint32_t brd0 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq) * 16;
@@ -399,6 +402,24 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4;
         accs[5] = acc5; accs[6] = acc6; accs[7] = acc7; accs[8] = acc8;
+    } else if constexpr (WN == 4) {
+        // the early hand-back of this loop splits the weight copies by wave: the first four copy each wave column's first half
+        const uint32_t lohalf = __builtin_amdgcn_readfirstlane(wave < WAVES / 2 ? 1u : 0u);
+        f32x16v acc0, acc1, acc2, acc3;
+        if constexpr (HWS) {
+            asm volatile(
+#include "gemm_flat_hw_loop.inc"
+                : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_CLOBBERS, "s87");
+        } else {
+            asm volatile(
+#include "gemm_flat_loop.inc"
+                : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_CLOBBERS, "s87");
+        }
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     } else if constexpr (HWS && NBW == 8) {
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
         asm volatile(
@@ -497,7 +518,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         }
     }
     if constexpr (STAGED) {
-        using E = StagedEpilogue<TN / 2>;
+        using E = StagedEpilogue<TN / WN>;
         static_assert(WAVES * E::WAVE_BYTES <= T::LDS_BYTES, "the waves' staging regions must fit the tile's LDS");
         if (out_dtype == LP_BF16) {
             // DUAL: only the first K half's waves are left; they stage in their own half's stage memory, which every
@@ -639,8 +660,8 @@ __global__ __launch_bounds__(256) void gemm_asm_rowscale(const uint8_t *__restri
 template <int TM, int TN, int KSUB, int PART, bool HWS = false>
 __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                            const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
-                                                           const int32_t *__restrict__ m_offsets, int E, int64_t N,
-                                                           int64_t K, int64_t max_mtiles, int64_t tiles_n,
+                                                           const int32_t *__restrict__ m_offsets, int E, int64_t M_total,
+                                                           int64_t N, int64_t K, int64_t max_mtiles, int64_t tiles_n,
                                                            void *__restrict__ C, int out_dtype)
 {
     constexpr int NT = TM * 2;
@@ -661,7 +682,8 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
     int base = 0;
     for (int e0 = 0; e0 < E; e0 += NT) {
         const int e = e0 + t;
-        const int cnt = e < E ? tiles_of(m_offsets[e + 1] - m_offsets[e]) : 0;
+        int64_t unused;
+        const int cnt = e < E ? tiles_of(gemm::expert_rows(m_offsets, e, M_total, unused)) : 0;
         int incl = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -684,12 +706,106 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
     }
     if (!in_range || found_e < 0) return;
     const int e = found_e;
-    const int64_t row_begin = m_offsets[e], row_end = m_offsets[e + 1];
+    int64_t row_begin;
+    const int64_t row_end = gemm::expert_rows(m_offsets, e, M_total, row_begin) + row_begin;
     const int64_t first = PART == 2 ? row_begin + (row_end - row_begin) / 256 * 256 : row_begin;
     const int64_t kblocks = K / KB;
     const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
     tile_asm<TM, TN, KSUB, HWS, false, 2, false, true>(smem, Aq, As, Bq + (int64_t)e * N * K, bs_e, first + (gmt - found_first) * TM, row_end,
                                 tn * TN, N, K, C, N, out_dtype);
+}
+
+// Grouped problem in ONE launch with two tile heights.  Every 256 rows of an expert, and a remainder of more than 128
+// rows, go to a 256 x 256 tile (class "big"); a remainder of 1 .. 128 rows goes to a 128 x 256 tile (class "small": eight
+// waves as 2 x 4, half the activation rows per step for the same 256 weight rows).  What a tile costs a CU is mostly the
+// bytes it pulls through the L2 -> LDS copies, and an expert with few rows is a stream of its weights: the flat tile
+// moves 48 KB per K step and 256 weight rows where two 128 x 128 tiles move 64 KB.
+// The tile list is built on the device from m_offsets (at most 512 experts): one scan gives every thread the two class
+// totals and the running tile counts of its expert, from which the workgroup finds its class, its tile and the expert
+// that owns it.  Within every XCD's sequence of workgroup ids the two classes are dealt in the ratio of their sizes
+// (1 big : ps small), and each class keeps the 8(M) x 4(N) blocks of neighbouring tiles per XCD that let operand panels
+// be re-used out of one L2.
+constexpr int kMixedMaxExperts = 512;
+
+__device__ __forceinline__ int64_t dev_padded_grid(int64_t tiles_m, int64_t tiles_n)
+{
+    const int64_t chunks = (tiles_m * tiles_n + gemm::CHUNK - 1) / gemm::CHUNK;
+    return ((chunks + 7) / 8) * 8 * gemm::CHUNK;
+}
+
+template <bool HWS>
+__global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                              const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                              const int32_t *__restrict__ m_offsets, int E, int64_t M_total,
+                                                              int64_t N, int64_t K, void *__restrict__ C, int out_dtype)
+{
+    constexpr int LDS_BIG = AsmTile<256, 256, 1>::LDS_BYTES, LDS_FLAT = AsmTile<128, 256, 1, 2, 4>::LDS_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BIG > LDS_FLAT ? LDS_BIG : LDS_FLAT];
+    __shared__ int wave_big[8], wave_small[8];
+    __shared__ int found_e, found_first, found_begin, found_rows;
+    const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+    // ---- this thread's expert: rows, tiles of both classes, running counts over the experts before it
+    int64_t begin = 0;
+    const int rows = t < E ? gemm::expert_rows(m_offsets, t, M_total, begin) : 0;
+    const int rem = rows & 255;
+    const int nb = (rows >> 8) + (rem > 128 ? 1 : 0), ns = rem > 0 && rem <= 128 ? 1 : 0;
+    int ib = nb, is = ns;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int ub = __shfl_up(ib, off), us = __shfl_up(is, off);
+        if (lane >= off) { ib += ub; is += us; }
+    }
+    if (lane == 63) { wave_big[wv] = ib; wave_small[wv] = is; }
+    if (t == 0) found_e = -1;
+    __syncthreads();
+    int tot_big = 0, tot_small = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        const int vb = wave_big[w], vs = wave_small[w];
+        if (w < wv) { ib += vb; is += vs; }
+        tot_big += vb;
+        tot_small += vs;
+    }
+    // ---- which class and which tile of it this workgroup takes
+    const int64_t tiles_n = N >> 8;
+    const int64_t slots_big = dev_padded_grid(tot_big, tiles_n) >> 3, slots_small = dev_padded_grid(tot_small, tiles_n) >> 3;
+    const int64_t xcd = blockIdx.x & 7, sidx = blockIdx.x >> 3;
+    if (sidx >= slots_big + slots_small) return;
+    int64_t ps = slots_big > 0 ? (slots_small + slots_big / 2) / slots_big : 1;
+    if (ps < 1) ps = 1;
+    const int64_t period = 1 + ps;
+    const int64_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
+    bool big;
+    int64_t idx;
+    if (sidx < rounds * period) {
+        const int64_t r = sidx % period, q = sidx / period;
+        big = r == 0;
+        idx = big ? q : q * ps + (r - 1);
+    } else {
+        const int64_t w = sidx - rounds * period, left_big = slots_big - rounds;
+        big = w < left_big;
+        idx = big ? rounds + w : rounds * ps + (w - left_big);
+    }
+    int64_t gmt, tn;
+    if (!gemm::tile_coords(idx * 8 + xcd, big ? tot_big : tot_small, tiles_n, gmt, tn)) return;
+    // ---- the expert that owns m-tile gmt of the class tells the others
+    {
+        const int cnt = big ? nb : ns, incl = big ? ib : is;
+        if (gmt >= incl - cnt && gmt < incl) { found_e = t; found_first = incl - cnt; found_begin = (int)begin; found_rows = rows; }
+    }
+    __syncthreads();
+    if (found_e < 0) return;
+    const int e = found_e;
+    const int64_t row_begin = found_begin, row_end = row_begin + found_rows, kblocks = K / KB;
+    const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
+    const uint8_t *bq_e = Bq + (int64_t)e * N * K;
+    const int64_t local = gmt - found_first;
+    if (big)
+        tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, bq_e, bs_e, row_begin + local * 256, row_end, tn * 256, N, K, C, N,
+                                                          out_dtype);
+    else
+        tile_asm<128, 256, 1, HWS, false, 2, false, true, 4>(smem, Aq, As, bq_e, bs_e, row_begin + (found_rows >> 8) * 256, row_end, tn * 256,
+                                                             N, K, C, N, out_dtype);
 }
 
 template <int SDT, int NB>
@@ -917,13 +1033,34 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
                        const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype,
                        hipStream_t st)
 {
+    static const char *force = getenv("LP_GEMM_GROUPED_MODE");          // tuning aid: 0 = 128 tiles, 1 = 256 + 128 in two launches, 2 = one mixed launch
+    const int mode = force ? atoi(force) : -1;
+    // One launch with both tile heights when the experts are not all tiny (with fewer than 128 rows per expert on
+    // average hardly any 256-row tile exists and the 128 x 128 kernel, two workgroups per CU, streams weights as well)
+    // and K is long: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden
+    // behind a second workgroup, and at K = 2048 (16 steps) that costs what the larger tiles gain (config 4, down
+    // projection: 1.64 ms against 1.59 with fp32 scales, 1.49 against 1.51 with e8m0).
+    // An expert has at most one small tile, and M_e / 256 big ones plus one when more than 128 rows are left over.
+    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 4096)) {
+        const int64_t grid = padded_grid((M_total + 128 * (int64_t)E) / 256 + 1, N / 256) + padded_grid(E, N / 256);
+        if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
+        if (E <= kMixedMaxExperts) {
+            if (scale_dtype == LP_E8M0)
+                hipLaunchKernelGGL((gemm_asm_grouped_mixed<true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype);
+            else
+                hipLaunchKernelGGL((gemm_asm_grouped_mixed<false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype);
+            return check_launch("lp_gemm_fp8_grouped(asm mixed heights)");
+        }
+    }
     if (scale_dtype == LP_E8M0) {
         // e8m0 scales: 128 x 128 tiles on the kernel whose matrix instructions apply the scales
         const int64_t mtiles = M_total / 128 + E;
         const int64_t grid = padded_grid(mtiles, N / 128);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 0, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
-                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, mtiles, N / 128, C,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, mtiles, N / 128, C,
                            out_dtype);
         return check_launch("lp_gemm_fp8_grouped(asm 128 e8m0)");
     }
@@ -932,14 +1069,13 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
     // of the expert list) let streaming tiles and compute-bound tiles overlap and bound the padding per expert
     // by 127 rows.  With many rows per expert the 256 x 256 kernel takes the full 256-row tiles and the
     // 128 x 128 kernel what is left.
-    static const char *force = getenv("LP_GEMM_GROUPED_MODE");          // tuning aid: 0 = 128 tiles, 1 = 256 + 128
-    const bool split = force ? atoi(force) == 1 : M_total >= (int64_t)E * 1024;
+    const bool split = mode >= 0 ? mode == 1 : M_total >= (int64_t)E * 1024;
     if (split) {
         const int64_t big_mtiles = M_total / 256;
         const int64_t grid = padded_grid(big_mtiles, N / 256);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         hipLaunchKernelGGL((gemm_asm_grouped<256, 256, 1, 1>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
-                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, big_mtiles, N / 256,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, big_mtiles, N / 256,
                            C, out_dtype);
         const int rc = check_launch("lp_gemm_fp8_grouped(asm 256)");
         if (rc) return rc;
@@ -948,7 +1084,7 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
         const int64_t grid2 = padded_grid(rest_mtiles, N / 128);
         if (grid2 > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 2>), dim3((unsigned)grid2), dim3(256), 0, st, (const uint8_t *)Aq,
-                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, rest_mtiles, N / 128,
+                           (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, rest_mtiles, N / 128,
                            C, out_dtype);
         return check_launch("lp_gemm_fp8_grouped(asm 128)");
     }
@@ -956,7 +1092,7 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
     const int64_t grid = padded_grid(mtiles, N / 128);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
     hipLaunchKernelGGL((gemm_asm_grouped<128, 128, 1, 0>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq,
-                       (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, N, K, mtiles, N / 128, C,
+                       (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, mtiles, N / 128, C,
                        out_dtype);
     return check_launch("lp_gemm_fp8_grouped(asm 128)");
 }

@@ -40,8 +40,12 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT
     HW = hw
+    # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
+    # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
+    # weight copies by wave (s87 = 1 for the first half of the waves) instead of by copy index.
+    HALFSPLIT = early and tn // waves_n == 64
     # wide: a wave owns 64 x 144 columns (nine 16-column blocks), e.g. the 256 x 288 tile that cuts 18432 weight rows
     # into exactly 64 tile columns.  144 columns always straddle two weight-scale blocks, at a 16-column boundary known
     # only at run time (s74 = first block that takes the second scale row): the folds read one set of scale products,
@@ -84,6 +88,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64 and not wide
     assert (tm // 8) % WAVES == 0 and ((tn // 8) % WAVES == 0 or wide)
     assert not early or ((tn // 8 // WAVES) % 2 == 0 and (tn // waves_n // 16) % 2 == 0)
+    assert not HALFSPLIT or WAVES == 8
     lines = []
 
 
@@ -125,12 +130,16 @@ def dma(stage, part="all"):
                 emit("s_nop 0")
                 emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
         ncopies = -(-B_BYTES // 1024 // WAVES)
+        if HALFSPLIT and part != "all":
+            global _uid
+            _uid += 1
+            emit(f"s_cmp_eq_u32 s87, {0 if part == 'mid' else 1}")          # mid: the first four waves copy, end: the others
+            emit(f"s_cbranch_scc1 Lnoh{_uid}%=")
         for i in range(ncopies):
-            if (part == "mid" and i % 2) or (part == "end" and i % 2 == 0):
+            if not HALFSPLIT and ((part == "mid" and i % 2) or (part == "end" and i % 2 == 0)):
                 continue
             partial = WIDE and (i + 1) * WAVES * 1024 > B_BYTES       # only the first waves have rows left for this copy
             if partial:
-                global _uid
                 _uid += 1
                 emit("s_cmp_eq_u32 s86, 0")
                 emit(f"s_cbranch_scc1 Lnobx{_uid}%=")
@@ -142,6 +151,8 @@ def dma(stage, part="all"):
                 emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
             if partial:
                 emit(f"Lnobx{_uid}%=:")
+        if HALFSPLIT and part != "all":
+            emit(f"Lnoh{_uid}%=:")
         if part in ("all", "mid"):
             emit("s_add_u32 s40, s40, 128")
             emit("s_addc_u32 s41, s41, 0")
@@ -155,6 +166,10 @@ def dma(stage, part="all"):
 def copies_per_part():
     """Requests of one wave in the mid-step part and in the end-of-step part of a stage (early hand-back)."""
     a, b = A_BYTES // 1024 // WAVES, B_BYTES // 1024 // WAVES
+    if HALFSPLIT:
+        # a wave issues its weight copies in one of the two parts; either way the two parts together are a + b
+        # requests, and counting none for the end part only makes the last trip's waits stricter
+        return a + b, 0
     return a + (b + 1) // 2, b // 2
 
 
@@ -424,6 +439,8 @@ def generate():
             lo, prev = int(WB_EXTRA[i][2:4]), int(WB_EXTRA[i - 1][2:4])
             emit(f"s_add_u32 s{lo}, s{prev}, %[bstride]")
             emit(f"s_addc_u32 s{lo + 1}, s{prev + 1}, 0")
+    if HALFSPLIT:
+        emit("s_mov_b32 s87, %[lohalf]")
     emit("s_mov_b32 s48, %[m0base]")
     emit("s_mov_b32 s49, %[trips]")
     emit("s_mov_b32 s53, %[copies]")
@@ -505,12 +522,14 @@ def generate():
 
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
-    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
+    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1, False, 2, False, True)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
                       ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True)),
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
                       ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, False, True)),
                       ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, False, True)),
+                      ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 2, False, True)),
+                      ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 2, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)

@@ -163,6 +163,10 @@ GROUPED = [
     (4, 256, 512, [300, 0, 255, 513]),
     (6, 512, 1024, [128, 129, 256, 257, 1, 640]),
     (5, 256, 1536, [0, 0, 7, 0, 0]),
+    # long K: one launch with 256 x 256 tiles for whole 256 rows (and left-overs above 128) and 128 x 256 tiles for the rest
+    (6, 512, 4096, [128, 129, 256, 257, 1, 640]),
+    (8, 256, 4096, [700, 0, 300, 1, 255, 256, 257, 600]),
+    (5, 768, 5120, [3, 1100, 0, 127, 385]),
 ]
 
 
@@ -192,7 +196,8 @@ def test_gemm_grouped(G, case):
 
 
 @pytest.mark.parametrize("case", [(8, 512, 512, [700, 0, 300, 1, 255, 256, 257, 600]), (4, 256, 1024, [300, 0, 255, 513]),
-                                  (3, 384, 512, [300, 0, 77])], ids=lambda c: "E%d_N%d_K%d" % c[:3])
+                                  (3, 384, 512, [300, 0, 77]), (6, 512, 4096, [128, 129, 256, 257, 1, 640]),
+                                  (5, 768, 5120, [3, 1100, 0, 127, 385])], ids=lambda c: "E%d_N%d_K%d" % c[:3])
 def test_gemm_grouped_e8m0_scales(G, case):
     """power-of-two scales on both operands: the kernels whose matrix instructions apply the scales"""
     E, N, K, m_splits = case
@@ -207,6 +212,26 @@ def test_gemm_grouped_e8m0_scales(G, case):
     out = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda())
     ref = T.grouped_gemm_fp8_ref(xq, xs.float(), wq, ws.float(), m_splits)
     check(out, ref, f"grouped e8m0 {case[:3]}")
+
+
+@pytest.mark.parametrize("K", [512, 4096], ids=["128-row-tiles", "mixed-heights"])
+def test_gemm_grouped_survives_a_bad_offset_table(G, K):
+    """Offsets that decrease or run past the rows are made harmless inside the kernels (both ends clamped to the row
+    count, a decreasing pair = an expert without rows): the call returns, experts with a sane range get their result,
+    nothing outside `out` is written (the guard rows behind it keep their fill)."""
+    E, N, M = 4, 256, 800
+    xq, xs, wq, ws = _grouped_problem(E, N, K, [M], seed=77)
+    offs = torch.tensor([0, 300, 200, 900, 5000], dtype=torch.int32)       # expert 1 "ends" before it begins, 2 and 3 overrun
+    buf = torch.full((M + 64, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    say("gemm grouped with a bad offset table, K =", K)
+    G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda(), out=buf[:M])
+    torch.cuda.synchronize()
+    assert (buf[M:] == 7.0).all()
+    # expert 0 owns rows 0 .. 299 and the clamped expert 2 rows 200 .. 799: outside the overlap each row has one owner
+    ref0 = T.grouped_gemm_fp8_ref(xq[:200], xs[:200], wq[:1], ws[:1], [200])
+    check(buf[:200], ref0, "expert 0 beside bad offsets")
+    ref2 = T.grouped_gemm_fp8_ref(xq[300:800], xs[300:800], wq[2:3], ws[2:3], [500])
+    check(buf[300:800], ref2, "expert 2 clamped to the rows that exist")
 
 
 def test_grouped_linear_module(G):
