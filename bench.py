@@ -292,6 +292,21 @@ def main():
                                       "bytes": bytes_q}
         extras["c1_dequant_128x128"] = {"ms": ms_d, "GB/s": bytes_q / ms_d / 1e6,
                                         "hbm_frac": bytes_q / ms_d / 1e6 / HBM_PEAK_GBS, "bytes": bytes_q}
+        # a bare stream of the same bytes: read 32 MiB + write 16 MiB (the quantiser's traffic) and the reverse
+        probes = {}
+        for wgs in (512, 1024, 2048, 4096):
+            fq = [(lambda i=i: chk(L.lp_probe_stream(xs[i].data_ptr(), R * C * 2, qs[i].data_ptr(), R * C, wgs, stream())))
+                  for i in range(sets)]
+            fd = [(lambda i=i: chk(L.lp_probe_stream(qs[i].data_ptr(), R * C, outs[i].data_ptr(), R * C * 2, wgs, stream())))
+                  for i in range(sets)]
+            probes[f"read32MiB_write16MiB_{wgs}_workgroups_us"] = time_launches(fq, 48, 12)[0] * 1e3
+            probes[f"read16MiB_write32MiB_{wgs}_workgroups_us"] = time_launches(fd, 48, 12)[0] * 1e3
+        bq_ = min(v for k, v in probes.items() if k.startswith("read32"))
+        bd_ = min(v for k, v in probes.items() if k.startswith("read16"))
+        probes["quant_over_bare_stream"] = ms_q * 1e3 / bq_
+        probes["dequant_over_bare_stream"] = ms_d * 1e3 / bd_
+        probes["bare_stream_hbm_frac"] = {"read32_write16": bytes_q / bq_ / 1e3 / HBM_PEAK_GBS, "read16_write32": bytes_q / bd_ / 1e3 / HBM_PEAK_GBS}
+        extras["c1_floor_probe"] = probes
         del xs, qs, ss, outs
         torch.cuda.empty_cache()
 
@@ -322,7 +337,21 @@ def main():
         extras["c3_skinny_gemm"] = {"ms": ms3, "GB/s": bytes3 / ms3 / 1e6, "hbm_frac": bytes3 / ms3 / 1e6 / HBM_PEAK_GBS,
                                     "weight_GB/s": N3 * K3 / ms3 / 1e6, "tflops": 2.0 * M3 * N3 * K3 / ms3 / 1e9,
                                     "bytes": bytes3}
-        del w3q, w3s
+        # what the box takes for an empty launch and for a bare stream of the same bytes (rotating buffers like above)
+        ms_empty, _ = time_launches([lambda: chk(L.lp_probe_stream(None, 0, None, 0, 256, stream()))], 48, 12)
+        sink = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+        wbytes = N3 * K3
+        probes = {"empty_launch_us": ms_empty * 1e3}
+        for wgs in (256, 512, 1024, 2048):
+            fns = [(lambda i=i: chk(L.lp_probe_stream(w3q[i].data_ptr(), wbytes, sink.data_ptr(), 4096 * wgs // 256, wgs, stream())))
+                   for i in range(sets)]
+            msp, _ = time_launches(fns, 48, 12)
+            probes[f"read_29MB_{wgs}_workgroups_us"] = msp * 1e3
+        best = min(v for k, v in probes.items() if k.startswith("read_"))
+        probes["read_29MB_best_GB/s"] = wbytes / best / 1e3
+        probes["skinny_gemm_over_bare_read"] = ms3 * 1e3 / best
+        extras["c3_floor_probe"] = probes
+        del w3q, w3s, sink
         torch.cuda.empty_cache()
 
     if want("c5"):

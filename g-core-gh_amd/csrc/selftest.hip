@@ -99,7 +99,44 @@ __global__ __launch_bounds__(256) void debug_cast(int kind, const float *__restr
     }
 }
 
+// Stream probe: each of the launch's workgroups reads a contiguous share of `src` with 16-byte non-temporal loads
+// (all lanes of a wave on consecutive addresses, 8 loads in flight per lane) and writes a share of `dst` with 16-byte
+// stores whose value depends on what was read, so neither side can be dropped.  No arithmetic to speak of: what
+// it takes is what the memory system and the launch take for that many bytes.
+__global__ __launch_bounds__(256) void stream_probe(const u32x4 *__restrict__ src, int64_t read_vecs, u32x4 *__restrict__ dst,
+                                                    int64_t write_vecs)
+{
+    const int64_t wgs = gridDim.x, wg = blockIdx.x;
+    const int64_t r_per = (read_vecs + wgs - 1) / wgs, w_per = (write_vecs + wgs - 1) / wgs;
+    const int64_t r0 = wg * r_per, r1 = r0 + r_per < read_vecs ? r0 + r_per : read_vecs;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (int64_t i = r0 + threadIdx.x; i < r1; i += 256 * 8) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = i + 256 * j < r1 ? __builtin_nontemporal_load(src + i + 256 * j) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { acc.x ^= v[j].x; acc.y ^= v[j].y; acc.z ^= v[j].z; acc.w ^= v[j].w; }
+    }
+    const int64_t w0 = wg * w_per, w1 = w0 + w_per < write_vecs ? w0 + w_per : write_vecs;
+    for (int64_t i = w0 + threadIdx.x; i < w1; i += 256) {
+        acc.x += 1u;
+        __builtin_nontemporal_store(acc, dst + i);
+    }
+}
+
 }  // namespace
+
+extern "C" int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t write_bytes, int workgroups, lp_stream_t stream)
+{
+    LP_REQUIRE(read_bytes >= 0 && write_bytes >= 0 && read_bytes % 16 == 0 && write_bytes % 16 == 0,
+               "lp_probe_stream: byte counts must be non-negative multiples of 16");
+    LP_REQUIRE(workgroups >= 1 && workgroups <= (1 << 20), "lp_probe_stream: 1 .. 2^20 workgroups");
+    LP_REQUIRE((read_bytes == 0 || src) && (write_bytes == 0 || dst), "lp_probe_stream: null pointer");
+    LP_REQUIRE(((uintptr_t)src | (uintptr_t)dst) % 16 == 0, "lp_probe_stream: buffers must be 16-byte aligned");
+    hipLaunchKernelGGL(stream_probe, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)src, read_bytes / 16,
+                       (u32x4 *)dst, write_bytes / 16);
+    return check_launch("lp_probe_stream");
+}
 
 extern "C" int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream)
 {

@@ -305,6 +305,16 @@ int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, int64_t col
  */
 int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream);
 
+/*
+ * Measurement aid: one launch of `workgroups` x 256 threads that reads read_bytes from src (16-byte non-temporal
+ * loads, contiguous share per workgroup) and writes write_bytes to dst (16-byte stores of a value derived from what
+ * was read).  Either count may be 0; with both 0 it is an empty launch.  It does no work the library needs: it
+ * shows what a launch and a stream of that many bytes cost on the box, next to the kernels of the same size
+ * (the benchmark times it beside the skinny GEMM's 29 MB weight stream and the 4096 x 4096 quantiser).
+ * No reference counterpart.
+ */
+int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t write_bytes, int workgroups, lp_stream_t stream);
+
 /* Bulk element-wise casts through the library's device code paths (debug aid
  * for tests): kind 0 = fp32 -> e4m3fn software, 1 = fp32 -> e4m3fn hardware
  * (inputs clamped to +-448 first), 2 = fp32 -> e8m0, 3 = fp32 -> bf16. */
