@@ -217,12 +217,13 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "s40", "s41", "s42", "s43",     \
         "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60",   \
         "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77",   \
-        "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86"
+        "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88"
 #define LP_ASM_INPUTS_WIDE                                                                                                \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
-        [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride)
+        [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
+        [g4] "s"(g4)
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
@@ -357,11 +358,13 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t sel2 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 64) >> 7) != (wcol0 >> 7)));
     (void)bs2_u; (void)sel1; (void)sel2;
     // 256 x 288 tile: first 16-column block of this wave that lies in the second weight-scale block, whether this wave has
-    // a fifth weight copy (36 blocks of 8 rows over 8 waves), distance between a wave's weight copies (64 rows)
+    // a fifth weight copy (36 groups of 8 rows over 8 waves) and which group that copy moves (16, 17 for waves 0, 1 and
+    // 34, 35 for waves 2, 3, as group g4 + wave), bytes between two groups of weight rows
     const uint32_t splitnb = __builtin_amdgcn_readfirstlane((uint32_t)(((((wcol0 >> 7) + 1) << 7) - wcol0) >> 4));
     const uint32_t bextra = __builtin_amdgcn_readfirstlane(wave < (TN / 8) % WAVES ? 1u : 0u);
-    const uint32_t bstride = __builtin_amdgcn_readfirstlane((uint32_t)(8 * WAVES * K));
-    (void)splitnb; (void)bextra; (void)bstride;
+    const uint32_t bstride = __builtin_amdgcn_readfirstlane((uint32_t)(8 * K));
+    const uint32_t g4 = __builtin_amdgcn_readfirstlane(wave < 2 ? 16u : 32u);
+    (void)splitnb; (void)bextra; (void)bstride; (void)g4;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
     // Layout: activation stages, weight stages, scale groups.

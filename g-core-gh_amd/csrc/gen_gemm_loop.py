@@ -55,7 +55,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # never clamped: N is a multiple of the tile width) with one scalar base per copy.
     WIDE = wide
     if wide:
-        assert tm == 256 and waves_m == 4 and waves_n == 2 and ksub == 1 and nstage == 2 and not brow and not early
+        assert tm == 256 and tn == 288 and waves_m == 4 and waves_n == 2 and ksub == 1 and nstage == 2 and not brow
         ACC, P, AF, WFB = 112, 80, 48, (32, 40)
         SAN, SC, SC2, SRD = 24, 28, 20, "v19"
         WS1, WS2, WSCUR = "v20", "v21", "v22"            # hardware-scaled variant: weight-scale bytes of row 1, row 2, in use
@@ -87,7 +87,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # are loaded and each pair of 16-column blocks takes the one the set-up code selected for it
     SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64 and not wide
     assert (tm // 8) % WAVES == 0 and ((tn // 8) % WAVES == 0 or wide)
-    assert not early or ((tn // 8 // WAVES) % 2 == 0 and (tn // waves_n // 16) % 2 == 0)
+    assert not early or wide or ((tn // 8 // WAVES) % 2 == 0 and (tn // waves_n // 16) % 2 == 0)
     assert not HALFSPLIT or WAVES == 8
     lines = []
 
@@ -105,7 +105,14 @@ def b_lds(stage, sub):
 SCP = (44, 224, 228)        # scale products per pair of 16-column blocks when a wave straddles two weight-scale blocks
 SRDB0, SRDB = 37, 38        # row-scaled weights: LDS address of the lane's weight-scale dwords (half 0, half in use)
 WSN, WSC = 96, 100          # ... the dwords of this group / of the next one, one per 16-row block
-WB_EXTRA = ("s[42:43]", "s[78:79]", "s[80:81]", "s[82:83]", "s[84:85]")     # wide: weight base per copy (64 rows apart)
+WB_EXTRA = ("s[42:43]", "s[78:79]", "s[80:81]", "s[82:83]", "s[84:85]")     # wide: weight base per copy
+# wide: the 36 groups of 8 weight rows are dealt to the waves so that the early hand-back can request the first 64 rows of
+# both wave columns (groups 0..7 and 18..25: the rows blocks 0..3 read) half way through a step and the other 80 rows of
+# each at its end.  Copy i of wave w moves group WIDE_GROUP[i] + w; the fifth copy exists for waves 0..3 only and moves
+# groups 16, 17 (waves 0, 1) and 34, 35 (waves 2, 3): its group comes in s88 (as an LDS offset) and its base in s[84:85].
+# All group numbers have the parity of w, so one per-lane source offset (row 8 w + lane / 8, swizzled chunk) serves all.
+WIDE_GROUP = (0, 18, 8, 26, None)
+WIDE_PART = ("mid", "mid", "end", "end", "end")
 
 _uid = 0
 
@@ -136,14 +143,23 @@ def dma(stage, part="all"):
             emit(f"s_cmp_eq_u32 s87, {0 if part == 'mid' else 1}")          # mid: the first four waves copy, end: the others
             emit(f"s_cbranch_scc1 Lnoh{_uid}%=")
         for i in range(ncopies):
-            if not HALFSPLIT and ((part == "mid" and i % 2) or (part == "end" and i % 2 == 0)):
+            if WIDE:
+                if part != "all" and WIDE_PART[i] != part:
+                    continue
+            elif not HALFSPLIT and ((part == "mid" and i % 2) or (part == "end" and i % 2 == 0)):
                 continue
             partial = WIDE and (i + 1) * WAVES * 1024 > B_BYTES       # only the first waves have rows left for this copy
             if partial:
                 _uid += 1
                 emit("s_cmp_eq_u32 s86, 0")
                 emit(f"s_cbranch_scc1 Lnobx{_uid}%=")
-            emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + i * WAVES * 1024}")
+            if WIDE and WIDE_GROUP[i] is None:
+                emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub)}")
+                emit("s_add_u32 m0, m0, s88")
+            elif WIDE:
+                emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + WIDE_GROUP[i] * 1024}")
+            else:
+                emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + i * WAVES * 1024}")
             emit("s_nop 0")
             if WIDE:
                 emit(f"global_load_lds_dwordx4 %[boff0], {WB_EXTRA[i]}")
@@ -166,6 +182,9 @@ def dma(stage, part="all"):
 def copies_per_part():
     """Requests of one wave in the mid-step part and in the end-of-step part of a stage (early hand-back)."""
     a, b = A_BYTES // 1024 // WAVES, B_BYTES // 1024 // WAVES
+    if WIDE:
+        # waves 0 .. 3 issue a third request in the end part; counting two makes their waits one request stricter
+        return a + 2, 2
     if HALFSPLIT:
         # a wave issues its weight copies in one of the two parts; either way the two parts together are a + b
         # requests, and counting none for the end part only makes the last trip's waits stricter
@@ -435,10 +454,17 @@ def generate():
         emit("s_mov_b64 s[72:73], %[bsptr2]")
         emit("s_mov_b32 s74, %[splitnb]")
         emit("s_mov_b32 s86, %[bextra]")
-        for i in range(1, len(WB_EXTRA)):                 # weight base of copy i: 64 rows further on
-            lo, prev = int(WB_EXTRA[i][2:4]), int(WB_EXTRA[i - 1][2:4])
-            emit(f"s_add_u32 s{lo}, s{prev}, %[bstride]")
-            emit(f"s_addc_u32 s{lo + 1}, s{prev + 1}, 0")
+        # weight base of copy i: WIDE_GROUP[i] groups of 8 rows further on (%[bstride] = bytes per group); the fifth
+        # copy's group comes from the set-up code (%[g4])
+        for i in range(1, len(WB_EXTRA)):
+            lo = int(WB_EXTRA[i][2:4])
+            if WIDE_GROUP[i] is None:
+                emit("s_mul_i32 s87, %[bstride], %[g4]")
+                emit("s_lshl_b32 s88, %[g4], 10")
+            else:
+                emit(f"s_mul_i32 s87, %[bstride], {WIDE_GROUP[i]}")
+            emit(f"s_add_u32 s{lo}, s42, s87")
+            emit(f"s_addc_u32 s{lo + 1}, s43, 0")
     if HALFSPLIT:
         emit("s_mov_b32 s87, %[lohalf]")
     emit("s_mov_b32 s48, %[m0base]")
@@ -526,8 +552,8 @@ def main():
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
                       ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True)),
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
-                      ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, False, True)),
-                      ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, False, True)),
+                      ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True)),
+                      ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True)),
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 2, False, True)),
                       ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 2, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
