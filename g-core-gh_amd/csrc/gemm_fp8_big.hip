@@ -207,7 +207,8 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106",   \
         "v107", "v108", "v109", "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120",   \
         "v121", "v122", "v123", "v124", "v125", "v126", "v127", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47",   \
-        "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63"
+        "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63",   \
+        "s98", "s99"
 #define LP_ASM_CLOBBERS_WIDE                                                                                              \
     "memory", "scc", "m0", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32",  \
         "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49",   \
@@ -217,18 +218,19 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "s40", "s41", "s42", "s43",     \
         "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60",   \
         "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77",   \
-        "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88"
+        "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s98", "s99"
 #define LP_ASM_INPUTS_WIDE                                                                                                \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
         [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
-        [g4] "s"(g4)
+        [g4] "s"(g4), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
-        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies)
+        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies),            \
+        [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 
 // Index arithmetic of the staged bf16 epilogue for a wave tile of 64 rows x COLS columns (COLS = 128, 96 or 64).
 // A row of the staging region holds COLS bf16 plus 16 bytes of padding (rows then start 4 banks apart: the 8-byte
@@ -268,7 +270,8 @@ struct AsmTile {
 // itself is unchanged: both groups run the same trips and meet at the same barriers), and the second group's
 // accumulators are added through LDS at the end.  For problems with about one tile per CU, where a workgroup's
 // time is its chain of K steps rather than its arithmetic: the chain halves.
-// NST: LDS stages (2, or 4 for the 128 x 128 tile with one K block per stage: three K steps in flight).
+// NST: LDS stages (2; 3 for the flat 128 x 256 tile, whose stage in use rotates through registers; 4 for the 128 x 128
+// tile with one K block per stage: three K steps in flight).
 // BROW: the weights carry an e8m0 scale per row and K block ([N, K/128] bytes) instead of per 128 rows; the matrix
 // instruction takes a scale per operand row anyway, so the loop only fetches them differently (hardware-scaled
 // 128 x 128 loop: waves 2 and 3 copy the weight-scale dwords of a group while waves 0 and 1 copy the activations').
@@ -292,9 +295,9 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 {
     using T = AsmTile<TM, TN, KSUB, NST, WN>;
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
-    static_assert(WN == 2 || (WN == 4 && TM == 128 && TN == 256 && KSUB == 1 && !DUAL && NST == 2 && !BROW), "four waves along N: the 128 x 256 tile");
+    static_assert(WN == 2 || (WN == 4 && TM == 128 && TN == 256 && KSUB == 1 && !DUAL && NST == 3 && !BROW), "four waves along N: the 128 x 256 tile, three stages");
     static_assert(!DUAL || (TM == 128 && TN == 128), "the K split inside a workgroup is built for the 128 x 128 tile");
-    static_assert(NST == 2 || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "four stages: 128 x 128 tile only");
+    static_assert(NST == 2 || (NST == 3 && WN == 4) || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "three stages: flat tile, four: 128 x 128 tile");
     static_assert(!BROW || (HWS && TM == 128 && TN == 128 && KSUB == 1 && !DUAL && NST == 2), "row-scaled weights: hardware-scaled 128 x 128 loop");
     static_assert((TM / 8 / WAVES == 4 || (WN == 4 && TM / 8 / WAVES == 2)) && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3),
                   "copies per operand and wave");
@@ -325,10 +328,15 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     // DMA source offsets (bytes from the matrix base; the host guarantees they fit 32 bits)
     const int ld_row = lane >> 3, ld_slot = lane & 7;
     uint32_t aoff[4], boff[4];
+    uint64_t amask[4];                                  // lanes of activation copy i whose row exists
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = 8 * (wave + WAVES * i) + ld_row;
-        const int64_t m = m0 + row < M ? m0 + row : M - 1;
+        amask[i] = __ballot(m0 + row < M);
+        // Rows past the end of the activations wrap around inside the tile's valid rows instead of all landing on the
+        // last one: with a few valid rows (an expert's short tile) every copy of every tile of that expert would
+        // otherwise ask one L2 channel for the same 128 bytes at the same time.
+        const int64_t m = m0 + row < M ? m0 + row : m0 + row % (int)(M - m0);
         const int64_t n = n0 + row < N ? n0 + row : N - 1;          // i = 3 is unused when there are three copies
         aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
         boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
@@ -414,13 +422,13 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
 #include "gemm_flat_hw_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
                 : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
-                : LP_ASM_CLOBBERS, "s87");
+                : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         } else {
             asm volatile(
 #include "gemm_flat_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
                 : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
-                : LP_ASM_CLOBBERS, "s87");
+                : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     } else if constexpr (HWS && NBW == 8) {
@@ -740,12 +748,12 @@ template <bool HWS>
 __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                               const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
                                                               const int32_t *__restrict__ m_offsets, int E, int64_t M_total,
-                                                              int64_t N, int64_t K, void *__restrict__ C, int out_dtype)
+                                                              int64_t N, int64_t K, void *__restrict__ C, int out_dtype, int small_first)
 {
-    constexpr int LDS_BIG = AsmTile<256, 256, 1>::LDS_BYTES, LDS_FLAT = AsmTile<128, 256, 1, 2, 4>::LDS_BYTES;
+    constexpr int LDS_BIG = AsmTile<256, 256, 1>::LDS_BYTES, LDS_FLAT = AsmTile<128, 256, 1, 3, 4>::LDS_BYTES;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BIG > LDS_FLAT ? LDS_BIG : LDS_FLAT];
     __shared__ int wave_big[8], wave_small[8];
-    __shared__ int found_e, found_first, found_begin, found_rows;
+    __shared__ int found_e, found_first, found_begin, found_rows, found_cnt;
     const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
     // ---- this thread's expert: rows, tiles of both classes, running counts over the experts before it
     int64_t begin = 0;
@@ -780,7 +788,13 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
     const int64_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
     bool big;
     int64_t idx;
-    if (sidx < rounds * period) {
+    if (small_first > 0) {
+        // XCDs below small_first work through their small tiles first and then their big ones, the others the other way
+        // round: every XCD has the same share of both classes, and at any time some XCDs stream weights while the
+        // others compute, each class with an L2 to itself
+        if (xcd < small_first) { big = sidx >= slots_small; idx = big ? sidx - slots_small : sidx; }
+        else { big = sidx < slots_big; idx = big ? sidx : sidx - slots_big; }
+    } else if (sidx < rounds * period) {
         const int64_t r = sidx % period, q = sidx / period;
         big = r == 0;
         idx = big ? q : q * ps + (r - 1);
@@ -789,12 +803,15 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
         big = w < left_big;
         idx = big ? rounds + w : rounds * ps + (w - left_big);
     }
-    int64_t gmt, tn;
-    if (!gemm::tile_coords(idx * 8 + xcd, big ? tot_big : tot_small, tiles_n, gmt, tn)) return;
-    // ---- the expert that owns m-tile gmt of the class tells the others
+    // Tiles of a class are numbered expert by expert (expert e owns tiles_n numbers per row tile) and an XCD takes 32
+    // consecutive numbers at a time, so the tiles it runs together belong to one expert, or to neighbours.
+    const int64_t lin = ((idx / gemm::CHUNK) * 8 + xcd) * gemm::CHUNK + idx % gemm::CHUNK;
+    if (lin >= (int64_t)(big ? tot_big : tot_small) * tiles_n) return;
+    const int64_t gmt = lin / tiles_n;
+    // ---- the expert that owns row tile gmt of the class tells the others
     {
         const int cnt = big ? nb : ns, incl = big ? ib : is;
-        if (gmt >= incl - cnt && gmt < incl) { found_e = t; found_first = incl - cnt; found_begin = (int)begin; found_rows = rows; }
+        if (gmt >= incl - cnt && gmt < incl) { found_e = t; found_first = incl - cnt; found_begin = (int)begin; found_rows = rows; found_cnt = cnt; }
     }
     __syncthreads();
     if (found_e < 0) return;
@@ -802,12 +819,26 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
     const int64_t row_begin = found_begin, row_end = row_begin + found_rows, kblocks = K / KB;
     const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
     const uint8_t *bq_e = Bq + (int64_t)e * N * K;
-    const int64_t local = gmt - found_first;
+    // Inside the expert: groups of 8 row tiles (the last may be short), in a group blocks of gn column tiles with the
+    // row tile running fastest, gn such that a block is about 32 tiles: the 32 tiles an XCD runs together share
+    // gm activation panels and gn weight panels of one expert (one row tile: its activations and the whole weight matrix once).
+    int64_t local, tn;
+    {
+        const int64_t in_e = lin - (int64_t)found_first * tiles_n, per_group = gemm::GROUP_M * tiles_n;
+        const int64_t grp = in_e / per_group, in_grp = in_e - grp * per_group;
+        const int64_t left = found_cnt - grp * gemm::GROUP_M;
+        const int64_t gm = left < gemm::GROUP_M ? left : gemm::GROUP_M;
+        const int64_t gn = gemm::CHUNK / gm;
+        const int64_t per_nblock = gm * gn;
+        const int64_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
+        local = grp * gemm::GROUP_M + in_blk % gm;
+        tn = nblk * gn + in_blk / gm;
+    }
     if (big)
         tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, bq_e, bs_e, row_begin + local * 256, row_end, tn * 256, N, K, C, N,
                                                           out_dtype);
     else
-        tile_asm<128, 256, 1, HWS, false, 2, false, true, 4>(smem, Aq, As, bq_e, bs_e, row_begin + (found_rows >> 8) * 256, row_end, tn * 256,
+        tile_asm<128, 256, 1, HWS, false, 3, false, true, 4>(smem, Aq, As, bq_e, bs_e, row_begin + (found_rows >> 8) * 256, row_end, tn * 256,
                                                              N, K, C, N, out_dtype);
 }
 
@@ -1048,12 +1079,14 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
         const int64_t grid = padded_grid((M_total + 128 * (int64_t)E) / 256 + 1, N / 256) + padded_grid(E, N / 256);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         if (E <= kMixedMaxExperts) {
+            static const char *order_env = getenv("LP_GEMM_GROUPED_ORDER");     // tuning aid: XCDs that take their small tiles first (0: classes dealt alternately)
+            const int small_first = order_env ? atoi(order_env) : 4;
             if (scale_dtype == LP_E8M0)
                 hipLaunchKernelGGL((gemm_asm_grouped_mixed<true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
-                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype);
+                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype, small_first);
             else
                 hipLaunchKernelGGL((gemm_asm_grouped_mixed<false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
-                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype);
+                                   (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype, small_first);
             return check_launch("lp_gemm_fp8_grouped(asm mixed heights)");
         }
     }

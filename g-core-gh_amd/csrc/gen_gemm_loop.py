@@ -40,7 +40,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT
     HW = hw
     # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
@@ -71,11 +71,18 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # next; the other weight rows follow at the end of the step as before.  Every request then has about one and a
     # half steps to land instead of one (the loop spends its waiting time at the end-of-step wait for the copies).
     EARLY = early
-    assert not early or (nstage == 2 and ksub == 1 and not brow)
+    assert not early or (nstage in (2, 3) and ksub == 1 and not brow)
+    # Three stages (with the early hand-back): the stage a step uses no longer follows from its place in the trip of four,
+    # so the stage offsets live in registers.  s89 / s90 = LDS offset of the stage in use (activations / weights), s91 / s92
+    # = of the stage just finished (what the end-of-step copies overwrite); the fragment read addresses v30 .. v33 are the
+    # lane's stage-0 addresses (asm operands) plus the offsets in use.  Requests then have two to two and a half steps to
+    # land: for tiles whose time is the latency of their weight stream (few activation rows per expert).
+    ROT = early and nstage == 3
+    assert not ROT or not wide
     NSTAGE = nstage
     BROW = brow                 # weight scales per row and K step (e8m0, hardware-scaled loop only) instead of per 128 rows
     assert not brow or (hw and tm == 128 and tn == 128)
-    assert nstage == 2 or (nstage == 4 and ksub == 1)
+    assert nstage == 2 or (nstage in (3, 4) and ksub == 1)
     assert tm == 64 * waves_m
     WAVES = waves_m * waves_n
     KSUB = ksub
@@ -133,9 +140,14 @@ def dma(stage, part="all"):
     for sub in range(KSUB):
         if part in ("all", "mid"):
             for i in range(A_BYTES // 1024 // WAVES):
-                emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
-                emit("s_nop 0")
+                if ROT:
+                    emit(f"s_add_u32 m0, s48, {i * WAVES * 1024}")
+                    emit("s_add_u32 m0, m0, s89")
+                else:
+                    emit(f"s_add_u32 m0, s48, {a_lds(stage, sub) + i * WAVES * 1024}")
+                emit(f"s_mov_b64 exec, %[amask{i}]")          # lanes whose activation row exists (see the prologue)
                 emit(f"global_load_lds_dwordx4 %[aoff{i}], s[40:41]")
+                emit("s_mov_b64 exec, s[98:99]")
         ncopies = -(-B_BYTES // 1024 // WAVES)
         if HALFSPLIT and part != "all":
             global _uid
@@ -158,6 +170,9 @@ def dma(stage, part="all"):
                 emit("s_add_u32 m0, m0, s88")
             elif WIDE:
                 emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + WIDE_GROUP[i] * 1024}")
+            elif ROT:
+                emit(f"s_add_u32 m0, s48, {bbase + i * WAVES * 1024}")
+                emit(f"s_add_u32 m0, m0, {'s90' if part == 'mid' else 's92'}")
             else:
                 emit(f"s_add_u32 m0, s48, {bbase + b_lds(stage, sub) + i * WAVES * 1024}")
             emit("s_nop 0")
@@ -192,17 +207,30 @@ def copies_per_part():
     return a + (b + 1) // 2, b // 2
 
 
+def younger_requests(c, at_end, last_trip):
+    """Requests of one wave that are younger than the ones a wait in step c depends on.  The mid-step wait needs the
+    end-of-step part issued NSTAGE steps earlier (the second weight half of this step), the end-of-step wait the
+    mid-step part issued NSTAGE - 1 steps earlier (activations and first weight half of the next step).  Parts are
+    issued in the order mid(j), end(j), mid(j + 1) ...; on the last trip a part of step j exists only if the step it
+    fills, j + NSTAGE, is still inside the trip (steps of earlier trips, j < 0, always do)."""
+    mid, end = copies_per_part()
+    need = ("mid", c - NSTAGE + 1) if at_end else ("end", c - NSTAGE)
+    upto = ("mid", c) if at_end else ("end", c - 1)
+    parts = []
+    for j in range(need[1], c + 1):
+        parts += [("mid", j), ("end", j)]
+    n = 0
+    for kind, j in parts[parts.index(need) + 1:parts.index(upto) + 1]:
+        if not last_trip or j < 0 or j + NSTAGE <= 3:
+            n += mid if kind == "mid" else end
+    return n
+
+
 def wait_copies(c, at_end, extra=""):
     """Early hand-back: wait until the requests this point depends on have landed.  Requests return in order, so it
-    is enough to bound how many younger ones may still be out: in the steady state the two parts issued since
-    (one mid-step part and one end-of-step part).  On the last trip nothing is requested for steps past the end,
-    so fewer, or none, are younger (c = step within the trip, s50 = 1 on the last trip)."""
-    mid, end = copies_per_part()
-    steady = mid + end
-    if at_end:
-        last = {0: steady, 1: steady, 2: end, 3: 0}[c]
-    else:
-        last = {0: steady, 1: steady, 2: steady, 3: 0}[c]
+    is enough to bound how many younger ones may still be out (c = step within the trip, s50 = 1 on the last trip,
+    on which nothing is requested for steps past the end)."""
+    steady, last = younger_requests(c, at_end, False), younger_requests(c, at_end, True)
     tag = f"{'e' if at_end else 'm'}{c}"
     if last != steady:
         emit("s_cmp_eq_u32 s50, 1")
@@ -314,6 +342,8 @@ def step(c):
     nstage, nsub = ((stage + 1) % NSTAGE, 0) if flip else (stage, sub + 1)
     aoff, boff = a_lds(stage, sub), b_lds(stage, sub)
     naoff, nboff = a_lds(nstage, nsub), b_lds(nstage, nsub)
+    if ROT:
+        aoff = boff = naoff = nboff = 0                  # the read addresses carry the stage
     if HW:
         pass
     elif SPLIT:
@@ -401,6 +431,20 @@ def step(c):
                         emit(f"s_waitcnt vmcnt({last}) lgkmcnt(0)")
                         emit(f"Lwj{c}%=:")
                 emit("s_barrier")
+                if ROT:
+                    # the next stage becomes the one in use
+                    emit("s_mov_b32 s91, s89")
+                    emit("s_mov_b32 s92, s90")
+                    emit(f"s_add_u32 s89, s89, {A_BYTES}")
+                    emit(f"s_cmp_eq_u32 s89, {NSTAGE * A_BYTES}")
+                    emit("s_cselect_b32 s89, 0, s89")
+                    emit(f"s_add_u32 s90, s90, {B_BYTES}")
+                    emit(f"s_cmp_eq_u32 s90, {NSTAGE * B_BYTES}")
+                    emit("s_cselect_b32 s90, 0, s90")
+                    emit(f"v_add_u32 {RA0}, s89, %[ard0]")
+                    emit(f"v_add_u32 {RA1}, s89, %[ard1]")
+                    emit(f"v_add_u32 {RB0}, s90, %[brd0]")
+                    emit(f"v_add_u32 {RB1}, s90, %[brd1]")
             else:
                 emit("s_waitcnt lgkmcnt(0)")
             read_frag(WFB[par(c + 1, 0)], RB0, RB1, nboff)
@@ -409,7 +453,7 @@ def step(c):
             fold(nb - 1, mb, c)
             if handback and mb == 0:
                 # the activation rows and the first weight half of the step after the next, into the rows just freed
-                cond = c + 1 + KSUB >= 4
+                cond = c + NSTAGE >= 4 if ROT else c + 1 + KSUB >= 4
                 if cond:
                     emit("s_cmp_eq_u32 s50, 1")
                     emit(f"s_cbranch_scc1 Lnodmam{c}%=")
@@ -420,7 +464,7 @@ def step(c):
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
                 if mb == 0 and flip:
                     # copies for the K blocks after the next stage overwrite the stage just finished
-                    cond = NSTAGE == 4 or c + 1 + KSUB >= 4
+                    cond = NSTAGE == 4 or (c + NSTAGE >= 4 if ROT else c + 1 + KSUB >= 4)
                     if cond:
                         emit("s_cmp_eq_u32 s50, 1")
                         emit(f"s_cbranch_scc1 Lnodma{c}%=")
@@ -442,6 +486,12 @@ def step(c):
 
 def generate():
     # ---- prologue
+    # Activation rows past the end of the matrix (or of an expert's rows) are not copied: their lanes are switched off
+    # for the copy instruction (%[amaskI] = lanes of copy I whose row exists).  Pointing them at a valid row instead
+    # makes a workgroup ask for cache lines it is already waiting for, and the in-order L1 then holds back the
+    # weight requests queued behind them: a tile with 64 of 128 rows valid ran a third slower than a full one.
+    # What the LDS rows of missing activation rows hold only reaches accumulator rows that are never stored.
+    emit("s_mov_b64 s[98:99], exec")
     emit("s_mov_b64 s[40:41], %[abase]")
     emit("s_mov_b64 s[42:43], %[bbase]")
     emit("s_mov_b64 s[44:45], %[sbase]")
@@ -486,10 +536,17 @@ def generate():
     if EARLY:
         # both stages are requested in the order of the steady state (mid part, end part), then stage 0 and the
         # scale group (older) are waited for: what may stay out is exactly what the first waits of the loop allow
-        for st in range(2):
+        for st in range(NSTAGE):
+            if ROT:
+                emit(f"s_mov_b32 s89, {st * A_BYTES}")
+                emit(f"s_mov_b32 s90, {st * B_BYTES}")
+                emit(f"s_mov_b32 s92, {st * B_BYTES}")
             dma(st, "mid")
             dma(st, "end")
-        emit(f"s_waitcnt vmcnt({sum(copies_per_part())}) lgkmcnt(0)")
+        if ROT:
+            emit("s_mov_b32 s89, 0")
+            emit("s_mov_b32 s90, 0")
+        emit(f"s_waitcnt vmcnt({(NSTAGE - 1) * sum(copies_per_part())}) lgkmcnt(0)")
         emit("s_barrier")
     else:
         dma(0)
@@ -554,8 +611,8 @@ def main():
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
                       ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True)),
                       ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True)),
-                      ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 2, False, True)),
-                      ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 2, False, True)),
+                      ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True)),
+                      ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)
