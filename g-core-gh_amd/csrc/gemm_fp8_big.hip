@@ -1071,11 +1071,11 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
     const int mode = force ? atoi(force) : -1;
     // One launch with both tile heights when the experts are not all tiny (with fewer than 128 rows per expert on
     // average hardly any 256-row tile exists and the 128 x 128 kernel, two workgroups per CU, streams weights as well)
-    // and K is long: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden
-    // behind a second workgroup, and at K = 2048 (16 steps) that costs what the larger tiles gain (config 4, down
-    // projection: 1.64 ms against 1.59 with fp32 scales, 1.49 against 1.51 with e8m0).
+    // and K is not short: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden
+    // behind a second workgroup (config 4, down projection, K = 2048: 1.76 ms against 1.87 for the 128 x 128 kernel
+    // with fp32 scales in the same process, 1.46 against 1.57 with e8m0).
     // An expert has at most one small tile, and M_e / 256 big ones plus one when more than 128 rows are left over.
-    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 4096)) {
+    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 2048)) {
         const int64_t grid = padded_grid((M_total + 128 * (int64_t)E) / 256 + 1, N / 256) + padded_grid(E, N / 256);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         if (E <= kMixedMaxExperts) {
