@@ -1076,7 +1076,9 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
     // with fp32 scales in the same process, 1.46 against 1.57 with e8m0).
     // An expert has at most one small tile, and M_e / 256 big ones plus one when more than 128 rows are left over.
     if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 2048)) {
-        const int64_t grid = padded_grid((M_total + 128 * (int64_t)E) / 256 + 1, N / 256) + padded_grid(E, N / 256);
+        // an expert with r rows has r / 256 tiles plus one when rows are left over, big or small: M_total / 256 + E row
+        // tiles at most over both classes, each class rounded up to whole groups of 8 x 32 workgroups
+        const int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         if (E <= kMixedMaxExperts) {
             static const char *order_env = getenv("LP_GEMM_GROUPED_ORDER");     // tuning aid: XCDs that take their small tiles first (0: classes dealt alternately)

@@ -179,7 +179,7 @@ def dma(stage, part="all"):
             if WIDE:
                 emit(f"global_load_lds_dwordx4 %[boff0], {WB_EXTRA[i]}")
             else:
-                emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]")
+                emit(f"global_load_lds_dwordx4 %[boff{i}], s[42:43]" + (" nt" if ROT else ""))     # the flat tile's weights are read once: streamed past the L2's resident lines
             if partial:
                 emit(f"Lnobx{_uid}%=:")
         if HALFSPLIT and part != "all":
