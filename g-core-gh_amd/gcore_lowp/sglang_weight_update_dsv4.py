@@ -10,9 +10,11 @@ trainer's 128 x 128 FP8 grid.  All arithmetic runs in the HIP kernels of this pa
 The dense quantiser of the reference is SGLang's `per_block_cast_to_fp8`, imported at run time
 (sglang_weight_update_dsv4.py:205-223).  SGLang is not part of the reference tree, so what is built in here is
 that function as published (amax clamped at 1e-4, x * (448 / amax) -> e4m3fn, scale amax / 448, fp32): scale mode
-LP_SCALE_MUL_FLOOR of lp_quant_fp8_block.  The DeepGEMM ue8m0 scale layout (`quant_weight_ue8m0` /
-`transform_scale_ue8m0`, an NVIDIA TMA layout) has no counterpart on this hardware: the hooks stay None, as in
-the reference when SGLang does not offer them, and every scale is float32.
+LP_SCALE_MUL_FLOOR of lp_quant_fp8_block.  The DeepGEMM pair `quant_weight_ue8m0` / `transform_scale_ue8m0` is
+restated the same way (power-of-two scales from LP_SCALE_POW2 with the 1e-4 amax floor; scale bytes expanded per weight
+row, packed four K blocks to an int32 and laid out MN-major with the row count aligned to 4, as the published
+DeepGEMM helper does) and installed as the default hooks.  Whether they are used is SGLang's decision
+(`_should_ue8m0_fn`, None here as on any sampler that does not run DeepGEMM): by default every scale is float32.
 """
 from __future__ import annotations
 
@@ -126,8 +128,49 @@ def per_block_cast_to_fp8(x: torch.Tensor):
     return q[:m, :n].contiguous().to(home), s.to(home)
 
 
+def quant_weight_ue8m0(weight_dequant: torch.Tensor, weight_block_size=None):
+    """SGLang's `quant_weight_ue8m0` as published: [..., n, k] -> e4m3fn codes of the same shape and fp32 scales
+    [..., ceil(n / 128), ceil(k / 128)] that are powers of two, 2^ceil(log2(max(amax, 1e-4) / 448)), codes
+    x * (1 / scale).  One launch of lp_quant_fp8_block (LP_SCALE_POW2) over the tensor viewed as (-1, k)."""
+    assert weight_block_size is None or list(weight_block_size) == [128, 128], weight_block_size
+    *lead, n, k = weight_dequant.shape
+    assert not lead or n % 128 == 0, "stacked matrices must hold whole 128-row blocks each"
+    flat = weight_dequant.reshape(-1, k)
+    m = flat.shape[0]
+    mp, kp = -(-m // 128) * 128, -(-k // 128) * 128
+    xg, home = A.to_device(flat.contiguous())
+    if (mp, kp) != (m, k):
+        pad = torch.zeros(mp, kp, dtype=xg.dtype, device=xg.device)
+        pad[:m, :k] = xg
+        xg = pad
+    q, s, _ = ops.quant_fp8_block(xg, (128, 128), scale_mode=A.SCALE_POW2, scale_dtype=torch.float32, amax_floor=1e-4)
+    q = q[:m, :k].contiguous().to(home).view(weight_dequant.shape)
+    return q, s.to(home).view(*lead, -(-n // 128), kp // 128)
+
+
+def transform_scale_ue8m0(sf: torch.Tensor, mn: int, use_torch_impl: bool = False) -> torch.Tensor:
+    """SGLang's `transform_scale_ue8m0` as published: power-of-two fp32 scales [..., ceil(mn / 128), kb] -> one scale row
+    per weight row, the exponent bytes of four consecutive K blocks packed into an int32 (block 4 j in the low byte,
+    kb padded with zero bytes), returned as [..., mn, ceil(kb / 4)] int32 whose mn index is the fastest in memory with
+    the column pitch rounded up to 4 rows (DeepGEMM's `get_mn_major_tma_aligned_packed_ue8m0_tensor`).  Pure index
+    arithmetic on a small tensor: torch ops on whatever device holds `sf`."""
+    assert sf.dtype == torch.float32 and sf.dim() >= 2, (sf.dtype, sf.shape)
+    rows = torch.arange(mn, device=sf.device) // 128
+    exp = (sf.index_select(-2, rows).contiguous().view(torch.int32) >> 23) & 0xFF          # [..., mn, kb]
+    kb = exp.shape[-1]
+    kq = -(-kb // 4)
+    if kq * 4 != kb:
+        exp = torch.nn.functional.pad(exp, (0, kq * 4 - kb))
+    e4 = exp.view(*exp.shape[:-1], kq, 4)
+    packed = e4[..., 0] | (e4[..., 1] << 8) | (e4[..., 2] << 16) | (e4[..., 3] << 24)      # [..., mn, kq]
+    pitch = -(-mn // 4) * 4
+    store = torch.zeros(*packed.shape[:-2], kq, pitch, dtype=torch.int32, device=sf.device)
+    store[..., :mn] = packed.transpose(-1, -2)
+    return store.transpose(-1, -2)[..., :mn, :]
+
+
 # Hooks with the reference's names (:193-197): the tests of the reference patch them, and a deployment that has
-# SGLang's own functions can install them here.  The ue8m0 pair stays None on this hardware.
+# SGLang's own functions can install them here.  `_should_ue8m0_fn` stays None unless the deployment sets it.
 _per_block_cast_fn = None
 _quant_weight_ue8m0_fn = None
 _transform_scale_ue8m0_fn = None
@@ -141,8 +184,13 @@ def _init_fp8_quantizers():
     if _fp8_ready:
         return
     A.lib()                                               # fail loudly here if the HIP library is missing
+    global _quant_weight_ue8m0_fn, _transform_scale_ue8m0_fn
     if _per_block_cast_fn is None:
         _per_block_cast_fn = per_block_cast_to_fp8
+    if _quant_weight_ue8m0_fn is None:
+        _quant_weight_ue8m0_fn = quant_weight_ue8m0
+    if _transform_scale_ue8m0_fn is None:
+        _transform_scale_ue8m0_fn = transform_scale_ue8m0
     _fp8_ready = True
 
 

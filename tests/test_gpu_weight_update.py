@@ -163,3 +163,31 @@ def test_vllm_reload_bucket_quantisation(expert_dtype):
     dq, ds = T.quant_fp8_e4m3_scale_e8m0(dense.bfloat16().float(), (128, 128))
     assert torch.equal(u8(got["layers.0.attn.wq_b.weight"]), u8(dq)) and torch.equal(u8(got["layers.0.attn.wq_b.scale"]), u8(ds))
     assert got["layers.0.attn.wo_b.weight"].dtype == torch.float32 and torch.equal(got["layers.0.attn.wo_b.weight"].cpu(), kept)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(256, 384), (3, 128, 256), (200, 320)])
+def test_quant_weight_ue8m0_is_pow2_block_quant(shape):
+    """quant_weight_ue8m0 == the power-of-two block quantiser with the 1e-4 amax floor (oracle), bit for bit, on whole
+    and ragged shapes and with an all-zero block; scales are powers of two and survive the packed layout."""
+    from gcore_lowp import sglang_weight_update_dsv4 as update
+    g = torch.Generator().manual_seed(17)
+    w = (torch.randn(*shape, generator=g) * 0.02).to(torch.bfloat16).float()
+    w.view(-1, shape[-1])[:128, :128] = 0
+    q, s = update.quant_weight_ue8m0(w.cuda(), weight_block_size=[128, 128])
+    flat = w.view(-1, shape[-1])
+    m, k = flat.shape
+    mp, kp = -(-m // 128) * 128, -(-k // 128) * 128
+    pad = torch.zeros(mp, kp)
+    pad[:m, :k] = flat
+    rq, rs = T.quant_block_pow2_scale(pad, (128, 128), amax_floor=1e-4)
+    assert q.dtype == torch.float8_e4m3fn and tuple(q.shape) == tuple(shape)
+    assert torch.equal(q.cpu().view(torch.uint8).view(m, k), rq.view(torch.uint8)[:m, :k])
+    assert torch.equal(s.cpu().reshape(rs.shape), rs)
+    mant = s.cpu().view(torch.int32) & 0x7FFFFF
+    assert int(mant.abs().max()) == 0
+    n = shape[-2]
+    packed = update.transform_scale_ue8m0(s, mn=n)
+    first = (packed[..., 0].cpu() & 0xFF)
+    assert torch.equal(first, ((s.cpu().view(torch.int32) >> 23) & 0xFF)[..., 0].repeat_interleave(128, dim=-1)[..., :n])
+

@@ -186,4 +186,32 @@ def test_routing_of_keys_to_quantisers():
         list(update.iter_fp8_quantized_weights(iter([("layers.0.attn.wq_b.scale", dense)])))
     assert update.should_fp8_quantize("mtp.0.h_proj.weight") and update.should_fp8_quantize("layers.9.ffn.shared_experts.w2.weight")
     assert not update.should_fp8_quantize("layers.9.ffn.gate.weight") and not update.should_fp8_quantize(_WO_A_KEY)
-    assert not update._use_ue8m0_scale(_EXPERT_KEY, moe_deepgemm=True)       # no DeepGEMM layout on this hardware
+    assert not update._use_ue8m0_scale(_EXPERT_KEY, moe_deepgemm=True)       # SGLang has not asked for the DeepGEMM layout
+
+
+def test_transform_scale_ue8m0_layout():
+    """The DeepGEMM scale layout, restated element by element: row r of the result takes the scales of weight-row
+    block r // 128, int32 j holds the exponent bytes of K blocks 4 j .. 4 j + 3 (low byte first, zero beyond the end),
+    and rows are the fastest index in memory with a column pitch of mn rounded up to 4.  (Parity with the DeepGEMM
+    helper itself is unpinned: the library is not in the reference tree.)"""
+    g = torch.Generator().manual_seed(5)
+    for lead, mn, kb in (((), 384, 7), ((), 130, 4), ((3,), 256, 9)):
+        nblk = -(-mn // 128)
+        expo = torch.randint(90, 140, (*lead, nblk, kb), generator=g)
+        sf = torch.pow(2.0, (expo - 127).float())
+        out = update.transform_scale_ue8m0(sf, mn=mn)
+        kq = -(-kb // 4)
+        assert out.dtype == torch.int32 and tuple(out.shape) == (*lead, mn, kq)
+        assert out.stride(-2) == 1 and out.stride(-1) == -(-mn // 4) * 4
+        flat_e = expo.reshape(-1, nblk, kb)
+        flat_o = out.reshape(-1, mn, kq)
+        for b in range(flat_e.shape[0]):
+            for r in (0, 1, 127, 128, mn - 1):
+                for j in range(kq):
+                    want = 0
+                    for i in range(4):
+                        k = 4 * j + i
+                        if k < kb:
+                            want |= int(flat_e[b, r // 128, k]) << (8 * i)
+                    got = int(flat_o[b, r, j]) & 0xFFFFFFFF
+                    assert got == want, (lead, mn, kb, b, r, j, hex(got), hex(want))
