@@ -514,7 +514,36 @@ def main():
         fnw = lambda: chk(L.lp_gemm_fp8_rowscale(a_w.data_ptr(), sa_w.data_ptr(), b_w.data_ptr(), sb_w.data_ptr(), A.E8M0,  # noqa: E731
                                                  4096, 7168, Pw, dw.data_ptr(), A.BF16, stream()))
         msw, _ = time_launches([fnw], 10, 3)
+        # the whole layer's weight gradient in one (two) launches: 256 problems [4096, 7168] x P_e, config 4's rows per
+        # expert padded as the wrapper pads them; operands are random codes (the time does not depend on the values), 15 GB of bf16 out
+        from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad
+        padw = choose_colwise_pad(m_splits.tolist())                   # rows the wrapper pads every expert to (512 here)
+        nblkw = [(int(m) + padw - 1) // padw * (padw // 128) for m in m_splits.tolist()]
+        pbw = sum(nblkw)
+        pre, fast, rest = 0, [], []
+        for e, nb in enumerate(nblkw):
+            if nb:
+                (fast if nb % 4 == 0 else rest).append((e, nb, pre, 0))
+            pre += nb
+        aT = torch.randint(0, 120, (4096 * pbw * 128,), dtype=torch.uint8, device=dev)
+        bT = torch.randint(0, 120, (7168 * pbw * 128,), dtype=torch.uint8, device=dev)
+        saT = torch.full((4096 * pbw,), 120, dtype=torch.uint8, device=dev)
+        sbT = torch.full((7168 * pbw,), 121, dtype=torch.uint8, device=dev)
+        dW = torch.empty(E4, 4096, 7168, dtype=torch.bfloat16, device=dev)
+        tabs = [(torch.tensor(g, dtype=torch.int32, device=dev), len(g), max(x[1] for x in g), mult) for g, mult in ((fast, 4), (rest, 1)) if g]
+
+        def fng():
+            for tab, n, mx, mult in tabs:
+                chk(L.lp_gemm_fp8_rowscale_grouped(aT.data_ptr(), saT.data_ptr(), bT.data_ptr(), sbT.data_ptr(), A.E8M0, tab.data_ptr(), n, mx,
+                                                   mult, 4096, 7168, dW.data_ptr(), A.BF16, stream()))
+        msg, _ = time_launches([fng], 3, 1)
+        flg = 2.0 * 4096 * 7168 * pbw * 128
+        del aT, bT, saT, sbT, dW, tabs
         extras["grouped_linear_backward"] = {
+            "wgrad_grouped_256_experts_4096x7168": {"ms": msg, "rows_padded_to": padw, "tflops_on_padded_rows": flg / msg / 1e9,
+                                                    "mfma_frac": flg / msg / 1e9 / FP8_PEAK_TFLOPS,
+                                                    "output_GB": E4 * 4096 * 7168 * 2 / 1e9,
+                                                    "output_write_GB/s": E4 * 4096 * 7168 * 2 / msg / 1e6, "launches": len([g for g in (fast, rest) if g])},
             "quant_colwise_t_65536x4096": {"ms": msq, "GB/s": byq / msq / 1e6, "hbm_frac": byq / msq / 1e6 / HBM_PEAK_GBS, "bytes": byq},
             "wgrad_gemm_rowscale_4096x7168xP1024": {"ms": msw, "tflops": 2.0 * 4096 * 7168 * Pw / msw / 1e9,
                                                     "mfma_frac": 2.0 * 4096 * 7168 * Pw / msw / 1e9 / FP8_PEAK_TFLOPS}}

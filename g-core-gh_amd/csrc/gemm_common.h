@@ -84,6 +84,8 @@ int64_t skinny_workspace_bytes(int64_t N, int splits);
 int launch_skinny(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                   int64_t K, void *C, int out_dtype, float *ws, int splits, int per, hipStream_t st);
 
+int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int64_t M,
+                                int64_t N, void *C, int out_dtype, hipStream_t st);
 bool launch_wide(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                  void *C, int64_t ldc, int out_dtype, hipStream_t st, int *rc);
 bool launch_mixed(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,

@@ -217,6 +217,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     store_tile(acc, ta.m0, M, ta.n0, ldc, C, out_dtype);
 }
 
+// Row-scaled problems that share M and N and differ in K, one launch (see gemm_asm_rowscale_grouped for `groups`).
+template <int SDT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_rowscale_grouped(
+    const uint8_t *__restrict__ Aq, const void *__restrict__ As, const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+    int scale_dtype, const int32_t *__restrict__ groups, int64_t M, int64_t N, int64_t tiles_m, int64_t tiles_n, int64_t per_group,
+    void *__restrict__ C, int out_dtype)
+{
+    __shared__ Smem sm;
+    const int64_t g = blockIdx.x / per_group, local = blockIdx.x - g * per_group;
+    int64_t tm, tn;
+    if (!tile_coords(local, tiles_m, tiles_n, tm, tn)) return;
+    const int64_t slot = groups[4 * g], kb = groups[4 * g + 1], before = groups[4 * g + 2];
+    if (kb <= 0) return;
+    const int64_t ssz = SDT == LP_F32 ? 4 : 1;
+    TileArgs ta;
+    ta.Aq = Aq + M * 128 * before; ta.As = (const char *)As + M * before * ssz;
+    ta.Bq = Bq + N * 128 * before; ta.Bs = (const char *)Bs + N * before * ssz;
+    ta.scale_dtype = scale_dtype;
+    ta.K = kb * 128; ta.kblocks = kb; ta.m0 = tm * TM; ta.m_end = M; ta.n0 = tn * TN;
+    ta.kb_begin = 0; ta.kb_end = (int)kb;
+    Acc acc;
+    gemm_tile<SDT, true>(ta, sm, acc);
+    store_tile(acc, ta.m0, M, ta.n0, N, (char *)C + slot * M * N * (out_dtype == LP_BF16 ? 2 : 4), out_dtype);
+}
+
 // ------------------------------------------------------------------ split-K
 // Skinny problems (few output tiles) are weight-streaming bound: K is cut into
 // `splits` contiguous ranges so that every CU pulls HBM; each range writes an
@@ -432,6 +457,32 @@ extern "C" int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *
         hipLaunchKernelGGL((gemm_dense<LP_E8M0, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
                            (const uint8_t *)Bq, Bs, scale_dtype, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
     return check_launch("lp_gemm_fp8_rowscale");
+}
+
+extern "C" int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                                            const int32_t *groups, int G, int max_k_blocks, int k_blocks_multiple, int64_t M, int64_t N,
+                                            void *C, int out_dtype, lp_stream_t stream)
+{
+    LP_REQUIRE(G >= 0 && max_k_blocks >= 0 && k_blocks_multiple >= 1, "lp_gemm_fp8_rowscale_grouped: bad group description");
+    if (G == 0 || max_k_blocks == 0) return LP_OK;
+    int rc = check_gemm_args("lp_gemm_fp8_rowscale_grouped", Aq, As, Bq, Bs, scale_dtype, M, N, (int64_t)max_k_blocks * 128, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    LP_REQUIRE(groups, "lp_gemm_fp8_rowscale_grouped: null pointer");
+    LP_REQUIRE(M % 128 == 0, "lp_gemm_fp8_rowscale_grouped: M (%lld) must be a multiple of 128", (long long)M);
+    hipStream_t st = (hipStream_t)stream;
+    // every problem's K a multiple of 512 (promised by the caller: k_blocks_multiple), e8m0 scales: the hand-scheduled loop
+    if (k_blocks_multiple % 4 == 0 && gemm::rowscale_asm_ok(As, Bs, scale_dtype, M, N, (int64_t)max_k_blocks * 128))
+        return gemm::launch_rowscale_grouped_asm(Aq, As, Bq, Bs, groups, G, M, N, C, out_dtype, st);
+    const int64_t tiles_m = M / TM, tiles_n = N / TN;
+    const int64_t per_group = padded_grid(tiles_m, tiles_n), grid = per_group * G;
+    LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_rowscale_grouped: problem too large");
+    if (scale_dtype == LP_F32)
+        hipLaunchKernelGGL(gemm_rowscale_grouped<LP_F32>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+    else
+        hipLaunchKernelGGL(gemm_rowscale_grouped<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
+                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+    return check_launch("lp_gemm_fp8_rowscale_grouped");
 }
 
 extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,

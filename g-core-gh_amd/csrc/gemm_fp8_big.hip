@@ -660,6 +660,28 @@ __global__ __launch_bounds__(256) void gemm_asm_rowscale(const uint8_t *__restri
     tile_asm<128, 128, 1, true, false, 2, true, true>(smem, Aq, As, Bq, Bs, tm * 128, M, tn * 128, N, K, C, ldc, out_dtype);
 }
 
+// The same for a list of problems that share M and N and differ in K (the weight gradients of the experts of a grouped
+// linear): entry g of `groups` = {output slot, K blocks of 128, K blocks of all problems before it in the operand
+// buffers, unused}.  Problem g reads Aq + M * 128 * before (its [M, K_g] codes), As + M * before, the same for B with
+// N, and writes C + slot * M * N.  per_group workgroups (a multiple of 256) belong to each entry.
+__global__ __launch_bounds__(256) void gemm_asm_rowscale_grouped(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
+                                                                 const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
+                                                                 const int32_t *__restrict__ groups, int64_t M, int64_t N,
+                                                                 int64_t tiles_m, int64_t tiles_n, int64_t per_group,
+                                                                 void *__restrict__ C, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<128, 128, 1>::LDS_BYTES + 4096];
+    const int64_t g = blockIdx.x / per_group, local = blockIdx.x - g * per_group;
+    int64_t tm, tn;
+    if (!gemm::tile_coords(local, tiles_m, tiles_n, tm, tn)) return;
+    const int64_t slot = groups[4 * g], kb = groups[4 * g + 1], before = groups[4 * g + 2];
+    if (kb <= 0) return;
+    char *c = (char *)C + slot * M * N * (out_dtype == LP_BF16 ? 2 : 4);
+    tile_asm<128, 128, 1, true, false, 2, true, true>(smem, Aq + M * 128 * before, (const float *)((const char *)As + M * before),
+                                                      Bq + N * 128 * before, (const float *)((const char *)Bs + N * before), tm * 128, M,
+                                                      tn * 128, N, kb * 128, c, N, out_dtype);
+}
+
 // Grouped variant: expert e owns rows m_offsets[e] .. m_offsets[e+1]-1 and the weight matrix e of Bq / Bs.
 // The grid is sized from an upper bound on the number of row tiles; each workgroup finds its expert with a
 // block-wide scan over the per-expert tile counts.  PART selects which rows of every expert a launch covers:
@@ -1053,6 +1075,17 @@ int launch_rowscale_asm(const void *Aq, const void *As, const void *Bq, const vo
     hipLaunchKernelGGL(gemm_asm_rowscale, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, (const float *)As,
                        (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
     return check_launch("lp_gemm_fp8_rowscale(asm)");
+}
+
+int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int64_t M,
+                                int64_t N, void *C, int out_dtype, hipStream_t st)
+{
+    const int64_t tiles_m = (M + 127) / 128, tiles_n = N / 128;
+    const int64_t per_group = gemm::padded_grid(tiles_m, tiles_n), grid = per_group * G;
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_rowscale_grouped: problem too large");
+    hipLaunchKernelGGL(gemm_asm_rowscale_grouped, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, (const float *)As,
+                       (const uint8_t *)Bq, (const float *)Bs, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+    return check_launch("lp_gemm_fp8_rowscale_grouped(asm)");
 }
 
 // Grouped problems on the hand-scheduled kernel: fp32 scales, N a multiple of 256, offsets that fit 32 bits.

@@ -277,6 +277,20 @@ int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const v
                          int64_t M, int64_t N, int64_t K, void *C, int out_dtype, lp_stream_t stream);
 
 /*
+ * The same for a list of problems that share M and N and differ in K, in one launch: the weight gradients of all
+ * experts of a grouped linear, which the reference issues as one grouped GEMM call
+ * (gpatch_v4/models/deepseek_v4/fp8.py:325-341).  `groups` is a device array of G entries of four int32:
+ * {output slot, K blocks of 128 of this problem, K blocks of all problems stored before it, unused}.  Problem g
+ * reads Aq + M * 128 * before (its [M, K_g] codes), As + M * before scales, Bq / Bs likewise with N, and writes
+ * C + slot * M * N elements.  max_k_blocks bounds every entry's K blocks (argument checks); k_blocks_multiple is
+ * the caller's promise that every entry's K block count is a multiple of it (4 selects the hand-scheduled loop
+ * with e8m0 scales).  M must be a multiple of 128.  Entries with 0 blocks write nothing.
+ */
+int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
+                                 const int32_t *groups, int G, int max_k_blocks, int k_blocks_multiple, int64_t M,
+                                 int64_t N, void *C, int out_dtype, lp_stream_t stream);
+
+/*
  * Column-wise quantiser with transposed output for expert-grouped rows.  x: device [rows, cols]
  * (LP_BF16 or LP_F32), rows of expert e = m_offsets[e] .. m_offsets[e+1]-1 (device int32 [E+1]),
  * cols % 128 == 0.  Per expert, P_e = ceil(M_e / pad_rows) * pad_rows (pad_rows 128, 256 or 512; with 512

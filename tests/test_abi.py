@@ -80,6 +80,9 @@ def test_host_side_validation(lib):
     assert L.lp_act_qdq_group(None, 0, 128, 1, 0, None, None, None) == 0
     assert L.lp_quant_fp8_colwise_t(None, lib.BF16, 0, 128, None, 0, 0, 128, None, None, lib.E8M0, None) == 0
     assert L.lp_gemm_fp8_rowscale(None, None, None, None, lib.E8M0, 0, 128, 128, None, lib.BF16, None) == 0
+    assert L.lp_gemm_fp8_rowscale_grouped(None, None, None, None, lib.E8M0, None, 0, 0, 1, 128, 128, None, lib.BF16, None) == 0
+    rc = L.lp_gemm_fp8_rowscale_grouped(one, one, one, one, lib.E8M0, one, 2, 4, 4, 100, 128, one, lib.BF16, None)
+    assert rc == -1 and "multiple of 128" in lib.last_error()
     assert L.lp_quant_fp8_block(None, lib.BF16, 0, 128, 128, 128, lib.SCALE_DIV, 0.0, 0, None, None, lib.F32, None, None) == 0
     assert L.lp_gemm_fp8_block(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None, 0, None) == 0
     assert L.lp_gemm_fp8_block_static(None, None, None, None, lib.F32, 0, 128, 128, None, lib.BF16, None) == 0

@@ -351,6 +351,40 @@ def test_gemm_rowscale(G, shape):
     assert torch.equal(outs[torch.bfloat16], outs[torch.float32].to(torch.bfloat16)), "bf16 output is the rounded fp32 output"
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_gemm_rowscale_grouped_equals_per_problem_launches(G, out_dtype):
+    """One grouped launch (two when some K are not multiples of 512) writes what one lp_gemm_fp8_rowscale launch per
+    problem writes, bit for bit: same kernels, same order of summation.  K blocks per problem cover multiples of 4,
+    other counts and an empty problem, which is zero-filled."""
+    M, N = 256, 384
+    k_blocks = [4, 1, 0, 8, 3, 12, 0, 5]
+    say("gemm rowscale grouped", (M, N), k_blocks, out_dtype)
+    total = sum(k_blocks)
+    a = I.act_like(M, total * 128, 21)
+    b = I.act_like(N, total * 128, 22) * 0.05
+    aq, a_s = T.quant_fp8_e4m3_scale_e8m0(a, (1, 128))
+    bq, b_s = T.quant_fp8_e4m3_scale_e8m0(b, (1, 128))
+    # problem e's operands stored as [M, K_e] / [N, K_e] one after the other
+    cut = lambda t, w: torch.cat([t[:, w * sum(k_blocks[:e]):w * sum(k_blocks[:e + 1])].contiguous().view(torch.uint8).flatten()
+                                  for e in range(len(k_blocks))]).cuda()
+    aqf, asf, bqf, bsf = cut(aq, 128), cut(a_s, 1), cut(bq, 128), cut(b_s, 1)
+    out = torch.full((len(k_blocks), M, N), float("nan"), dtype=out_dtype, device="cuda")
+    G.gemm_fp8_rowscale_grouped(aqf, asf, bqf, bsf, k_blocks, M, N, out)
+    before = 0
+    for e, kb in enumerate(k_blocks):
+        if kb == 0:
+            assert not out[e].any()
+            continue
+        one = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+        G.gemm_fp8_rowscale(aqf[M * 128 * before:], asf[M * before:], bqf[N * 128 * before:], bsf[N * before:], M, N, kb * 128, one)
+        assert torch.equal(out[e], one), (e, kb)
+        sl = slice(before * 128, (before + kb) * 128)
+        ref = T.dequant_act_f32(aq[:, sl].cuda(), a_s[:, before:before + kb].float().cuda()) @ \
+            T.dequant_act_f32(bq[:, sl].cuda(), b_s[:, before:before + kb].float().cuda()).T
+        check(out[e], ref, f"rowscale grouped problem {e} kb={kb}")
+        before += kb
+
+
 @pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200], [2048, 1024, 0, 4096]],
                          ids=["even", "uneven", "empty", "pad512"])
 def test_grouped_linear_backward(G, m_splits):
