@@ -39,9 +39,10 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 # Bytes per launch of the headline GEMM kernel between its L2s and the memory side (Infinity Cache / HBM): reads from
 # the request-size counters (32 / 64 / 128-byte TCC->EA reads, exact; the derived FETCH_SIZE prices the 128-byte
-# requests of LDS-direct and non-temporal loads at 64) plus WRITE_SIZE, from counter runs of this script.
-GEMM_BIG_TRAFFIC_BYTES = 430.0e6     # gemm_asm<256,256,1> on 16384 weight rows; profiles/gemm_fp8_block_config2_hbm_traffic.txt
-GEMM_MIXED_TRAFFIC_BYTES = 528.4e6   # gemm_asm_mixed on the whole problem; same file
+# requests of LDS-direct and non-temporal loads at 64) plus WRITE_SIZE.  Counters cannot be read from inside this process:
+# the figures are those of rocprofv3 --pmc runs of this script (profiles/gemm_kernels_mfma_lds_hbm_counters.txt), not of this run.
+GEMM_BIG_TRAFFIC_BYTES = 430.0e6     # gemm_asm<256,256,1> on 16384 weight rows: 362.9 MB read + 67.1 MB written
+GEMM_WIDE_TRAFFIC_BYTES = 457.9e6    # gemm_asm_wide<false> on the whole problem: 379.8 MB read + 78.1 MB written
 
 
 def main():
@@ -625,7 +626,7 @@ def main():
         "config": {"workload": "C2 dense block-FP8 GEMM: A[2048,7168] 1x128 e4m3 x B[18432,7168] 128x128 e4m3, fp32 scales -> bf16 [2048,18432]",
                    "M": M, "N": N, "K": K, "operands": "pre-quantised, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_MIXED_TRAFFIC_BYTES,
+                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_WIDE_TRAFFIC_BYTES,
                      "kernel": "gemm_asm_wide<false>: the whole problem in one launch, 512 tiles of 256x288 (two full rounds of 256 CUs)",
                      "launch_ms": ms, "flops_per_launch": flops, "wall_ms_per_step": wall_ms,
                      "tiles_256x256_alone": {"kernel": "gemm_asm<256,256,1>: M=2048, weight rows 0..16383 of 18432, K=7168 (512 tiles)",
