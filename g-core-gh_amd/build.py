@@ -54,11 +54,9 @@ def _compile(src: str, force: bool) -> str:
 
 
 def _generate():
-    """Regenerate the hand-scheduled GEMM loop when its generator is newer than the output."""
-    gen = os.path.join(CSRC, "gen_gemm_loop.py")
-    out = os.path.join(CSRC, "gemm_big_loop.inc")
-    if not os.path.exists(out) or os.path.getmtime(out) < os.path.getmtime(gen):
-        subprocess.check_call([sys.executable, gen])
+    """Run the generator of the hand-scheduled GEMM loops: it rewrites exactly those of its outputs (csrc/gemm_*_loop.inc)
+    whose content differs from what it generates, so a stale or hand-edited file never reaches the compiler."""
+    subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_gemm_loop.py")])
 
 
 def _audit_asm_operands():

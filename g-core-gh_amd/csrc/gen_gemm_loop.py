@@ -617,10 +617,14 @@ def main():
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)
         generate()
-        with open(os.path.join(here, name), "w") as f:
-            f.write("// Generated by gen_gemm_loop.py -- do not edit.\n")
-            for ln in lines:
-                f.write('"' + ln + '\\n"\n')
+        text = "// Generated by gen_gemm_loop.py -- do not edit.\n" + "".join('"' + ln + '\\n"\n' for ln in lines)
+        path = os.path.join(here, name)
+        # only files whose content differs are rewritten (their time stamps drive the rebuild), so running the
+        # generator on every build also undoes a hand edit to any of its outputs
+        if not os.path.exists(path) or open(path).read() != text:
+            with open(path, "w") as f:
+                f.write(text)
+            print("regenerated", name)
 
 
 if __name__ == "__main__":
