@@ -62,9 +62,10 @@ def _dequant_a(xq, xs):
     return xq.float() * _f32(xs).repeat_interleave(128, 1)
 
 
+@pytest.mark.parametrize("shape", [(2048, 18432, 7168), (4096, 7168, 18432)], ids=["config2", "deepK"])
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
-def test_prefill_gemm_at_benchmark_shape(G, pow2):
-    M, N, K = 2048, 18432, 7168
+def test_prefill_gemm_at_benchmark_shape(G, pow2, shape):
+    M, N, K = shape
     x, w = _randn(M, K, 1.0, 11), _randn(N, K, 0.02, 12)
     if pow2:
         xq, xs = G.quant_fp8_e4m3_scale_e8m0(x, (1, 128))
