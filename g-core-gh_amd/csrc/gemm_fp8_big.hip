@@ -416,18 +416,21 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     } else if constexpr (WN == 4) {
         // the early hand-back of this loop splits the weight copies by wave: the first four copy each wave column's first half
         const uint32_t lohalf = __builtin_amdgcn_readfirstlane(wave < WAVES / 2 ? 1u : 0u);
+        // a tile of at most 64 rows (an expert's short remainder) leaves the second wave row without activation rows: those
+        // waves run the loop's copy-and-barrier skeleton only
+        const uint32_t idle = __builtin_amdgcn_readfirstlane(wm == 1 && M - m0 <= 64 ? 1u : 0u);
         f32x16v acc0, acc1, acc2, acc3;
         if constexpr (HWS) {
             asm volatile(
 #include "gemm_flat_hw_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf), [idle] "s"(idle)
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         } else {
             asm volatile(
 #include "gemm_flat_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf), [idle] "s"(idle)
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;

@@ -35,12 +35,15 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE
+    # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
+    # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
+    WITH_IDLE, IDLE = idle, False
     HW = hw
     # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
@@ -124,7 +127,16 @@ WIDE_PART = ("mid", "mid", "end", "end", "end")
 _uid = 0
 
 
+IDLE = False        # emitting the loop body of a wave whose rows of the tile are all missing (see generate)
+
+
 def emit(s):
+    if IDLE:
+        # such a wave keeps its share of the copies, the barriers and the counters, and drops the arithmetic: fragment
+        # and scale reads, matrix instructions, folds, scale products, and the waits that only order those
+        if s.startswith(("ds_read", "v_mfma", "v_fmac", "v_mul_f32", "v_mov_b32", "v_add_u32", "s_load_dword", "s_waitcnt lgkmcnt")):
+            return
+        s = s.replace("%=", "i%=")
     lines.append(s)
 
 
@@ -484,6 +496,33 @@ def step(c):
         fold(NB - 1, mb, c)
 
 
+def loop_body():
+    emit("Lloop%=:")
+    if HW:
+        # scales of this group: the lane's activation-scale bytes and the weight-scale bytes (uniform)
+        for mb in range(MB):
+            emit(f"v_mov_b32 v{SAN + mb}, v{SC + mb}")
+        if BROW:
+            for nb in range(NB):
+                emit(f"v_mov_b32 v{WSN + nb}, v{WSC + nb}")
+        else:
+            emit(f"v_mov_b32 {WS1}, s60")
+            if WIDE:
+                emit(f"v_mov_b32 {WS2}, s68")
+    emit("s_mov_b64 s[56:57], s[60:61]")
+    emit("s_mov_b64 s[58:59], s[62:63]")
+    if SPLIT or WIDE:
+        emit("s_mov_b64 s[64:65], s[68:69]")
+        emit("s_mov_b64 s[66:67], s[70:71]")
+    emit("s_sub_u32 s49, s49, 1")
+    emit("s_cmp_eq_u32 s49, 0")
+    emit("s_cselect_b32 s50, 1, 0")
+    for c in range(4):
+        step(c)
+    emit("s_cmp_lg_u32 s50, 1")
+    emit("s_cbranch_scc1 Lloop%=")
+
+
 def generate():
     # ---- prologue
     # Activation rows past the end of the matrix (or of an expert's rows) are not copied: their lanes are switched off
@@ -572,30 +611,17 @@ def generate():
     for mb in range(MB):
         read_frag(AF + 8 * mb, RA0, RA1, mb * 2048)
     # ---- main loop: one trip = four K steps = one group of scales
-    emit("Lloop%=:")
-    if HW:
-        # scales of this group: the lane's activation-scale bytes and the weight-scale bytes (uniform)
-        for mb in range(MB):
-            emit(f"v_mov_b32 v{SAN + mb}, v{SC + mb}")
-        if BROW:
-            for nb in range(NB):
-                emit(f"v_mov_b32 v{WSN + nb}, v{WSC + nb}")
-        else:
-            emit(f"v_mov_b32 {WS1}, s60")
-            if WIDE:
-                emit(f"v_mov_b32 {WS2}, s68")
-    emit("s_mov_b64 s[56:57], s[60:61]")
-    emit("s_mov_b64 s[58:59], s[62:63]")
-    if SPLIT or WIDE:
-        emit("s_mov_b64 s[64:65], s[68:69]")
-        emit("s_mov_b64 s[66:67], s[70:71]")
-    emit("s_sub_u32 s49, s49, 1")
-    emit("s_cmp_eq_u32 s49, 0")
-    emit("s_cselect_b32 s50, 1, 0")
-    for c in range(4):
-        step(c)
-    emit("s_cmp_lg_u32 s50, 1")
-    emit("s_cbranch_scc1 Lloop%=")
+    global IDLE
+    if WITH_IDLE:
+        emit("s_cmp_eq_u32 %[idle], 1")
+        emit("s_cbranch_scc1 Lloopi%=")
+    loop_body()
+    if WITH_IDLE:
+        emit("s_branch Ldone%=")
+        IDLE = True
+        loop_body()
+        IDLE = False
+        emit("Ldone%=:")
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     if HW:
         emit("s_nop 15")                         # the last MFMAs have written the accumulators before they are read
@@ -611,8 +637,8 @@ def main():
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
                       ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True)),
                       ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True)),
-                      ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True)),
-                      ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True)),
+                      ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
+                      ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)
