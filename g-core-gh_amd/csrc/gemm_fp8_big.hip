@@ -224,13 +224,13 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
         [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
-        [g4] "s"(g4), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [g4] "s"(g4), [idle] "s"(idle), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
         [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies),            \
-        [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [idle] "s"(idle), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 
 // Index arithmetic of the staged bf16 epilogue for a wave tile of 64 rows x COLS columns (COLS = 128, 96 or 64).
 // A row of the staging region holds COLS bf16 plus 16 bytes of padding (rows then start 4 banks apart: the 8-byte
@@ -372,6 +372,10 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t bextra = __builtin_amdgcn_readfirstlane(wave < (TN / 8) % WAVES ? 1u : 0u);
     const uint32_t bstride = __builtin_amdgcn_readfirstlane((uint32_t)(8 * K));
     const uint32_t g4 = __builtin_amdgcn_readfirstlane(wave < 2 ? 16u : 32u);
+    // A wave none of whose 64 activation rows exist (the tail of M, or an expert's short tile) runs the loop's
+    // copy-and-barrier skeleton only, in the loops generated with that second body (256-row and flat tiles).
+    const uint32_t idle = __builtin_amdgcn_readfirstlane((int64_t)wm * 64 >= M - m0 ? 1u : 0u);
+    (void)idle;
     (void)splitnb; (void)bextra; (void)bstride; (void)g4;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
@@ -416,21 +420,18 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     } else if constexpr (WN == 4) {
         // the early hand-back of this loop splits the weight copies by wave: the first four copy each wave column's first half
         const uint32_t lohalf = __builtin_amdgcn_readfirstlane(wave < WAVES / 2 ? 1u : 0u);
-        // a tile of at most 64 rows (an expert's short remainder) leaves the second wave row without activation rows: those
-        // waves run the loop's copy-and-barrier skeleton only
-        const uint32_t idle = __builtin_amdgcn_readfirstlane(wm == 1 && M - m0 <= 64 ? 1u : 0u);
         f32x16v acc0, acc1, acc2, acc3;
         if constexpr (HWS) {
             asm volatile(
 #include "gemm_flat_hw_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf), [idle] "s"(idle)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         } else {
             asm volatile(
 #include "gemm_flat_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf), [idle] "s"(idle)
+                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
