@@ -764,12 +764,6 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
 // be re-used out of one L2.
 constexpr int kMixedMaxExperts = 512;
 
-__device__ __forceinline__ int64_t dev_padded_grid(int64_t tiles_m, int64_t tiles_n)
-{
-    const int64_t chunks = (tiles_m * tiles_n + gemm::CHUNK - 1) / gemm::CHUNK;
-    return ((chunks + 7) / 8) * 8 * gemm::CHUNK;
-}
-
 template <bool HWS>
 __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                               const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
@@ -803,37 +797,45 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
         tot_big += vb;
         tot_small += vs;
     }
-    // ---- which class and which tile of it this workgroup takes
-    const int64_t tiles_n = N >> 8;
-    const int64_t slots_big = dev_padded_grid(tot_big, tiles_n) >> 3, slots_small = dev_padded_grid(tot_small, tiles_n) >> 3;
-    const int64_t xcd = blockIdx.x & 7, sidx = blockIdx.x >> 3;
+    // ---- which class and which tile of it this workgroup takes (32-bit arithmetic: the grid is below 2^31, and 64-bit
+    // divisions by run-time values would cost this prologue about a microsecond per workgroup)
+    const uint32_t tiles_n = (uint32_t)(N >> 8);
+    auto padded_slots = [](uint32_t tiles) -> uint32_t {                   // workgroups per XCD for that many tiles
+        const uint32_t chunks = (tiles + gemm::CHUNK - 1) / gemm::CHUNK;
+        return ((chunks + 7) / 8) * gemm::CHUNK;
+    };
+    const uint32_t slots_big = padded_slots((uint32_t)tot_big * tiles_n), slots_small = padded_slots((uint32_t)tot_small * tiles_n);
+    const uint32_t xcd = blockIdx.x & 7, sidx = blockIdx.x >> 3;
     if (sidx >= slots_big + slots_small) return;
-    int64_t ps = slots_big > 0 ? (slots_small + slots_big / 2) / slots_big : 1;
-    if (ps < 1) ps = 1;
-    const int64_t period = 1 + ps;
-    const int64_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
     bool big;
-    int64_t idx;
+    uint32_t idx;
     if (small_first > 0) {
         // XCDs below small_first work through their small tiles first and then their big ones, the others the other way
         // round: every XCD has the same share of both classes, and at any time some XCDs stream weights while the
         // others compute, each class with an L2 to itself
-        if (xcd < small_first) { big = sidx >= slots_small; idx = big ? sidx - slots_small : sidx; }
+        if (xcd < (uint32_t)small_first) { big = sidx >= slots_small; idx = big ? sidx - slots_small : sidx; }
         else { big = sidx < slots_big; idx = big ? sidx : sidx - slots_big; }
-    } else if (sidx < rounds * period) {
-        const int64_t r = sidx % period, q = sidx / period;
-        big = r == 0;
-        idx = big ? q : q * ps + (r - 1);
     } else {
-        const int64_t w = sidx - rounds * period, left_big = slots_big - rounds;
-        big = w < left_big;
-        idx = big ? rounds + w : rounds * ps + (w - left_big);
+        // the classes dealt alternately in the ratio of their sizes (1 big : ps small)
+        uint32_t ps = slots_big > 0 ? (slots_small + slots_big / 2) / slots_big : 1;
+        if (ps < 1) ps = 1;
+        const uint32_t period = 1 + ps;
+        const uint32_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
+        if (sidx < rounds * period) {
+            const uint32_t r = sidx % period, q = sidx / period;
+            big = r == 0;
+            idx = big ? q : q * ps + (r - 1);
+        } else {
+            const uint32_t w = sidx - rounds * period, left_big = slots_big - rounds;
+            big = w < left_big;
+            idx = big ? rounds + w : rounds * ps + (w - left_big);
+        }
     }
     // Tiles of a class are numbered expert by expert (expert e owns tiles_n numbers per row tile) and an XCD takes 32
     // consecutive numbers at a time, so the tiles it runs together belong to one expert, or to neighbours.
-    const int64_t lin = ((idx / gemm::CHUNK) * 8 + xcd) * gemm::CHUNK + idx % gemm::CHUNK;
-    if (lin >= (int64_t)(big ? tot_big : tot_small) * tiles_n) return;
-    const int64_t gmt = lin / tiles_n;
+    const uint32_t lin = ((idx / gemm::CHUNK) * 8 + xcd) * gemm::CHUNK + idx % gemm::CHUNK;
+    if (lin >= (uint32_t)(big ? tot_big : tot_small) * tiles_n) return;
+    const int gmt = (int)(lin / tiles_n);
     // ---- the expert that owns row tile gmt of the class tells the others
     {
         const int cnt = big ? nb : ns, incl = big ? ib : is;
@@ -850,13 +852,13 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
     // gm activation panels and gn weight panels of one expert (one row tile: its activations and the whole weight matrix once).
     int64_t local, tn;
     {
-        const int64_t in_e = lin - (int64_t)found_first * tiles_n, per_group = gemm::GROUP_M * tiles_n;
-        const int64_t grp = in_e / per_group, in_grp = in_e - grp * per_group;
-        const int64_t left = found_cnt - grp * gemm::GROUP_M;
-        const int64_t gm = left < gemm::GROUP_M ? left : gemm::GROUP_M;
-        const int64_t gn = gemm::CHUNK / gm;
-        const int64_t per_nblock = gm * gn;
-        const int64_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
+        const uint32_t in_e = lin - (uint32_t)found_first * tiles_n, per_group = gemm::GROUP_M * tiles_n;
+        const uint32_t grp = in_e / per_group, in_grp = in_e - grp * per_group;
+        const uint32_t left = (uint32_t)found_cnt - grp * gemm::GROUP_M;
+        const uint32_t gm = left < gemm::GROUP_M ? left : gemm::GROUP_M;
+        const uint32_t gn = gemm::CHUNK / gm;
+        const uint32_t per_nblock = gm * gn;
+        const uint32_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
         local = grp * gemm::GROUP_M + in_blk % gm;
         tn = nblk * gn + in_blk / gm;
     }
