@@ -460,6 +460,13 @@ def main():
                 "m_splits_histogram": {f"<={hi}": int(((m_splits > lo) & (m_splits <= hi)).sum())
                                        for lo, hi in ((-1, 0), (0, 64), (64, 128), (128, 256), (256, 512), (512, 1024),
                                                       (1024, 2048), (2048, 4096), (4096, 8192))}}
+        # rows the launch multiplies over rows that exist: every 256 rows of an expert and a remainder above 128 rows
+        # are 256-row tiles, a remainder of 1 .. 128 rows is a 128-row tile; waves whose 64 rows are all missing skip
+        # their matrix instructions, so the matrix cores see the rows rounded up to 64
+        ms_l = m_splits.tolist()
+        tile_rows = sum((r >> 8) * 256 + (256 if (r & 255) > 128 else (128 if (r & 255) else 0)) for r in ms_l)
+        mfma_rows = sum((r + 63) // 64 * 64 for r in ms_l)
+        res4["padded_over_useful_flops"] = {"by_tile_rows": tile_rows / Mt, "after_idle_wave_rows_are_skipped": mfma_rows / Mt}
         for name, (N4, K4) in (("gate_up", (4096, 7168)), ("down", (7168, 2048))):
             x4 = randn(Mt, K4)
             x4q = torch.empty(Mt, K4, dtype=torch.uint8, device=dev)
