@@ -575,7 +575,11 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
             const int64_t n = wcol0 + nb * 16 + 4 * lq;
             if (n >= N) continue;
             const float v0 = accs[nb][mb * 4], v1 = accs[nb][mb * 4 + 1], v2 = accs[nb][mb * 4 + 2], v3 = accs[nb][mb * 4 + 3];
-            if (out_dtype == LP_BF16) {
+            if (out_dtype == LP_E4M3) {
+                // e4m3fn output (the unscaled NT GEMM routed here): round to nearest even, saturate at +-448, NaN stays NaN
+                auto sat = [](float x) { const float c = __builtin_fminf(__builtin_fmaxf(x, -kE4M3Max), kE4M3Max); return x != x ? x : c; };
+                *(uint32_t *)((uint8_t *)C + arow[mb] * ldc + n) = cvt4(sat(v0), sat(v1), sat(v2), sat(v3));
+            } else if (out_dtype == LP_BF16) {
                 u32x2 o = {pack_bf16(v0, v1), pack_bf16(v2, v3)};
                 *(u32x2 *)((uint16_t *)C + arow[mb] * ldc + n) = o;
             } else {
@@ -949,6 +953,25 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
     if (scale_dtype == LP_F32) GO(LP_F32);
     GO(LP_E8M0);
 #undef GO
+}
+
+// Unscaled fp8 NT GEMM on the hardware-scaled 256 x 256 loop with every scale byte 0x7F (2^0): `ones` holds at least
+// max(M, N / 128) * K / 128 such bytes.  out_dtype may be LP_E4M3 here (see tile_asm's last store loop).
+int launch_nt_unit_scales(const void *A, const void *B, const void *ones, int64_t M, int64_t N, int64_t K, void *C, int out_dtype,
+                          hipStream_t st)
+{
+    const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
+    const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_nt: problem too large");
+    hipLaunchKernelGGL((gemm_asm<256, 256, 1, true>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)A, (const float *)ones,
+                       (const uint8_t *)B, (const float *)ones, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+    return check_launch("lp_gemm_nt(asm, unit scales)");
+}
+
+bool nt_unit_scales_ok(const void *ones, int64_t M, int64_t N, int64_t K)
+{
+    static const bool no_asm = getenv("LP_GEMM_NO_ASM") != nullptr;
+    return !no_asm && asm_shape_ok(ones, ones, M, N, K, LP_E8M0);
 }
 
 // 256 x 288 tiles when they divide N and fill the last round of tiles better than 256 x 256 tiles would; false when

@@ -8,6 +8,9 @@
 // 16 x 16 block), two v_mfma_f32_16x16x32_bf16 for bf16.  The weight fragment is the MFMA A
 // operand, the activation fragment the B operand: a lane then holds 4 consecutive output columns
 // of one output row, which makes the stores 8 / 16 bytes wide.
+#include <pthread.h>
+#include <stdlib.h>
+
 #include "gemm_common.h"
 
 using namespace lowp;
@@ -169,6 +172,45 @@ int launch(const void *A, const void *B, int64_t M, int64_t N, int64_t row_bytes
     return check_launch("lp_gemm_nt");
 }
 
+// Unit scales for routing fp8 problems through the block-scaled kernels (below): 1 MiB of e8m0 bytes 0x7F (= 2^0) in the
+// library's device image, one copy per GPU, filled by a small kernel at a GPU's first use.  Host code reaches the array
+// through the address hipGetSymbolAddress returns for the current device.
+constexpr int64_t kUnitScaleBytes = 1 << 20;
+__device__ __align__(256) uint8_t unit_scales[kUnitScaleBytes];
+constexpr int kMaxDevices = 64;
+void *g_unit_ptr[kMaxDevices];               // device address per device ordinal once the array is filled
+pthread_mutex_t g_unit_lock = PTHREAD_MUTEX_INITIALIZER;
+
+__global__ __launch_bounds__(256) void fill_bytes(u32x4 *dst, uint32_t word)
+{
+    dst[(int64_t)blockIdx.x * 256 + threadIdx.x] = u32x4{word, word, word, word};
+}
+
+// nullptr when the array cannot be used for this call: device ordinal out of range, a HIP error, or the first use on
+// this device falls inside a stream capture (the fill must have run before anything reads the array).
+const void *unit_scale_array(hipStream_t st)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    pthread_mutex_lock(&g_unit_lock);
+    void *p = g_unit_ptr[dev];
+    if (!p) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        void *q = nullptr;
+        if (hipStreamIsCapturing(st, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone &&
+            hipGetSymbolAddress(&q, HIP_SYMBOL(unit_scales)) == hipSuccess && q) {
+            hipLaunchKernelGGL(fill_bytes, dim3((unsigned)(kUnitScaleBytes / 16 / 256)), dim3(256), 0, st, (u32x4 *)q, 0x7F7F7F7Fu);
+            // the fill is ordered before this call's kernels on `st`; other streams may only use the array once it is
+            // complete, so the address is published after the stream has drained (once per device and process)
+            if (hipGetLastError() == hipSuccess && hipStreamSynchronize(st) == hipSuccess) g_unit_ptr[dev] = p = q;
+        } else {
+            (void)hipGetLastError();
+        }
+    }
+    pthread_mutex_unlock(&g_unit_lock);
+    return p;
+}
+
 }  // namespace
 
 extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M, int64_t N, int64_t K, void *C,
@@ -187,6 +229,15 @@ extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M,
     LP_REQUIRE((uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 && (uintptr_t)C % 16 == 0,
                "lp_gemm_nt: operands must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
+    // fp8 operands, K in whole groups of 512, enough 256 x 256 tiles to fill the chip: the block-scaled GEMM's hand-scheduled
+    // loop with every scale 2^0 (e8m0 scales are applied inside the matrix instruction at no cost), instead of the
+    // compiler-scheduled kernel below.  LP_GEMM_NT_PLAIN=1 keeps that one.
+    static const bool plain = getenv("LP_GEMM_NT_PLAIN") != nullptr;
+    if (!plain && in_dtype == LP_E4M3 && K % 512 == 0 && N % 16 == 0 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
+        M * (K / 128) <= kUnitScaleBytes && ((N + 127) / 128) * (K / 128) <= kUnitScaleBytes) {
+        const void *ones = unit_scale_array(st);
+        if (ones && gemm::nt_unit_scales_ok(ones, M, N, K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, K, C, out_dtype, st);
+    }
     // 256 x 256 tiles once they fill the machine about twice, 128 x 128 otherwise
     const bool big = M >= 192 && ((M + 255) / 256) * ((N + 255) / 256) >= 400;
     if (in_dtype == LP_BF16)
