@@ -224,13 +224,13 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
         [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
-        [g4] "s"(g4), [idle] "s"(idle), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [g4] "s"(g4), [idle] "s"(idle), [grp] "s"(grp), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
         [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies),            \
-        [idle] "s"(idle), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [idle] "s"(idle), [grp] "s"(grp), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 
 // Index arithmetic of the staged bf16 epilogue for a wave tile of 64 rows x COLS columns (COLS = 128, 96 or 64).
 // A row of the staging region holds COLS bf16 plus 16 bytes of padding (rows then start 4 banks apart: the 8-byte
@@ -376,6 +376,9 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     // copy-and-barrier skeleton only, in the loops generated with that second body (256-row and flat tiles).
     const uint32_t idle = __builtin_amdgcn_readfirstlane((int64_t)wm * 64 >= M - m0 ? 1u : 0u);
     (void)idle;
+    // second half of the workgroup's waves: on every SIMD it shares the matrix pipe with a wave of the first half
+    const uint32_t grp = __builtin_amdgcn_readfirstlane((DUAL ? (t >> 6) & (WAVES - 1) : t >> 6) >= WAVES / 2 ? 1u : 0u);
+    (void)grp;
     (void)splitnb; (void)bextra; (void)bstride; (void)g4;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).

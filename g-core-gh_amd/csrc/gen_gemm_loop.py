@@ -35,15 +35,23 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False, pingpong=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP
     # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
     # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
     WITH_IDLE, IDLE = idle, False
+    # pingpong: a SIMD holds one wave of the first half of the workgroup's waves and one of the second half, and its
+    # arbiter prefers the older one: measured on the 256 x 256 loop, waves 0..3 spent 38 % of the loop waiting at the
+    # barriers for waves 4..7 (12 %), which then ran alone and could not keep the matrix pipe busy.  With pingpong the
+    # two halves run their own copy of the loop in which the wave priority (s_setprio) alternates from block to block,
+    # opposite in the two copies: one wave issues its block's matrix instructions while the other folds and reads.
+    # Measured: the two halves then wait alike (13 % and 9 %) and the 256 x 256 and 256 x 288 loops gain 1 - 2 %; the
+    # flat 128 x 256 loop of the grouped kernel gains nothing and keeps one body.
+    PINGPONG, GRP = pingpong, 0
     HW = hw
     # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
@@ -128,15 +136,18 @@ _uid = 0
 
 
 IDLE = False        # emitting the loop body of a wave whose rows of the tile are all missing (see generate)
+GRP = 0             # which half of the waves the body being emitted is for (see configure: pingpong)
 
 
 def emit(s):
     if IDLE:
         # such a wave keeps its share of the copies, the barriers and the counters, and drops the arithmetic: fragment
         # and scale reads, matrix instructions, folds, scale products, and the waits that only order those
-        if s.startswith(("ds_read", "v_mfma", "v_fmac", "v_mul_f32", "v_mov_b32", "v_add_u32", "s_load_dword", "s_waitcnt lgkmcnt")):
+        if s.startswith(("ds_read", "v_mfma", "v_fmac", "v_mul_f32", "v_mov_b32", "v_add_u32", "s_load_dword", "s_waitcnt lgkmcnt", "s_setprio")):
             return
         s = s.replace("%=", "i%=")
+    elif GRP == 1:
+        s = s.replace("%=", "b%=")
     lines.append(s)
 
 
@@ -391,11 +402,15 @@ def step(c):
             emit(f"v_add_u32 v{SRDB}, s55, v{SRDB0}")
     read_frag(WFB[par(c, 1)], RB0, RB1, boff + 2048)
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
+    if PINGPONG:
+        emit(f"s_setprio {(c * NB + GRP + 1) & 1}")
     for mb in range(MB):
         emit(f"s_waitcnt lgkmcnt({8 - 2 * mb})")
         mfma(0, mb, c)
     read_scales((c + 1) & 3)
     for nb in range(1, NB):
+        if PINGPONG:
+            emit(f"s_setprio {(c * NB + nb + GRP + 1) & 1}")
         if HW and WIDE:
             # from the first block in the second weight-scale block on, the matrix instructions take that row's bytes
             emit(f"s_cmp_eq_u32 s74, {nb}")
@@ -612,16 +627,28 @@ def generate():
         read_frag(AF + 8 * mb, RA0, RA1, mb * 2048)
     # ---- main loop: one trip = four K steps = one group of scales
     global IDLE
+    global GRP
     if WITH_IDLE:
         emit("s_cmp_eq_u32 %[idle], 1")
         emit("s_cbranch_scc1 Lloopi%=")
+    if PINGPONG:
+        emit("s_cmp_eq_u32 %[grp], 1")
+        emit("s_cbranch_scc1 Lloopb%=")
     loop_body()
+    if PINGPONG:
+        emit("s_branch Ldone%=")
+        GRP = 1
+        loop_body()
+        GRP = 0
     if WITH_IDLE:
         emit("s_branch Ldone%=")
         IDLE = True
         loop_body()
         IDLE = False
+    if WITH_IDLE or PINGPONG:
         emit("Ldone%=:")
+    if PINGPONG:
+        emit("s_setprio 0")
     emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     if HW:
         emit("s_nop 15")                         # the last MFMAs have written the accumulators before they are read
@@ -629,14 +656,17 @@ def generate():
 
 
 
+PP = os.environ.get("LP_GEN_PINGPONG", "1") == "1"
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
-    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1, False, 2, False, True, False, True)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
+    for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1, False, 2, False, True, False, True, PP)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
                       ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
-                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True)),
+                      ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True, PP)),
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
-                      ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True, True)),
-                      ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True, True)),
+                      ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True, True, PP)),
+                      ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True, True, PP)),
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
                       ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
