@@ -47,11 +47,14 @@ def load_template(path: str):
     patterns = []
     for text in lines:
         literal |= _regs(re.sub(r"%\[\w+\]", " ", text))
+        if re.search(r"\bvcc", text) or re.search(r"\bv_(?:add_co|addc_co|sub_co|subb_co|div_scale|cmpx?_\w+(?<!_e64)\s)", text):
+            raise RuntimeError(f"{path}: the loop uses vcc, which the compiler may assign to a scalar operand: {text}")
         parts = re.split(r"(%\[\w+\])", text)
         rx, n = "", 0
         for p in parts:
             if p.startswith("%["):
-                rx += rf"(?P<{p[2:-1]}__{n}>[vs](?:\d+|\[\d+:\d+\]))"
+                # the compiler may hand a scalar operand vcc (a loop that names vcc fails in load_template)
+                rx += rf"(?P<{p[2:-1]}__{n}>[vs](?:\d+|\[\d+:\d+\])|vcc(?:_lo|_hi)?)"
                 n += 1
             else:
                 rx += r"\s+".join(re.escape(w) for w in p.split(" ")).replace("%=", r"\d+") if p else ""

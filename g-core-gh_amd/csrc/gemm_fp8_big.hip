@@ -223,14 +223,14 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
-        [trips] "s"(trips), [copies] "s"(copies), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
-        [g4] "s"(g4), [idle] "s"(idle), [grp] "s"(grp), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [trips] "s"(trips), [flags] "s"(flags), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
+        [g4] "s"(g4), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
         [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u),       \
-        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [copies] "s"(copies),            \
-        [idle] "s"(idle), [grp] "s"(grp), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+        [sbase] "s"(s_u), [bsptr] "s"(bs_u), [m0base] "s"(m0base), [trips] "s"(trips), [flags] "s"(flags),              \
+        [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 
 // Index arithmetic of the staged bf16 epilogue for a wave tile of 64 rows x COLS columns (COLS = 128, 96 or 64).
 // A row of the staging region holds COLS bf16 plus 16 bytes of padding (rows then start 4 banks apart: the 8-byte
@@ -302,7 +302,11 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     static_assert((TM / 8 / WAVES == 4 || (WN == 4 && TM / 8 / WAVES == 2)) && (TN / 8 / WAVES == 4 || TN / 8 / WAVES == 3),
                   "copies per operand and wave");
     constexpr int NBC = TN / 8 / WAVES;                 // weight copies per wave and K block
-    const int t = threadIdx.x, lane = t & 63, wave = DUAL ? (t >> 6) & (WAVES - 1) : t >> 6;
+    // The thread index is made opaque: called in a loop over tiles, everything below that depends only on it would otherwise be
+    // kept in registers across the previous tile's loop, which leaves the compiler v0 .. v29, and be spilled.
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    const int lane = t & 63, wave = DUAL ? (t >> 6) & (WAVES - 1) : t >> 6;
     const int kg = DUAL ? __builtin_amdgcn_readfirstlane(t >> 6) / WAVES : 0;                 // which half of K
     const int wm = wave / WN, wn = wave % WN;
     const int l16 = lane & 15, lq = lane >> 4;
@@ -333,10 +337,8 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     for (int i = 0; i < 4; ++i) {
         const int row = 8 * (wave + WAVES * i) + ld_row;
         amask[i] = __ballot(m0 + row < M);
-        // Rows past the end of the activations wrap around inside the tile's valid rows instead of all landing on the
-        // last one: with a few valid rows (an expert's short tile) every copy of every tile of that expert would
-        // otherwise ask one L2 channel for the same 128 bytes at the same time.
-        const int64_t m = m0 + row < M ? m0 + row : m0 + row % (int)(M - m0);
+        // a lane whose row is past the end of the activations is switched off for the copy (amask): its offset only has to exist
+        const int64_t m = m0 + row < M ? m0 + row : m0;
         const int64_t n = n0 + row < N ? n0 + row : N - 1;          // i = 3 is unused when there are three copies
         aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
         boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
@@ -375,10 +377,16 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     // A wave none of whose 64 activation rows exist (the tail of M, or an expert's short tile) runs the loop's
     // copy-and-barrier skeleton only, in the loops generated with that second body (256-row and flat tiles).
     const uint32_t idle = __builtin_amdgcn_readfirstlane((int64_t)wm * 64 >= M - m0 ? 1u : 0u);
-    (void)idle;
     // second half of the workgroup's waves: on every SIMD it shares the matrix pipe with a wave of the first half
     const uint32_t grp = __builtin_amdgcn_readfirstlane((DUAL ? (t >> 6) & (WAVES - 1) : t >> 6) >= WAVES / 2 ? 1u : 0u);
-    (void)grp;
+    // the wave's flags travel in one scalar operand: bit 0 copies scales, 1 idle, 2 second half of the waves, 3 first half
+    // (read into the scalar register by hand: left to the compiler, the combined value can end up in a vector register,
+    // which the loop's scalar instructions cannot take.  The s_nop: the compiler does not look into the statement, and
+    // when the instruction it places right in front is the one that writes the vector register, v_readfirstlane reads
+    // the register's old value -- seen as waves that copied no activation scales, or the wrong waves' scales.)
+    const uint32_t flags_v = copies | idle << 1 | grp << 2 | (grp ^ 1u) << 3;
+    uint32_t flags;
+    asm volatile("s_nop 4\n\tv_readfirstlane_b32 %0, %1" : "=s"(flags) : "v"(flags_v));
     (void)splitnb; (void)bextra; (void)bstride; (void)g4;
 
     // LDS addresses: DMA base of this wave, fragment read addresses of this lane (stage 0).
@@ -422,19 +430,18 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         accs[5] = acc5; accs[6] = acc6; accs[7] = acc7; accs[8] = acc8;
     } else if constexpr (WN == 4) {
         // the early hand-back of this loop splits the weight copies by wave: the first four copy each wave column's first half
-        const uint32_t lohalf = __builtin_amdgcn_readfirstlane(wave < WAVES / 2 ? 1u : 0u);
         f32x16v acc0, acc1, acc2, acc3;
         if constexpr (HWS) {
             asm volatile(
 #include "gemm_flat_hw_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_INPUTS
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         } else {
             asm volatile(
 #include "gemm_flat_loop.inc"
                 : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
-                : LP_ASM_INPUTS, [lohalf] "s"(lohalf)
+                : LP_ASM_INPUTS
                 : LP_ASM_CLOBBERS, "s87", "s89", "s90", "s91", "s92");
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
@@ -780,30 +787,38 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
     constexpr int LDS_BIG = AsmTile<256, 256, 1>::LDS_BYTES, LDS_FLAT = AsmTile<128, 256, 1, 3, 4>::LDS_BYTES;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BIG > LDS_FLAT ? LDS_BIG : LDS_FLAT];
     __shared__ int wave_big[8], wave_small[8];
-    __shared__ int found_e, found_first, found_begin, found_rows, found_cnt;
+    // row tiles of the experts up to and including e, per class (what a workgroup searches for its tile's expert)
+    __shared__ int upto_big[kMixedMaxExperts], upto_small[kMixedMaxExperts];
+    constexpr int kTable = 256;
+    __shared__ int4 table[kTable];                      // this workgroup's next tiles
     const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
-    // ---- this thread's expert: rows, tiles of both classes, running counts over the experts before it
-    int64_t begin = 0;
-    const int rows = t < E ? gemm::expert_rows(m_offsets, t, M_total, begin) : 0;
-    const int rem = rows & 255;
-    const int nb = (rows >> 8) + (rem > 128 ? 1 : 0), ns = rem > 0 && rem <= 128 ? 1 : 0;
-    int ib = nb, is = ns;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const int ub = __shfl_up(ib, off), us = __shfl_up(is, off);
-        if (lane >= off) { ib += ub; is += us; }
-    }
-    if (lane == 63) { wave_big[wv] = ib; wave_small[wv] = is; }
-    if (t == 0) found_e = -1;
-    __syncthreads();
     int tot_big = 0, tot_small = 0;
+    {
+        // thread t's expert: rows, tiles of both classes, running counts over the experts before it
+        int64_t begin = 0;
+        const int rows = t < E ? gemm::expert_rows(m_offsets, t, M_total, begin) : 0;
+        const int rem = rows & 255;
+        const int nb = (rows >> 8) + (rem > 128 ? 1 : 0), ns = rem > 0 && rem <= 128 ? 1 : 0;
+        int ib = nb, is = ns;
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-        const int vb = wave_big[w], vs = wave_small[w];
-        if (w < wv) { ib += vb; is += vs; }
-        tot_big += vb;
-        tot_small += vs;
+        for (int off = 1; off < 64; off <<= 1) {
+            const int ub = __shfl_up(ib, off), us = __shfl_up(is, off);
+            if (lane >= off) { ib += ub; is += us; }
+        }
+        if (lane == 63) { wave_big[wv] = ib; wave_small[wv] = is; }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            const int vb = wave_big[w], vs = wave_small[w];
+            if (w < wv) { ib += vb; is += vs; }
+            tot_big += vb;
+            tot_small += vs;
+        }
+        upto_big[t] = ib;
+        upto_small[t] = is;
     }
+    tot_big = __builtin_amdgcn_readfirstlane(tot_big);
+    tot_small = __builtin_amdgcn_readfirstlane(tot_small);
     // ---- which class and which tile of it this workgroup takes (32-bit arithmetic: the grid is below 2^31, and 64-bit
     // divisions by run-time values would cost this prologue about a microsecond per workgroup)
     const uint32_t tiles_n = (uint32_t)(N >> 8);
@@ -812,69 +827,100 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
         return ((chunks + 7) / 8) * gemm::CHUNK;
     };
     const uint32_t slots_big = padded_slots((uint32_t)tot_big * tiles_n), slots_small = padded_slots((uint32_t)tot_small * tiles_n);
-    const uint32_t xcd = blockIdx.x & 7, sidx = blockIdx.x >> 3;
-    if (sidx >= slots_big + slots_small) return;
-    bool big;
-    uint32_t idx;
-    if (small_first > 0) {
-        // XCDs below small_first work through their small tiles first and then their big ones, the others the other way
-        // round: every XCD has the same share of both classes, and at any time some XCDs stream weights while the
-        // others compute, each class with an L2 to itself
-        if (xcd < (uint32_t)small_first) { big = sidx >= slots_small; idx = big ? sidx - slots_small : sidx; }
-        else { big = sidx < slots_big; idx = big ? sidx : sidx - slots_big; }
-    } else {
-        // the classes dealt alternately in the ratio of their sizes (1 big : ps small)
-        uint32_t ps = slots_big > 0 ? (slots_small + slots_big / 2) / slots_big : 1;
-        if (ps < 1) ps = 1;
-        const uint32_t period = 1 + ps;
-        const uint32_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
-        if (sidx < rounds * period) {
-            const uint32_t r = sidx % period, q = sidx / period;
-            big = r == 0;
-            idx = big ? q : q * ps + (r - 1);
-        } else {
-            const uint32_t w = sidx - rounds * period, left_big = slots_big - rounds;
-            big = w < left_big;
-            idx = big ? rounds + w : rounds * ps + (w - left_big);
+    // A workgroup takes slots blockIdx.x, blockIdx.x + gridDim.x, ...: with one workgroup per CU (grid = number of CUs, a
+    // multiple of 8, so a workgroup stays on its XCD's share of the slots) the scan above is paid once per CU instead of
+    // once per tile; with a grid of all slots the loop below runs once.  The workgroup's tiles are looked up kTable slots at a
+    // time, one slot per thread, and listed in LDS: between two tiles only a table entry is read (a workgroup has its CU to
+    // itself, so whatever happens between two K loops is time the matrix cores stand still).
+    __syncthreads();                                    // the running counts are written
+    const uint32_t slots = slots_big + slots_small;
+    const uint64_t all_slots = (uint64_t)slots * 8;     // below 2^31
+    const int64_t kblocks = K / KB;
+    for (uint64_t first = blockIdx.x; first < all_slots; first += (uint64_t)kTable * gridDim.x) {
+        __syncthreads();                                // every thread has read the previous batch's last entry
+        if (t < kTable) {
+            const uint64_t slot64 = first + (uint64_t)t * gridDim.x;
+            int4 entry = {-1, 0, 0, 0};                 // expert (-1: no tile; bit 30: 256-row tile), first row, end of the expert's rows, first column
+            if (slot64 < all_slots) {
+                const uint32_t slot = (uint32_t)slot64;
+                const uint32_t xcd = slot & 7, sidx = slot >> 3;
+                bool big;
+                uint32_t idx;
+                if (small_first > 0) {
+                    // XCDs below small_first work through their small tiles first and then their big ones, the others the
+                    // other way round: every XCD has the same share of both classes, and at any time some XCDs stream weights
+                    // while the others compute, each class with an L2 to itself
+                    if (xcd < (uint32_t)small_first) { big = sidx >= slots_small; idx = big ? sidx - slots_small : sidx; }
+                    else { big = sidx < slots_big; idx = big ? sidx : sidx - slots_big; }
+                } else {
+                    // the classes dealt alternately in the ratio of their sizes (1 big : ps small)
+                    uint32_t ps = slots_big > 0 ? (slots_small + slots_big / 2) / slots_big : 1;
+                    if (ps < 1) ps = 1;
+                    const uint32_t period = 1 + ps;
+                    const uint32_t rounds = slots_big < slots_small / ps ? slots_big : slots_small / ps;      // periods in which both classes have tiles
+                    if (sidx < rounds * period) {
+                        const uint32_t q = sidx / period, rr = sidx - q * period;
+                        big = rr == 0;
+                        idx = big ? q : q * ps + (rr - 1);
+                    } else {
+                        const uint32_t w = sidx - rounds * period, left_big = slots_big - rounds;
+                        big = w < left_big;
+                        idx = big ? rounds + w : rounds * ps + (w - left_big);
+                    }
+                }
+                // Tiles of a class are numbered expert by expert (expert e owns tiles_n numbers per row tile) and an XCD takes
+                // 32 consecutive numbers at a time, so the tiles it runs together belong to one expert, or to neighbours.
+                const uint32_t lin = ((idx / gemm::CHUNK) * 8 + xcd) * gemm::CHUNK + idx % gemm::CHUNK;
+                if (lin < (uint32_t)(big ? tot_big : tot_small) * tiles_n) {
+                    const int gmt = (int)(lin / tiles_n);
+                    // the expert that owns row tile gmt of the class: the first whose running count exceeds gmt
+                    const int *upto = big ? upto_big : upto_small;
+                    int e = 0;
+                    for (int span = kMixedMaxExperts / 2; span > 0; span >>= 1)
+                        if (upto[e + span - 1] <= gmt) e += span;
+                    if (e < E) {
+                        const int before = e > 0 ? upto[e - 1] : 0, cnt = upto[e] - before;
+                        int64_t row_begin;
+                        const int rows = gemm::expert_rows(m_offsets, e, M_total, row_begin);
+                        // Inside the expert: groups of 8 row tiles (the last may be short), in a group blocks of gn column
+                        // tiles with the row tile running fastest, gn such that a block is about 32 tiles: the 32 tiles an XCD
+                        // runs together share gm activation panels and gn weight panels of one expert (one row tile: its
+                        // activations and the whole weight matrix once).
+                        const uint32_t in_e = lin - (uint32_t)before * tiles_n, per_group = gemm::GROUP_M * tiles_n;
+                        const uint32_t grp = in_e / per_group, in_grp = in_e - grp * per_group;
+                        const uint32_t left = (uint32_t)cnt - grp * gemm::GROUP_M;
+                        const uint32_t gm = left < gemm::GROUP_M ? left : gemm::GROUP_M;
+                        const uint32_t gn = gemm::CHUNK / gm;
+                        const uint32_t per_nblock = gm * gn;
+                        const uint32_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
+                        const uint32_t local = grp * gemm::GROUP_M + in_blk % gm, tn = nblk * gn + in_blk / gm;
+                        entry.x = e | (big ? 1 << 30 : 0);
+                        entry.y = (int)(row_begin + (big ? (int64_t)local * 256 : (int64_t)(rows >> 8) * 256));     // M_total < 2^31
+                        entry.z = (int)(row_begin + rows);
+                        entry.w = (int)(tn * 256);
+                    }
+                }
+            }
+            table[t] = entry;
+        }
+        __syncthreads();
+        for (int i = 0; i < kTable; ++i) {
+            if (first + (uint64_t)i * gridDim.x >= all_slots) break;
+            const int4 entry = table[i];
+            const int ex = __builtin_amdgcn_readfirstlane(entry.x);
+            if (ex < 0) continue;
+            const int e = ex & 0xFFFF;
+            const int64_t m0 = __builtin_amdgcn_readfirstlane(entry.y), row_end = __builtin_amdgcn_readfirstlane(entry.z);
+            const int64_t n0 = __builtin_amdgcn_readfirstlane(entry.w);
+            const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
+            const uint8_t *bq_e = Bq + (int64_t)e * N * K;
+            __syncthreads();                            // every wave is done with the previous tile's use of the stage memory
+            if (ex >> 30)
+                tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
+            else
+                tile_asm<128, 256, 1, HWS, false, 3, false, true, 4>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
         }
     }
-    // Tiles of a class are numbered expert by expert (expert e owns tiles_n numbers per row tile) and an XCD takes 32
-    // consecutive numbers at a time, so the tiles it runs together belong to one expert, or to neighbours.
-    const uint32_t lin = ((idx / gemm::CHUNK) * 8 + xcd) * gemm::CHUNK + idx % gemm::CHUNK;
-    if (lin >= (uint32_t)(big ? tot_big : tot_small) * tiles_n) return;
-    const int gmt = (int)(lin / tiles_n);
-    // ---- the expert that owns row tile gmt of the class tells the others
-    {
-        const int cnt = big ? nb : ns, incl = big ? ib : is;
-        if (gmt >= incl - cnt && gmt < incl) { found_e = t; found_first = incl - cnt; found_begin = (int)begin; found_rows = rows; found_cnt = cnt; }
-    }
-    __syncthreads();
-    if (found_e < 0) return;
-    const int e = found_e;
-    const int64_t row_begin = found_begin, row_end = row_begin + found_rows, kblocks = K / KB;
-    const float *bs_e = (const float *)((const char *)Bs + (int64_t)e * (N / 128) * kblocks * (HWS ? 1 : 4));
-    const uint8_t *bq_e = Bq + (int64_t)e * N * K;
-    // Inside the expert: groups of 8 row tiles (the last may be short), in a group blocks of gn column tiles with the
-    // row tile running fastest, gn such that a block is about 32 tiles: the 32 tiles an XCD runs together share
-    // gm activation panels and gn weight panels of one expert (one row tile: its activations and the whole weight matrix once).
-    int64_t local, tn;
-    {
-        const uint32_t in_e = lin - (uint32_t)found_first * tiles_n, per_group = gemm::GROUP_M * tiles_n;
-        const uint32_t grp = in_e / per_group, in_grp = in_e - grp * per_group;
-        const uint32_t left = (uint32_t)found_cnt - grp * gemm::GROUP_M;
-        const uint32_t gm = left < gemm::GROUP_M ? left : gemm::GROUP_M;
-        const uint32_t gn = gemm::CHUNK / gm;
-        const uint32_t per_nblock = gm * gn;
-        const uint32_t nblk = in_grp / per_nblock, in_blk = in_grp - nblk * per_nblock;
-        local = grp * gemm::GROUP_M + in_blk % gm;
-        tn = nblk * gn + in_blk / gm;
-    }
-    if (big)
-        tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, bq_e, bs_e, row_begin + local * 256, row_end, tn * 256, N, K, C, N,
-                                                          out_dtype);
-    else
-        tile_asm<128, 256, 1, HWS, false, 3, false, true, 4>(smem, Aq, As, bq_e, bs_e, row_begin + (found_rows >> 8) * 256, row_end, tn * 256,
-                                                             N, K, C, N, out_dtype);
 }
 
 template <int SDT, int NB>
@@ -1128,6 +1174,20 @@ bool big_grouped_ok(const void *As, const void *Bs, int scale_dtype, int64_t M_t
            asm_shape_ok(As, Bs, M_total, N, K, scale_dtype);
 }
 
+// CUs of the current device (0 if it cannot be asked); asked once per device
+static int compute_units()
+{
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+        cached[dev] = n > 0 ? n : -1;
+    }
+    return cached[dev] > 0 ? cached[dev] : 0;
+}
+
 int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
                        const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype,
                        hipStream_t st)
@@ -1143,9 +1203,13 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
     if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 2048)) {
         // an expert with r rows has r / 256 tiles plus one when rows are left over, big or small: M_total / 256 + E row
         // tiles at most over both classes, each class rounded up to whole groups of 8 x 32 workgroups
-        const int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;
+        int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         if (E <= kMixedMaxExperts) {
+            // one workgroup per CU that works through every grid-th slot (a workgroup owns its CU: the tiles' LDS)
+            static const char *persist_env = getenv("LP_GEMM_GROUPED_PERSIST");  // tuning aid: 0 = one workgroup per slot
+            const int cus = (persist_env && atoi(persist_env) == 0) ? 0 : compute_units();
+            if (cus >= 8 && grid > cus) grid = cus / 8 * 8;
             static const char *order_env = getenv("LP_GEMM_GROUPED_ORDER");     // tuning aid: XCDs that take their small tiles first (0: classes dealt alternately)
             const int small_first = order_env ? atoi(order_env) : 4;
             if (scale_dtype == LP_E8M0)

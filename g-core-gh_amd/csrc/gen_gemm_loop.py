@@ -570,10 +570,10 @@ def generate():
             emit(f"s_add_u32 s{lo}, s42, s87")
             emit(f"s_addc_u32 s{lo + 1}, s43, 0")
     if HALFSPLIT:
-        emit("s_mov_b32 s87, %[lohalf]")
+        emit("s_bfe_u32 s87, %[flags], 0x10003")           # bit 3 of the wave flags: first half of the waves
     emit("s_mov_b32 s48, %[m0base]")
     emit("s_mov_b32 s49, %[trips]")
-    emit("s_mov_b32 s53, %[copies]")
+    emit("s_and_b32 s53, %[flags], 1")                    # wave flags (one operand): bit 0 = this wave copies scales,
     emit("s_mov_b32 s54, 0")
     emit("s_mov_b32 s55, 0")
     for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
@@ -629,10 +629,10 @@ def generate():
     global IDLE
     global GRP
     if WITH_IDLE:
-        emit("s_cmp_eq_u32 %[idle], 1")
+        emit("s_bitcmp1_b32 %[flags], 1")                  # bit 1 = none of its activation rows exist,
         emit("s_cbranch_scc1 Lloopi%=")
     if PINGPONG:
-        emit("s_cmp_eq_u32 %[grp], 1")
+        emit("s_bitcmp1_b32 %[flags], 2")                  # bit 2 = second half of the waves (bit 3: first half, flat tile)
         emit("s_cbranch_scc1 Lloopb%=")
     loop_body()
     if PINGPONG:
