@@ -1207,8 +1207,11 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped: problem too large");
         if (E <= kMixedMaxExperts) {
             // one workgroup per CU that works through every grid-th slot (a workgroup owns its CU: the tiles' LDS)
-            static const char *persist_env = getenv("LP_GEMM_GROUPED_PERSIST");  // tuning aid: 0 = one workgroup per slot
-            const int cus = (persist_env && atoi(persist_env) == 0) ? 0 : compute_units();
+            // (LP_GEMM_GROUPED_PERSIST, read at every call so that a test can change it: 0 = one workgroup per slot, n >= 8 =
+            // that many workgroups, e.g. few enough that each walks more slots than one table holds)
+            const char *persist_env = getenv("LP_GEMM_GROUPED_PERSIST");
+            const int forced = persist_env ? atoi(persist_env) : -1;
+            const int cus = forced == 0 ? 0 : (forced >= 8 ? forced : compute_units());
             if (cus >= 8 && grid > cus) grid = cus / 8 * 8;
             static const char *order_env = getenv("LP_GEMM_GROUPED_ORDER");     // tuning aid: XCDs that take their small tiles first (0: classes dealt alternately)
             const int small_first = order_env ? atoi(order_env) : 4;

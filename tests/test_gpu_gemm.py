@@ -214,6 +214,28 @@ def test_gemm_grouped_e8m0_scales(G, case):
     check(out, ref, f"grouped e8m0 {case[:3]}")
 
 
+def test_gemm_grouped_same_bits_however_the_slots_are_dealt(G, monkeypatch):
+    """The mixed-height grouped kernel lets one workgroup per CU walk its share of the tile slots, looking them up 256 at
+    a time.  With 8 workgroups each walks more than one table's worth (two look-up batches); with one workgroup per
+    slot nothing is walked.  All three launches must give the same bits, and the reference's result."""
+    E, N, K = 96, 2048, 2048
+    m_splits = [300 + (i * 37) % 500 if i % 11 else 0 for i in range(E)]
+    xq, xs, wq, ws = _grouped_problem(E, N, K, m_splits, seed=5)
+    M = sum(m_splits)
+    offs = torch.zeros(E + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+    args = (xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda())
+    say("gemm grouped, slot walk", E, N, K, "M=", M)
+    monkeypatch.delenv("LP_GEMM_GROUPED_PERSIST", raising=False)
+    out = G.grouped_gemm_fp8(*args)
+    ref = T.grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits)
+    check(out, ref, "grouped, one workgroup per CU")
+    for grid in ("8", "0"):
+        say("LP_GEMM_GROUPED_PERSIST =", grid)
+        monkeypatch.setenv("LP_GEMM_GROUPED_PERSIST", grid)
+        assert torch.equal(G.grouped_gemm_fp8(*args), out), grid
+
+
 @pytest.mark.parametrize("K", [512, 4096], ids=["128-row-tiles", "mixed-heights"])
 def test_gemm_grouped_survives_a_bad_offset_table(G, K):
     """Offsets that decrease or run past the rows are made harmless inside the kernels (both ends clamped to the row
