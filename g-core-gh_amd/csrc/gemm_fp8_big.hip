@@ -562,8 +562,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
                     *(u32x2 *)(stage + E::write_offset(mb, nb, l16, lq)) = o;
                 }
             }
-            if constexpr (DUAL) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave reads back only what it wrote
-            else __syncthreads();
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // a wave reads back only what it wrote: no barrier
             const int64_t row_base = m0 + wm * 64;
 #pragma unroll
             for (int p = 0; p < E::PASSES; ++p) {
