@@ -110,6 +110,27 @@ def test_every_tile_exactly_once(name, small_first, N):
         assert covered == r, (e, r, b, s)
 
 
+@pytest.mark.parametrize("workgroups", [8, 256, 304, 1 << 20])
+@pytest.mark.parametrize("all_slots", [0, 8 * 32, 8 * 32 * 47, 8 * 32 * 300])
+def test_slot_walk_of_the_persistent_launch(workgroups, all_slots):
+    """With fewer workgroups than slots, workgroup b takes slots b, b + G, b + 2 G ... (G = workgroups rounded down to a
+    multiple of 8, what the host launches), looked up 256 at a time, one slot per thread: every slot comes up exactly once,
+    and always on the XCD (slot mod 8) of the workgroup that takes it, which keeps the per-XCD order of the schedule."""
+    K_TABLE = 256
+    G = workgroups // 8 * 8 if all_slots > workgroups else max(all_slots, 8)
+    seen = []
+    for b in range(min(G, all_slots)):
+        first = b
+        while first < all_slots:                            # one look-up batch
+            for t in range(K_TABLE):
+                slot = first + t * G
+                if slot < all_slots:
+                    assert slot % 8 == b % 8
+                    seen.append(slot)
+            first += K_TABLE * G
+    assert sorted(seen) == list(range(all_slots))
+
+
 def test_an_xcd_runs_neighbouring_tiles_together():
     """32 consecutive positions of an XCD's sequence within a class are 32 consecutive tile numbers: at most two
     experts unless experts have fewer than 16 tiles, and for an expert with at least 8 row tiles a block of 8 x 4."""
