@@ -118,7 +118,15 @@ def audit(quiet: bool = False) -> int:
             print(f"FAIL {name}: the loop names registers that are neither early-clobber outputs nor clobbers: {' '.join(missing)}")
             bad += 1
     for kernel, body in blocks:
-        if len(body) < 100:                   # the loops are thousands of lines; small asm statements are not audited
+        if len(body) < 100:
+            # Small statements: the compiler inserts the wait states a lane-crossing read of a vector register needs after
+            # the instruction that writes it, but not across the border of an asm statement.  A statement whose first
+            # instruction is such a read must bring its own (s_nop in front): without it v_readfirstlane has returned the
+            # register's previous value whenever the scheduler put the producing v_mov right in front of the statement.
+            first = next((l.strip() for l in body if l.strip() and not l.strip().startswith(";")), "")
+            if re.match(r"v_(readfirstlane|readlane|permlane|writelane)", first) or " dpp" in first or "row_" in first:
+                print(f"FAIL {kernel}: an asm statement starts with a lane-crossing instruction without wait states: {first}")
+                bad += 1
             continue
         match = None
         for name, (patterns, literal) in templates.items():
