@@ -247,6 +247,18 @@ def main():
                                                   "reference_ms_on_its_hardware": 0.575}
         del a_nt, b_nt, c_nt
         torch.cuda.empty_cache()
+        # what the matrix cores hold with the loop's arithmetic and nothing else: the fp8 16x16x128 instruction on registers
+        # only, two waves per SIMD, with 0 / 4 / 8 fp32 FMAs after each (the fp32-scaled loops fold with four), on zeros and
+        # on random e4m3 operands -- the ceiling the GEMM figures above are to be read against (no LDS, no memory traffic)
+        rnd = (torch.randint(0, 256, (4096,), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8) & 0x77)
+        iters, wgs = 2000, 256
+        fl_p = 2.0 * 16 * 16 * 128 * 8 * iters * 8 * wgs
+        probe = {}
+        for tag, ptr in (("zero_operands", None), ("random_e4m3_operands", rnd.data_ptr())):
+            for k in (0, 4, 8):
+                ms_p, _ = time_launches([lambda k=k, ptr=ptr: chk(L.lp_probe_mfma(k, iters, ptr, wgs, stream()))], 6, 2)
+                probe[f"{tag}_{k}_fmas_per_instruction"] = {"ms": ms_p, "tflops": fl_p / ms_p / 1e9, "mfma_frac": fl_p / ms_p / 1e9 / FP8_PEAK_TFLOPS}
+        extras["matrix_pipe_probe_registers_only"] = probe
 
     if want("copy"):
         # -------------------------------------------------------------- calibration: a plain device copy of known size

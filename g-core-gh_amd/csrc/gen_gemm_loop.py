@@ -673,14 +673,34 @@ def main():
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
         configure(*cfg)
         generate()
-        text = "// Generated by gen_gemm_loop.py -- do not edit.\n" + "".join('"' + ln + '\\n"\n' for ln in lines)
-        path = os.path.join(here, name)
-        # only files whose content differs are rewritten (their time stamps drive the rebuild), so running the
-        # generator on every build also undoes a hand edit to any of its outputs
-        if not os.path.exists(path) or open(path).read() != text:
-            with open(path, "w") as f:
-                f.write(text)
-            print("regenerated", name)
+        write(here, name)
+    probe_bodies(here)
+
+
+def probe_bodies(here):
+    """Bodies of the matrix-pipe probe (selftest.hip: probe_mfma): eight matrix instructions into eight result buffers
+    v[32:63], each followed by k FMAs that fold a buffer finished four instructions ago into v[64:127] -- the arithmetic
+    of the fp32-scaled loops with no operand movement at all."""
+    global lines
+    for k in (0, 2, 4, 6, 8):
+        lines = []
+        for j in range(8):
+            lines.append(f"v_mfma_f32_16x16x128_f8f6f4 v[{32 + 4 * j}:{35 + 4 * j}], v[0:7], v[8:15], 0")
+            src = (j + 4) % 8
+            for f in range(k):
+                lines.append(f"v_fmac_f32 v{64 + (j * 8 + f) % 64}, v{32 + 4 * src + f % 4}, v20")
+        write(here, f"probe_mfma_body{k}.inc")
+
+
+def write(here, name):
+    text = "// Generated by gen_gemm_loop.py -- do not edit.\n" + "".join('"' + ln + '\\n"\n' for ln in lines)
+    path = os.path.join(here, name)
+    # only files whose content differs are rewritten (their time stamps drive the rebuild), so running the
+    # generator on every build also undoes a hand edit to any of its outputs
+    if not os.path.exists(path) or open(path).read() != text:
+        with open(path, "w") as f:
+            f.write(text)
+        print("regenerated", name)
 
 
 if __name__ == "__main__":

@@ -124,7 +124,69 @@ __global__ __launch_bounds__(256) void stream_probe(const u32x4 *__restrict__ sr
     }
 }
 
+// Matrix-pipe probe: the fp8 16x16x128 matrix instruction in a register-only loop, FMAS fp32 FMAs after each (0, 2, 4, 6
+// or 8: the fp32-scaled GEMM loops fold with four), eight waves per workgroup = two per SIMD, no LDS and no memory traffic
+// inside the loop.  The operand registers v[0:15] hold 64 bytes per lane from `operands` (e4m3 codes), or zeros.  What it
+// takes is what the chip's clock under that arithmetic allows: the ceiling of any kernel built from these instructions.
+#define LP_PROBE_CLOBBERS                                                                                                       \
+    "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v20", "v32", "v33", "v34", "v35",   \
+        "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54",   \
+        "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73",   \
+        "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92",   \
+        "v93", "v94", "v95", "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109",      \
+        "v110", "v111", "v112", "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",     \
+        "v126", "v127"
+template <int FMAS>
+__global__ __launch_bounds__(512) void probe_mfma(const uint8_t *__restrict__ operands, int iters)
+{
+    const uint8_t *p = operands + (size_t)(threadIdx.x & 63) * 64;
+    if (operands != nullptr)
+        asm volatile("global_load_dwordx4 v[0:3], %0, off\n\tglobal_load_dwordx4 v[4:7], %0, off offset:16\n\t"
+                     "global_load_dwordx4 v[8:11], %0, off offset:32\n\tglobal_load_dwordx4 v[12:15], %0, off offset:48\n\t"
+                     "s_waitcnt vmcnt(0)\n\tv_mov_b32 v20, 0x3f8ccccd" ::"v"(p) : "memory", LP_PROBE_CLOBBERS);
+    else
+        asm volatile("v_mov_b32 v0, 0\n\tv_mov_b32 v1, 0\n\tv_mov_b32 v2, 0\n\tv_mov_b32 v3, 0\n\tv_mov_b32 v4, 0\n\tv_mov_b32 v5, 0\n\t"
+                     "v_mov_b32 v6, 0\n\tv_mov_b32 v7, 0\n\tv_mov_b32 v8, 0\n\tv_mov_b32 v9, 0\n\tv_mov_b32 v10, 0\n\tv_mov_b32 v11, 0\n\t"
+                     "v_mov_b32 v12, 0\n\tv_mov_b32 v13, 0\n\tv_mov_b32 v14, 0\n\tv_mov_b32 v15, 0\n\tv_mov_b32 v20, 0" ::: LP_PROBE_CLOBBERS);
+    for (int i = 0; i < iters; ++i) {
+        if constexpr (FMAS == 0) asm volatile(
+#include "probe_mfma_body0.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else if constexpr (FMAS == 2) asm volatile(
+#include "probe_mfma_body2.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else if constexpr (FMAS == 4) asm volatile(
+#include "probe_mfma_body4.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else if constexpr (FMAS == 6) asm volatile(
+#include "probe_mfma_body6.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else asm volatile(
+#include "probe_mfma_body8.inc"
+            ::: LP_PROBE_CLOBBERS);
+    }
+}
+
 }  // namespace
+
+extern "C" int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream)
+{
+    LP_REQUIRE(fmas_per_instruction == 0 || fmas_per_instruction == 2 || fmas_per_instruction == 4 || fmas_per_instruction == 6 ||
+                   fmas_per_instruction == 8, "lp_probe_mfma: 0, 2, 4, 6 or 8 FMAs per matrix instruction");
+    LP_REQUIRE(iters >= 1 && iters <= (1 << 24), "lp_probe_mfma: 1 .. 2^24 iterations");
+    LP_REQUIRE(workgroups >= 1 && workgroups <= (1 << 20), "lp_probe_mfma: 1 .. 2^20 workgroups");
+    LP_REQUIRE((uintptr_t)operands % 16 == 0, "lp_probe_mfma: operands must be 16-byte aligned (4096 bytes, or NULL)");
+    hipStream_t st = (hipStream_t)stream;
+    const uint8_t *ops = (const uint8_t *)operands;
+    switch (fmas_per_instruction) {
+    case 0: hipLaunchKernelGGL(probe_mfma<0>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case 2: hipLaunchKernelGGL(probe_mfma<2>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case 4: hipLaunchKernelGGL(probe_mfma<4>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case 6: hipLaunchKernelGGL(probe_mfma<6>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    default: hipLaunchKernelGGL(probe_mfma<8>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    }
+    return check_launch("lp_probe_mfma");
+}
 
 extern "C" int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t write_bytes, int workgroups, lp_stream_t stream)
 {

@@ -329,6 +329,16 @@ int lp_selftest(int which, uint64_t *mismatches, lp_stream_t stream);
  */
 int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t write_bytes, int workgroups, lp_stream_t stream);
 
+/*
+ * Measurement aid: one launch of `workgroups` x 512 threads (two waves per SIMD) that issues, `iters` times, eight fp8
+ * 16x16x128 matrix instructions each followed by fmas_per_instruction (0, 2, 4, 6, 8) fp32 FMAs, on registers only: no
+ * LDS, no memory traffic in the loop.  operands: 4096 bytes of e4m3 codes (64 per lane) for the matrix operands, or NULL
+ * for zeros.  Flops = workgroups x 8 waves x iters x 8 x 2 x 16 x 16 x 128.  It shows the rate the matrix cores hold
+ * with the arithmetic of an fp32-scaled GEMM loop (four FMAs per instruction) and nothing else: the ceiling the GEMM
+ * kernels' fraction of peak is to be read against.  No reference counterpart.
+ */
+int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream);
+
 /* Bulk element-wise casts through the library's device code paths (debug aid
  * for tests): kind 0 = fp32 -> e4m3fn software, 1 = fp32 -> e4m3fn hardware
  * (inputs clamped to +-448 first), 2 = fp32 -> e8m0, 3 = fp32 -> bf16. */

@@ -62,3 +62,25 @@ def test_zero_rows_gemm_and_grouped_linear():
     assert tuple(y.shape) == (0, 256)
     y.sum().backward()
     assert tuple(x.grad.shape) == (0, 512) and tuple(w.grad.shape) == (3, 256, 512) and not w.grad.any()
+
+
+def test_measurement_probes_launch_and_reject_bad_arguments():
+    """The two measurement aids of the library (bare stream, register-only matrix-pipe loop) are what the benchmark's
+    floor figures come from: they must launch for every variant the benchmark uses and refuse what they do not implement."""
+    from gcore_lowp import _abi as A
+    L = A.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    src = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(1 << 19, dtype=torch.uint8, device="cuda")
+    say("probes: stream")
+    A.check(L.lp_probe_stream(src.data_ptr(), src.numel(), dst.data_ptr(), dst.numel(), 64, st))
+    A.check(L.lp_probe_stream(None, 0, None, 0, 8, st))
+    ops = (torch.arange(4096, device="cuda") % 120).to(torch.uint8)
+    for k in (0, 2, 4, 6, 8):
+        say("probes: matrix pipe, FMAs per instruction", k)
+        A.check(L.lp_probe_mfma(k, 10, ops.data_ptr(), 16, st))
+        A.check(L.lp_probe_mfma(k, 10, None, 16, st))
+    torch.cuda.synchronize()
+    assert L.lp_probe_mfma(3, 10, None, 16, st) != 0
+    assert L.lp_probe_mfma(4, 0, None, 16, st) != 0
+    assert L.lp_probe_stream(src.data_ptr(), 15, dst.data_ptr(), 16, 8, st) != 0
