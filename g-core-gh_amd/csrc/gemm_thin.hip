@@ -180,8 +180,8 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
         uint8_t *dst = wring + (j % SLOTS) * 4096;
         const int64_t off = (int64_t)kb * 128;
-        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + off), LDS_PTR(dst), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + off), LDS_PTR(dst + 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + off), LDS_PTR(dst), 16, 0, 2);                   // weights: streaming hint
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + off), LDS_PTR(dst + 1024), 16, 0, 2);
         __builtin_amdgcn_global_load_lds(GLB_PTR(asrc0 + off), LDS_PTR(dst + 2048), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(GLB_PTR(asrc1 + off), LDS_PTR(dst + 3072), 16, 0, 0);
     };
@@ -321,8 +321,10 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
     auto request_b = [&](int j) {
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
         uint8_t *dst = wb + (j % BS) * 2048;
-        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + (int64_t)kb * 128), LDS_PTR(dst), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + (int64_t)kb * 128), LDS_PTR(dst + 1024), 16, 0, 0);
+        // the weights are read once by the whole launch: with the streaming hint (last argument) they pass the L2 without
+        // pushing out the activations every workgroup reads (13.2 -> 13.0 us on M = 64, N = 4096, K = 7168)
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + (int64_t)kb * 128), LDS_PTR(dst), 16, 0, 2);
+        __builtin_amdgcn_global_load_lds(GLB_PTR(bsrc + 8 * K + (int64_t)kb * 128), LDS_PTR(dst + 1024), 16, 0, 2);
     };
     auto request_a = [&](int u) {                        // unit u: rows 32 (u % U) .. + 31 of block u / U
         const int j = u / U, v = u % U;
