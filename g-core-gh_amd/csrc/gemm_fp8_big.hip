@@ -254,6 +254,20 @@ struct StagedEpilogue {
     __host__ __device__ static constexpr int read_offset(int row, int chunk) { return row * PITCH + chunk * 16; }
 };
 
+// The same for e4m3 results (one byte per element; the unscaled NT GEMM's fp8 output): a row of the staging region holds
+// COLS bytes plus 16 of padding, a lane writes its 4 bytes of block (mb, nb), and 16-byte chunks of 16 columns are read back.
+template <int COLS>
+struct StagedEpilogueFp8 {
+    static constexpr int PITCH = COLS + 16;
+    static constexpr int WAVE_BYTES = 64 * PITCH;
+    static constexpr int CHUNKS = COLS / 16;
+    static constexpr int PASSES = CHUNKS;
+    __host__ __device__ static constexpr int write_offset(int mb, int nb, int l16, int lq) { return (mb * 16 + l16) * PITCH + nb * 16 + 4 * lq; }
+    __host__ __device__ static constexpr int read_row(int pass, int lane) { return (pass * 64 + lane) / CHUNKS; }
+    __host__ __device__ static constexpr int read_chunk(int pass, int lane) { return (pass * 64 + lane) % CHUNKS; }
+    __host__ __device__ static constexpr int read_offset(int row, int chunk) { return row * PITCH + chunk * 16; }
+};
+
 // WN: waves side by side along N (2, or 4 for the flat 128 x 256 tile); a wave owns 64 rows x TN / WN columns.
 template <int TM, int TN, int KSUB, int NST = 2, int WN = 2>
 struct AsmTile {
@@ -578,6 +592,37 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
                 }
             }
             return;
+        }
+        if constexpr (!DUAL && (TN / WN) % 16 == 0) {
+            if (out_dtype == LP_E4M3 && N % 16 == 0 && ldc % 16 == 0 && (uintptr_t)C % 16 == 0) {
+                // e4m3fn results (the unscaled NT GEMM routed here) the same way: 4-byte stores per lane cost the 4096^3
+                // problem a tenth of its time
+                using E8 = StagedEpilogueFp8<TN / WN>;
+                static_assert(WAVES * E8::WAVE_BYTES <= T::LDS_BYTES, "the waves' staging regions must fit the tile's LDS");
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __syncthreads();
+                uint8_t *stage = smem + wave * E8::WAVE_BYTES;
+                auto sat = [](float x) { const float c = __builtin_fminf(__builtin_fmaxf(x, -kE4M3Max), kE4M3Max); return x != x ? x : c; };
+#pragma unroll
+                for (int mb = 0; mb < 4; ++mb) {
+#pragma unroll
+                    for (int nb = 0; nb < NBW; ++nb)
+                        *(uint32_t *)(stage + E8::write_offset(mb, nb, l16, lq)) =
+                            cvt4(sat(accs[nb][mb * 4]), sat(accs[nb][mb * 4 + 1]), sat(accs[nb][mb * 4 + 2]), sat(accs[nb][mb * 4 + 3]));
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                const int64_t row_base = m0 + wm * 64;
+#pragma unroll
+                for (int p = 0; p < E8::PASSES; ++p) {
+                    const int row = E8::read_row(p, lane), chunk = E8::read_chunk(p, lane);
+                    const int64_t n = wcol0 + chunk * 16;
+                    if (row_base + row < M && n < N) {
+                        const u32x4 v = *(const u32x4 *)(stage + E8::read_offset(row, chunk));
+                        __builtin_nontemporal_store(v, (u32x4 *)((uint8_t *)C + (row_base + row) * ldc + n));
+                    }
+                }
+                return;
+            }
         }
     }
 #pragma unroll

@@ -54,3 +54,32 @@ def test_staged_epilogue_bank_spread():
                     for b in ((off // 4) % 64, (off // 4 + 1) % 64):
                         hits[b] = hits.get(b, 0) + 1
             assert max(hits.values()) <= 2, (cols, nb, max(hits.values()))
+
+
+@pytest.mark.parametrize(("cols", "waves", "lds_bytes"), [(128, 8, 8 * 64 * (128 * 2 + 16)), (64, 4, 2 * (128 + 128) * 128 + 2 * 128 * 16)])
+def test_staged_fp8_epilogue_mapping(cols, waves, lds_bytes):
+    """The e4m3 form (StagedEpilogueFp8: one byte per element, 4 bytes written per lane and block, 16-byte chunks of 16
+    columns read back): every byte of the 64-row wave tile exactly once, aligned, inside the region."""
+    pitch, chunks = cols + 16, cols // 16
+    wave_bytes = 64 * pitch
+    assert waves * wave_bytes <= lds_bytes
+    region = [None] * wave_bytes
+    for mb in range(4):
+        for nb in range(cols // 16):
+            for l16 in range(16):
+                for lq in range(4):
+                    off = (mb * 16 + l16) * pitch + nb * 16 + 4 * lq
+                    assert off % 4 == 0 and off + 4 <= wave_bytes
+                    for r in range(4):
+                        assert region[off + r] is None
+                        region[off + r] = (mb * 16 + l16, nb * 16 + 4 * lq + r)
+    seen = set()
+    for p in range(chunks):
+        for lane in range(64):
+            row, chunk = (p * 64 + lane) // chunks, (p * 64 + lane) % chunks
+            off = row * pitch + chunk * 16
+            assert off % 16 == 0 and off + 16 <= wave_bytes and 0 <= row < 64
+            for j in range(16):
+                assert region[off + j] == (row, chunk * 16 + j)
+                seen.add((row, chunk * 16 + j))
+    assert len(seen) == 64 * cols
