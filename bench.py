@@ -42,7 +42,7 @@ FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
 # requests of LDS-direct and non-temporal loads at 64) plus WRITE_SIZE.  Counters cannot be read from inside this process:
 # the figures are those of rocprofv3 --pmc runs of this script (profiles/gemm_kernels_mfma_lds_hbm_counters.txt), not of this run.
 GEMM_BIG_TRAFFIC_BYTES = 430.0e6     # gemm_asm<256,256,1> on 16384 weight rows: 362.9 MB read + 67.1 MB written
-GEMM_WIDE_TRAFFIC_BYTES = 457.9e6    # gemm_asm_wide<false> on the whole problem: 379.8 MB read + 78.1 MB written
+GEMM_WIDE_TRAFFIC_BYTES = 461.2e6    # gemm_asm_wide<false> on the whole problem: 376.5 MB read + 84.7 MB written
 
 
 def main():
