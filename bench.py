@@ -259,6 +259,24 @@ def main():
                 ms_p, _ = time_launches([lambda k=k, ptr=ptr: chk(L.lp_probe_mfma(k, iters, ptr, wgs, stream()))], 6, 2)
                 probe[f"{tag}_{k}_fmas_per_instruction"] = {"ms": ms_p, "tflops": fl_p / ms_p / 1e9, "mfma_frac": fl_p / ms_p / 1e9 / FP8_PEAK_TFLOPS}
         extras["matrix_pipe_probe_registers_only"] = probe
+        # what a CU's copy path out of the L2 delivers in the loops' request shape (1 KB per wave and request, rows 7168 bytes
+        # apart, one step in flight behind a wait and a barrier; 2 MB per region, L2-resident): into LDS with one 8-wave
+        # workgroup or two 4-wave workgroups per CU, and into registers.  A 128 x 128 tile needs 32 KB per 16 matrix
+        # instructions of a SIMD (512 cycles), a 256 x 256 tile 64 KB per 64 (2048 cycles).
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        rows_src = torch.zeros(4 * 512 * 7168, dtype=torch.uint8, device=dev)
+        sink = torch.zeros(2048, dtype=torch.uint8, device=dev)
+        cp = {}
+        steps_c = 2048
+        for tag, to_lds, waves, per_cu in (("to_lds_8_waves_1_wg_per_cu", 1, 8, 1), ("to_lds_4_waves_2_wg_per_cu", 1, 4, 2),
+                                           ("to_registers_8_waves_1_wg_per_cu", 0, 8, 1)):
+            wg = cus * per_cu
+            ms_c, _ = time_launches([lambda to_lds=to_lds, waves=waves, wg=wg: chk(L.lp_probe_copy(
+                to_lds, waves, steps_c, rows_src.data_ptr(), rows_src.numel(), 7168, sink.data_ptr(), wg, stream()))], 6, 2)
+            by = float(wg) * waves * steps_c * 8192
+            cp[tag] = {"ms": ms_c, "TB/s": by / ms_c / 1e9, "bytes_per_ns_per_cu": by / ms_c / 1e6 / cus}
+        extras["l2_to_cu_copy_probe"] = cp
+        del rows_src, sink
 
     if want("copy"):
         # -------------------------------------------------------------- calibration: a plain device copy of known size

@@ -167,7 +167,61 @@ __global__ __launch_bounds__(512) void probe_mfma(const uint8_t *__restrict__ op
     }
 }
 
+#define LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
+#define GLB_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
+
+// What a CU's copy path out of the L2 delivers, in the shape the GEMM loops use it: every wave issues eight 1 KB requests
+// per step (8 rows x 128 bytes each, rows row_stride apart, 16 bytes per lane), two steps' worth of LDS, one step kept in
+// flight behind a wait and a workgroup barrier.  The source is four regions of 512 rows; the workgroups of an XCD read the
+// same region and every step moves on by 128 bytes inside the rows (eight windows, then again), so after the first pass
+// everything is served by the L2.  TO_LDS: global_load_lds (no registers); otherwise 16-byte loads into registers.
+template <int WAVES, bool TO_LDS>
+__global__ __launch_bounds__(WAVES * 64) void probe_copy(const uint8_t *__restrict__ src, int steps, int64_t row_stride, uint32_t *sink)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[2 * WAVES * 8 * 1024];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint8_t *base = src + (int64_t)((blockIdx.x >> 3) & 3) * 512 * row_stride;
+    const int row = lane >> 3, chunk = lane & 7;
+    u32x4 acc = {0, 0, 0, 0};
+    for (int s = 0; s < steps; ++s) {
+        const int64_t win = (int64_t)(s & 7) * 128;
+        uint8_t *stage = lds + (s & 1) * (WAVES * 8 * 1024);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = 8 * (wave + WAVES * i) + row;                     // < 512
+            const uint8_t *g = base + (int64_t)r * row_stride + win + chunk * 16;
+            if constexpr (TO_LDS) __builtin_amdgcn_global_load_lds(GLB_PTR(g), LDS_PTR(stage + (wave + WAVES * i) * 1024), 16, 0, 0);
+            else { const u32x4 v = *(const u32x4 *)g; acc += v; }
+        }
+        if constexpr (TO_LDS) {
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (!TO_LDS && acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[t] = acc.z + acc.w;      // keeps the loads alive
+}
+
 }  // namespace
+
+extern "C" int lp_probe_copy(int to_lds, int waves, int steps, const void *src, int64_t src_bytes, int64_t row_stride, void *sink,
+                             int workgroups, lp_stream_t stream)
+{
+    LP_REQUIRE(waves == 4 || waves == 8, "lp_probe_copy: 4 or 8 waves per workgroup");
+    LP_REQUIRE(steps >= 1 && steps <= (1 << 24), "lp_probe_copy: 1 .. 2^24 steps");
+    LP_REQUIRE(workgroups >= 1 && workgroups <= (1 << 20), "lp_probe_copy: 1 .. 2^20 workgroups");
+    LP_REQUIRE(row_stride >= 1024 && row_stride % 16 == 0, "lp_probe_copy: row_stride must be a multiple of 16, at least 1024");
+    LP_REQUIRE(src && sink && (uintptr_t)src % 16 == 0, "lp_probe_copy: src (16-byte aligned) and sink (2048 bytes) must be given");
+    LP_REQUIRE(src_bytes >= 4 * 512 * row_stride, "lp_probe_copy: src must hold 4 x 512 rows of row_stride bytes");
+    hipStream_t st = (hipStream_t)stream;
+    const uint8_t *p = (const uint8_t *)src;
+    uint32_t *sk = (uint32_t *)sink;
+    if (waves == 8 && to_lds) hipLaunchKernelGGL((probe_copy<8, true>), dim3((unsigned)workgroups), dim3(512), 0, st, p, steps, row_stride, sk);
+    else if (waves == 8) hipLaunchKernelGGL((probe_copy<8, false>), dim3((unsigned)workgroups), dim3(512), 0, st, p, steps, row_stride, sk);
+    else if (to_lds) hipLaunchKernelGGL((probe_copy<4, true>), dim3((unsigned)workgroups), dim3(256), 0, st, p, steps, row_stride, sk);
+    else hipLaunchKernelGGL((probe_copy<4, false>), dim3((unsigned)workgroups), dim3(256), 0, st, p, steps, row_stride, sk);
+    return check_launch("lp_probe_copy");
+}
 
 extern "C" int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream)
 {

@@ -339,6 +339,20 @@ int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t writ
  */
 int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream);
 
+/*
+ * Measurement aid: what a CU's copy path out of the L2 delivers in the shape the GEMM loops use it.  One launch of
+ * `workgroups` x 64 * waves threads (waves = 4: 64 KB of LDS per workgroup, two fit a CU; 8: 128 KB, one per CU); every
+ * wave issues, `steps` times, eight requests of 1 KB (8 rows x 128 bytes, rows row_stride bytes apart, 16 bytes per lane)
+ * and keeps one step in flight behind a wait and a workgroup barrier, as a two-stage K loop does.  to_lds != 0: straight
+ * into LDS (global_load_lds, what the loops use); 0: into registers.  src: 4 regions of 512 rows x row_stride bytes
+ * (src_bytes says how much is there), read over and over, so it is served by the L2 after the first pass; sink: 2048
+ * bytes that are never written in practice.  Bytes moved = workgroups x waves x steps x 8192.  It shows the ceiling of
+ * the operand copies: a 128 x 128 tile asks for 32 KB per 16 matrix instructions of each SIMD, a 256 x 256 tile for 64 KB
+ * per 64.  No reference counterpart.
+ */
+int lp_probe_copy(int to_lds, int waves, int steps, const void *src, int64_t src_bytes, int64_t row_stride, void *sink,
+                  int workgroups, lp_stream_t stream);
+
 /* Bulk element-wise casts through the library's device code paths (debug aid
  * for tests): kind 0 = fp32 -> e4m3fn software, 1 = fp32 -> e4m3fn hardware
  * (inputs clamped to +-448 first), 2 = fp32 -> e8m0, 3 = fp32 -> bf16. */

@@ -65,7 +65,7 @@ def test_zero_rows_gemm_and_grouped_linear():
 
 
 def test_measurement_probes_launch_and_reject_bad_arguments():
-    """The two measurement aids of the library (bare stream, register-only matrix-pipe loop) are what the benchmark's
+    """The measurement aids of the library (bare stream, register-only matrix-pipe loop, L2-to-LDS copy loop) are what the benchmark's
     floor figures come from: they must launch for every variant the benchmark uses and refuse what they do not implement."""
     from gcore_lowp import _abi as A
     L = A.lib()
@@ -80,6 +80,20 @@ def test_measurement_probes_launch_and_reject_bad_arguments():
         say("probes: matrix pipe, FMAs per instruction", k)
         A.check(L.lp_probe_mfma(k, 10, ops.data_ptr(), 16, st))
         A.check(L.lp_probe_mfma(k, 10, None, 16, st))
+    # the copy probe: every variant at the smallest and at the GEMM's row stride; the source is exactly as large as it asks for
+    sink = torch.zeros(2048, dtype=torch.uint8, device="cuda")
+    for stride in (1024, 7168):
+        rows = torch.zeros(4 * 512 * stride, dtype=torch.uint8, device="cuda")
+        for to_lds in (1, 0):
+            for waves in (4, 8):
+                say("probes: copy", stride, to_lds, waves)
+                A.check(L.lp_probe_copy(to_lds, waves, 9, rows.data_ptr(), rows.numel(), stride, sink.data_ptr(), 24, st))
+        torch.cuda.synchronize()
+        assert L.lp_probe_copy(1, 8, 9, rows.data_ptr(), rows.numel() - 16, stride, sink.data_ptr(), 24, st) != 0      # source too small
+    assert not sink.any()
+    assert L.lp_probe_copy(1, 6, 9, rows.data_ptr(), rows.numel(), 7168, sink.data_ptr(), 24, st) != 0
+    assert L.lp_probe_copy(1, 8, 9, rows.data_ptr(), rows.numel(), 512, sink.data_ptr(), 24, st) != 0
+    assert L.lp_probe_copy(1, 8, 9, None, 0, 1024, sink.data_ptr(), 24, st) != 0
     torch.cuda.synchronize()
     assert L.lp_probe_mfma(3, 10, None, 16, st) != 0
     assert L.lp_probe_mfma(4, 0, None, 16, st) != 0
