@@ -56,7 +56,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
     # weight copies by wave (s87 = 1 for the first half of the waves) instead of by copy index.
-    HALFSPLIT = early and tn // waves_n == 64
+    HALFSPLIT = early and tn // waves_n == 64 and waves_m * waves_n == 8
     # wide: a wave owns 64 x 144 columns (nine 16-column blocks), e.g. the 256 x 288 tile that cuts 18432 weight rows
     # into exactly 64 tile columns.  144 columns always straddle two weight-scale blocks, at a 16-column boundary known
     # only at run time (s74 = first block that takes the second scale row): the folds read one set of scale products,
@@ -82,7 +82,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # next; the other weight rows follow at the end of the step as before.  Every request then has about one and a
     # half steps to land instead of one (the loop spends its waiting time at the end-of-step wait for the copies).
     EARLY = early
-    assert not early or (nstage in (2, 3) and ksub == 1 and not brow)
+    assert not early or (nstage in (2, 3) and ksub == 1)
     # Three stages (with the early hand-back): the stage a step uses no longer follows from its place in the trip of four,
     # so the stage offsets live in registers.  s89 / s90 = LDS offset of the stage in use (activations / weights), s91 / s92
     # = of the stage just finished (what the end-of-step copies overwrite); the fragment read addresses v30 .. v33 are the
@@ -670,7 +670,7 @@ def main():
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
                       ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
-                      ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True))):
+                      ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True, True))):
         configure(*cfg)
         generate()
         write(here, name)
