@@ -662,9 +662,9 @@ PP = os.environ.get("LP_GEN_PINGPONG", "1") == "1"
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
     for name, cfg in (("gemm_big_loop.inc", (256, 256, 4, 2, 1, False, 2, False, True, False, True, PP)), ("gemm_big192_loop.inc", (256, 192, 4, 2, 1)),
-                      ("gemm_mid_loop.inc", (128, 128, 2, 2, 1)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
+                      ("gemm_mid_loop.inc", (128, 128, 2, 2, 1, False, 2, False, True)), ("gemm_mid2_loop.inc", (128, 128, 2, 2, 2)),
                       ("gemm_big_hw_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True, PP)),
-                      ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True)),
+                      ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True, 2, False, True)),
                       ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True, True, PP)),
                       ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True, True, PP)),
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
