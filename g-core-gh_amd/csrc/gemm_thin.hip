@@ -266,7 +266,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
 // Plan of the requests of one wave, in issue order, so that every wait can name how many younger requests may
 // still be in flight: weight blocks 0 .. BS-1 (2 requests each), activation units 0 and 1 (4 each); then at
 // step u, after the reads, unit u + 2 and, on the first unit of a block j, weight block j + BS.
-template <int PER, int U, int BS>
+template <int PER, int U, int BS, int AD>
 struct RingPlan {
     int a_end[PER * U];          // requests issued up to and including activation unit u
     int b_end[PER];              // ... weight block j
@@ -275,27 +275,27 @@ struct RingPlan {
     {
         int n = 0;
         for (int j = 0; j < (BS < PER ? BS : PER); ++j) { n += 2; b_end[j] = n; }
-        for (int u = 0; u < (2 < PER * U ? 2 : PER * U); ++u) { n += 4; a_end[u] = n; }
+        for (int u = 0; u < (AD < PER * U ? AD : PER * U); ++u) { n += 4; a_end[u] = n; }
         for (int u = 0; u < PER * U; ++u) {
             before[u] = n;
-            if (u + 2 < PER * U) { n += 4; a_end[u + 2] = n; }
+            if (u + AD < PER * U) { n += 4; a_end[u + AD] = n; }
             if (u % U == 0 && u / U + BS < PER) { n += 2; b_end[u / U + BS] = n; }
         }
     }
 };
 
-template <int SDT, int PER, int MB>
+template <int SDT, int PER, int MB, int BS = 4, int AD = 2>
 __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                                    const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                                    int M, int64_t N, int64_t K, void *__restrict__ C,
                                                                    int out_dtype)
 {
-    constexpr int U = (MB + 1) / 2, BS = 4, UNITS = PER * U;
-    constexpr int B0 = BS < PER ? BS : PER, A0 = 2 < UNITS ? 2 : UNITS;
+    constexpr int U = (MB + 1) / 2, UNITS = PER * U;
+    constexpr int B0 = BS < PER ? BS : PER, A0 = AD < UNITS ? AD : UNITS;
     constexpr int SV = (16 * MB * kThinWaves * kThinRun + 64 * kThinWaves - 1) / (64 * kThinWaves);      // table entries per lane
-    constexpr RingPlan<PER, U, BS> plan{};
+    constexpr RingPlan<PER, U, BS, AD> plan{};
     __shared__ __attribute__((aligned(1024))) uint8_t bring[kThinWaves * BS * 2048];
-    __shared__ __attribute__((aligned(1024))) uint8_t aring[kThinWaves * 2 * 4096];      // later: the waves' partial sums
+    __shared__ __attribute__((aligned(1024))) uint8_t aring[kThinWaves * AD * 4096];     // later: the waves' partial sums
     __shared__ float sSa[SV * 64 * kThinWaves];          // activation scales, [row][K block] as in memory
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 
     const int ld_row = lane >> 3, chunk = (lane & 7) ^ ld_row;
     const uint8_t *bsrc = Bq + (n0 + ld_row) * K + chunk * 16;
-    uint8_t *wb = bring + wave * (BS * 2048), *wa = aring + wave * (2 * 4096);
+    uint8_t *wb = bring + wave * (BS * 2048), *wa = aring + wave * (AD * 4096);
     auto request_b = [&](int j) {
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
         uint8_t *dst = wb + (j % BS) * 2048;
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
     auto request_a = [&](int u) {                        // unit u: rows 32 (u % U) .. + 31 of block u / U
         const int j = u / U, v = u % U;
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
-        uint8_t *dst = wa + (u % 2) * 4096;
+        uint8_t *dst = wa + (u % AD) * 4096;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = 32 * v + 8 * i + ld_row;
@@ -388,12 +388,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
         constexpr int need = (v == 0 && plan.b_end[j] > plan.a_end[u]) ? plan.b_end[j] : plan.a_end[u];
         wait_requests<plan.before[u] - need>();
         constexpr bool two = 2 * v + 1 < MB;             // the unit holds a second row group
-        const uint32_t ao = wa0 + (u % 2) * 4096;
+        const uint32_t ao = wa0 + (u % AD) * 4096;
         u32x4 x0 = lds_read16(ao + rdo0), x1 = lds_read16(ao + rdo1), y0 = x0, y1 = x1;
         if constexpr (two) { y0 = lds_read16(ao + 2048 + rdo0); y1 = lds_read16(ao + 2048 + rdo1); }
         if constexpr (v == 0) { w0 = lds_read16(wb0 + (j % BS) * 2048 + rdo0); w1 = lds_read16(wb0 + (j % BS) * 2048 + rdo1); }
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x0), "+v"(x1), "+v"(y0), "+v"(y1), "+v"(w0), "+v"(w1)::"memory");
-        if constexpr (u + 2 < UNITS) request_a(u + 2);
+        if constexpr (u + AD < UNITS) request_a(u + AD);
         if constexpr (v == 0 && j + BS < PER) request_b(j + BS);
         const i32x8 wf = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
         {
@@ -418,16 +418,16 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
     unrolled(step, std::make_integer_sequence<int, UNITS>{});
 
     // partial sums into the wave's own (drained) activation ring, then row group g is added up by wave g
-    f32x4v *red = (f32x4v *)aring;                       // [wave][8][lane]: the first 4 KB of each wave's own 8 KB
+    f32x4v *red = (f32x4v *)aring;                       // [wave][4 AD][lane]: the first 4 KB of each wave's own ring
 #pragma unroll
-    for (int g = 0; g < MB; ++g) red[(wave * 8 + g) * 64 + lane] = acc[g];
+    for (int g = 0; g < MB; ++g) red[(wave * 4 * AD + g) * 64 + lane] = acc[g];
     __syncthreads();
     if (wave >= MB) return;
     const int row = 16 * wave + l16;
     f32x4v sum = red[wave * 64 + lane];                  // wave 0's partial of group `wave`
 #pragma unroll
     for (int w = 1; w < kThinWaves; ++w) {
-        const f32x4v x = red[(w * 8 + wave) * 64 + lane];
+        const f32x4v x = red[(w * 4 * AD + wave) * 64 + lane];
         sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
     }
     if (row >= M) return;
@@ -465,7 +465,9 @@ void launch_thin_per(const void *Aq, const void *As, const void *Bq, const void 
     }
     const dim3 grid((unsigned)(N / 16)), block(64 * kThinWaves);
     const uint8_t *a = (const uint8_t *)Aq, *b = (const uint8_t *)Bq;
-    if (M > 48) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    // 49 to 64 rows: weight ring three blocks deep and activation ring three units (158 KB of LDS; with four and two,
+    // 142 KB, M = 64, N = 4096, K = 7168 takes 12.9 instead of 12.75 us)
+    if (M > 48) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 4, 3, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
     else if (M > 32) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
     else if (M > 16) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
     else if (kind == 0) hipLaunchKernelGGL((gemm_thin<SDT, PER>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
