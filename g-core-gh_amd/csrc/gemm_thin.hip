@@ -261,11 +261,11 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
 // ---------------------------------------------------------------------------------------------------------
 // 17 to 64 activation rows: the same cut (16 weight rows x all of K per workgroup), but the activations of a K
 // block are now 2 to 4 row groups of 16, up to 8 KB against 2 KB of weights, and would fill a common ring with
-// bytes that come from L2.  So the two operands get rings of their own: weights 4 K blocks deep (what HBM
-// latency asks for), activations two units of 32 rows (L2 latency), a K block being one or two units.
+// bytes that come from L2.  So the two operands get rings of their own: weights BS K blocks deep (HBM
+// latency), activations AD units of 32 rows (L2 latency), a K block being one or two units (BS = 4, AD = 2, or 3 and 3).
 // Plan of the requests of one wave, in issue order, so that every wait can name how many younger requests may
-// still be in flight: weight blocks 0 .. BS-1 (2 requests each), activation units 0 and 1 (4 each); then at
-// step u, after the reads, unit u + 2 and, on the first unit of a block j, weight block j + BS.
+// still be in flight: weight blocks 0 .. BS-1 (2 requests each), activation units 0 .. AD-1 (4 each); then at
+// step u, after the reads, unit u + AD and, on the first unit of a block j, weight block j + BS.
 template <int PER, int U, int BS, int AD>
 struct RingPlan {
     int a_end[PER * U];          // requests issued up to and including activation unit u
