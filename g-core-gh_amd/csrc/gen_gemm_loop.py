@@ -678,7 +678,7 @@ def main():
 
 
 def probe_bodies(here):
-    """Bodies of the matrix-pipe probe (selftest.hip: probe_mfma): eight matrix instructions into eight result buffers
+    """Bodies of the matrix-pipe probe (probe/probe.hip: probe_mfma): eight matrix instructions into eight result buffers
     v[32:63], each followed by k FMAs that fold a buffer finished four instructions ago into v[64:127] -- the arithmetic
     of the fp32-scaled loops with no operand movement at all."""
     global lines
@@ -689,7 +689,7 @@ def probe_bodies(here):
             src = (j + 4) % 8
             for f in range(k):
                 lines.append(f"v_fmac_f32 v{64 + (j * 8 + f) % 64}, v{32 + 4 * src + f % 4}, v20")
-        write(here, f"probe_mfma_body{k}.inc")
+        write(os.path.join(here, "probe"), f"probe_mfma_body{k}.inc")
 
 
 def write(here, name):

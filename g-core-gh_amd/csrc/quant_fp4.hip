@@ -173,41 +173,7 @@ __global__ __launch_bounds__(256) void quant_fp4_generic(const void *__restrict_
     }
 }
 
-// self test: hardware conversion with the tie adjustment == software rounding, every finite fp32, three scales
-__global__ __launch_bounds__(256) void st_cvt_to_fp4(uint64_t *out)
-{
-    const uint32_t base = (blockIdx.x * 256u + threadIdx.x) * 16u;
-    bool bad = false;
-    for (int k = 0; k < 3; ++k) {
-        const int e = k == 0 ? 0 : (k == 1 ? -7 : 9);
-        const uint32_t eb = (uint32_t)e << 23;
-        const uint32_t t0 = 0x3F400000u + eb, t1 = 0x3FE00000u + eb, t2 = 0x40600000u + eb;
-        const float s = u2f((uint32_t)(e + 127) << 23);
-        for (uint32_t i = 0; i < 16u; i += 2) {
-            uint32_t b0 = base + i, b1 = base + i + 1;
-            const uint32_t a0 = b0 & 0x7FFFFFFFu, a1 = b1 & 0x7FFFFFFFu;
-            const bool ok0 = a0 < 0x7F800000u, ok1 = a1 < 0x7F800000u;
-            const uint32_t want0 = sw_f32_to_e2m1_half_down(u2f(b0) / s), want1 = sw_f32_to_e2m1_half_down(u2f(b1) / s);
-            b0 -= (a0 == t0) | (a0 == t1) | (a0 == t2);
-            b1 -= (a1 == t0) | (a1 == t1) | (a1 == t2);
-            const uint32_t w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, ok0 ? u2f(b0) : 0.0f, ok1 ? u2f(b1) : 0.0f, s, 0);
-            if (ok0) bad |= (w & 15u) != want0;
-            if (ok1) bad |= ((w >> 4) & 15u) != want1;
-        }
-    }
-    unsigned long long b = __ballot(bad);
-    if ((threadIdx.x & 63) == 0 && b) atomicAdd((unsigned long long *)out, (unsigned long long)__popcll(b));
-}
-
 }  // namespace
-
-namespace lowp {
-int selftest_cvt_to_fp4(uint64_t *mismatches, hipStream_t st)
-{
-    hipLaunchKernelGGL(st_cvt_to_fp4, dim3(1u << 20), dim3(256), 0, st, mismatches);
-    return check_launch("lp_selftest");
-}
-}  // namespace lowp
 
 extern "C" int lp_quant_fp4_block(const void *x, int x_dtype, int64_t rows, int64_t cols, int bm, int bn, void *packed_out,
                                   void *scale_out, int32_t *nan_count, lp_stream_t stream)
