@@ -7,10 +7,17 @@
 // Data movement: each step's operand tiles (256 x 128 B of activations, TN x
 // 128 B of weights) are copied HBM/L2 -> LDS by global_load_lds_dwordx4, with
 // no VGPR staging, into one of two stages (the copy of step k+1 overlaps the
-// math of step k).  A row holds 8 chunks of 16 bytes; chunk c of row r is
-// stored in slot c ^ ((r >> 1) & 7), which makes both the linear 1 KB DMA
-// writes and the fragment reads (16 lanes = 16 consecutive rows, same chunk)
-// conflict free across the 64 LDS banks without padding.
+// math of step k).  A row holds 8 chunks of 16 bytes.  The LDS serves a
+// 16-byte-per-lane read at 256 bytes per clock only when every 8 consecutive
+// lanes stay inside one 128-byte half of the 256-byte bank line (address bit 7
+// equal) and take 8 different 16-byte slots there; rows stored in tile order
+// alternate between the halves and such a read takes twice as long (measured:
+// 1.83 x, SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE).  So inside every
+// block of 16 tile rows the rows are stored in the order 0, 8, 1, 9, ... 7, 15
+// (lds_row): the 8 rows lanes 0..7 of a fragment read address sit on even LDS
+// rows, those of lanes 8..15 on odd ones, and chunk c of tile row r is stored
+// in slot c ^ (r & 7).  The copies write LDS linearly (1 KB per instruction),
+// so the order only decides which global row a lane of a copy fetches.
 //
 // Math: v_mfma_f32_16x16x128_f8f6f4 -- one instruction covers the whole 128-wide
 // scale block, so every MFMA starts from a zero accumulator and its 4 results
@@ -37,19 +44,10 @@ constexpr int THREADS = 512;
 #define LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
 #define GLB_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
 
-#ifndef LP_SWZ
-#define LP_SWZ 0
-#endif
-__device__ __forceinline__ int swz(int row, int chunk)
-{
-#if LP_SWZ == 0
-    return chunk ^ ((row >> 1) & 7);
-#elif LP_SWZ == 1
-    return chunk ^ (row & 7);
-#else
-    return chunk ^ ((row >> 2) & 7);
-#endif
-}
+// LDS row that holds tile row r, the tile row an LDS row holds, and the slot of chunk c of tile row r
+__device__ __forceinline__ int lds_row(int r) { return (r & ~15) | ((r & 7) << 1) | ((r >> 3) & 1); }
+__device__ __forceinline__ int tile_row(int p) { return (p & ~15) | ((p >> 1) & 7) | ((p & 1) << 3); }
+__device__ __forceinline__ int swz(int r, int chunk) { return chunk ^ (r & 7); }
 
 // NB = 16-column blocks per wave; TN = 2 * 16 * NB
 template <int SDT, int NB>
@@ -78,13 +76,13 @@ __global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ 
     const uint8_t *b_src[TN / 64];
 #pragma unroll
     for (int i = 0; i < BM / 64; ++i) {
-        const int row = 8 * (wave + 8 * i) + ld_row;
+        const int row = tile_row(8 * (wave + 8 * i) + ld_row);
         const int64_t m = m0 + row < M ? m0 + row : M - 1;
         a_src[i] = Aq + m * K + swz(row, ld_slot) * 16;
     }
 #pragma unroll
     for (int i = 0; i < TN / 64; ++i) {
-        const int row = 8 * (wave + 8 * i) + ld_row;
+        const int row = tile_row(8 * (wave + 8 * i) + ld_row);
         const int64_t n = n0 + row < N ? n0 + row : N - 1;
         b_src[i] = Bq + n * K + swz(row, ld_slot) * 16;
     }
@@ -147,15 +145,15 @@ __global__ __launch_bounds__(THREADS) void gemm_big(const uint8_t *__restrict__ 
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
             const int row = wm * 64 + mb * 16 + l16;
-            const u32x4 x0 = *(const u32x4 *)(sa + row * KB + swz(row, 2 * lq) * 16);
-            const u32x4 x1 = *(const u32x4 *)(sa + row * KB + swz(row, 2 * lq + 1) * 16);
+            const u32x4 x0 = *(const u32x4 *)(sa + lds_row(row) * KB + swz(row, 2 * lq) * 16);
+            const u32x4 x1 = *(const u32x4 *)(sa + lds_row(row) * KB + swz(row, 2 * lq + 1) * 16);
             af[mb] = i32x8{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
         }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const int row = wn * (TN / 2) + nb * 16 + l16;
-            const u32x4 y0 = *(const u32x4 *)(sb + row * KB + swz(row, 2 * lq) * 16);
-            const u32x4 y1 = *(const u32x4 *)(sb + row * KB + swz(row, 2 * lq + 1) * 16);
+            const u32x4 y0 = *(const u32x4 *)(sb + lds_row(row) * KB + swz(row, 2 * lq) * 16);
+            const u32x4 y1 = *(const u32x4 *)(sb + lds_row(row) * KB + swz(row, 2 * lq + 1) * 16);
             const i32x8 wf = i32x8{(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
             const int which = nb >= split_nb ? 1 : 0;
 #pragma unroll
@@ -349,7 +347,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     uint64_t amask[4];                                  // lanes of activation copy i whose row exists
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int row = 8 * (wave + WAVES * i) + ld_row;
+        const int row = tile_row(8 * (wave + WAVES * i) + ld_row);      // the tile row this lane's 16 bytes of LDS hold
         amask[i] = __ballot(m0 + row < M);
         // a lane whose row is past the end of the activations is switched off for the copy (amask): its offset only has to exist
         const int64_t m = m0 + row < M ? m0 + row : m0;
@@ -370,7 +368,7 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     // weight scale row(s) of this wave.  With TN / 2 = 128 or 64 columns per wave they lie in one scale block;
     // 96 columns can straddle two, and each pair of 16-column blocks is told which of the two rows it uses.
     const int64_t wcol0 = n0 + wn * (TN / WN);
-    const int64_t last_blk = (N >> 7) - 1;
+    const int64_t last_blk = N >= 128 ? (N >> 7) - 1 : 0;       // never in front of the table, whatever the caller's N
     int64_t sblk = wcol0 >> 7;
     if (sblk > last_blk) sblk = last_blk;
     const uint64_t bs_u = uniform((const char *)Bs + sblk * kblocks * SS);
@@ -408,10 +406,10 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
     const uint32_t m0base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
     const int arow_l = wm * 64 + l16, brow_l = wn * (TN / WN) + l16;
-    const uint32_t ard0 = lds0 + arow_l * KB + swz(arow_l, 2 * lq) * 16;
-    const uint32_t ard1 = lds0 + arow_l * KB + swz(arow_l, 2 * lq + 1) * 16;
-    const uint32_t brd0 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq) * 16;
-    const uint32_t brd1 = lds0 + T::B_LDS + brow_l * KB + swz(brow_l, 2 * lq + 1) * 16;
+    const uint32_t ard0 = lds0 + lds_row(arow_l) * KB + swz(arow_l, 2 * lq) * 16;
+    const uint32_t ard1 = lds0 + lds_row(arow_l) * KB + swz(arow_l, 2 * lq + 1) * 16;
+    const uint32_t brd0 = lds0 + T::B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq) * 16;
+    const uint32_t brd1 = lds0 + T::B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq + 1) * 16;
     // scale staging: 16 bytes per activation row (fp32, four K steps), or 4 bytes per row in 1 KB per copying wave (e8m0)
     const uint32_t srd = HWS ? lds0 + T::S_LDS + wm * 1024 + l16 * 4 : lds0 + T::S_LDS + arow_l * 16;
     // row-scaled weights: their dwords live behind the two activation halves, 1 KB per copying wave like those

@@ -233,7 +233,8 @@ extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M,
     // loop with every scale 2^0 (e8m0 scales are applied inside the matrix instruction at no cost), instead of the
     // compiler-scheduled kernel below.  LP_GEMM_NT_PLAIN=1 keeps that one.
     static const bool plain = getenv("LP_GEMM_NT_PLAIN") != nullptr;
-    if (!plain && in_dtype == LP_E4M3 && K % 512 == 0 && N % 16 == 0 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
+    // (N >= 128: the loop indexes weight scales by 128-row block and needs at least one whole block)
+    if (!plain && in_dtype == LP_E4M3 && K % 512 == 0 && N % 16 == 0 && N >= 128 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
         M * (K / 128) <= kUnitScaleBytes && ((N + 127) / 128) * (K / 128) <= kUnitScaleBytes) {
         const void *ones = unit_scale_array(st);
         if (ones && gemm::nt_unit_scales_ok(ones, M, N, K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, K, C, out_dtype, st);

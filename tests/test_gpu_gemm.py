@@ -276,7 +276,10 @@ def test_grouped_linear_module(G):
 # ---------------------------------------------------------------------------------------------
 # unscaled NT GEMM (gemm_impl): shapes and tolerance of the reference's test_gemm_fp8
 NT_SHAPES = [(128, 4096, 2048), (512, 1024, 4096), (2048, 4096, 1024), (4096, 4096, 4096), (200, 1280, 4096),
-             (1000, 16384, 512), (1, 16, 128), (77, 4112, 256)]
+             (1000, 16384, 512), (1, 16, 128), (77, 4112, 256),
+             # enough tiles for the hand-scheduled loop with unit scales: a ragged last column block, and fewer columns
+             # than one weight-scale block (which must stay on the compiler-scheduled kernel)
+             (4096, 4112, 512), (51200, 48, 512)]
 
 
 @pytest.mark.parametrize("shape", NT_SHAPES, ids=lambda s: "M%d_N%d_K%d" % s)
