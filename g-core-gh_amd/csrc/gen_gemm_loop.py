@@ -40,7 +40,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP, SPREAD
     # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
     # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
     WITH_IDLE, IDLE = idle, False
@@ -57,6 +57,9 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
     # weight copies by wave (s87 = 1 for the first half of the waves) instead of by copy index.
     HALFSPLIT = early and tn // waves_n == 64 and waves_m * waves_n == 8
+    # one copy behind each matrix instruction instead of runs of copies (see dma_chunks); the flat tile, whose weight
+    # copies are split by wave behind one branch, keeps its runs
+    SPREAD = early and not HALFSPLIT and SPREAD_ON
     # wide: a wave owns 64 x 144 columns (nine 16-column blocks), e.g. the 256 x 288 tile that cuts 18432 weight rows
     # into exactly 64 tile columns.  144 columns always straddle two weight-scale blocks, at a 16-column boundary known
     # only at run time (s74 = first block that takes the second scale row): the folds read one set of scale products,
@@ -215,6 +218,43 @@ def dma(stage, part="all"):
                 lo = int(WB_EXTRA[i][2:4])
                 emit(f"s_add_u32 s{lo}, s{lo}, 128")
                 emit(f"s_addc_u32 s{lo + 1}, s{lo + 1}, 0")
+
+
+def dma_chunks(stage, part):
+    """The copies of dma(stage, part) as a list of pieces, one copy instruction each (with its m0 / exec set-up and the
+    label that closes a copy only some waves have); the advance of the operand bases rides on the last piece.  The
+    loop issues one piece behind each matrix instruction instead of all copies in one run: the eight waves reach the
+    copies together (they follow a barrier), a run of six from each queues 48 KB of requests in front of the CU's one
+    address unit, and a wave stuck at its third copy issues no matrix instruction either."""
+    global lines
+    saved, lines = lines, []
+    dma(stage, part)
+    body, lines = lines, saved
+    out, cur, i = [], [], 0
+    while i < len(body):
+        cur.append(body[i])
+        if body[i].startswith("global_load_lds"):
+            while i + 1 < len(body) and (body[i + 1].startswith("Lnobx") or body[i + 1].startswith("s_mov_b64 exec, s[98:99]")):
+                cur.append(body[i + 1])
+                i += 1
+            out.append(cur)
+            cur = []
+        i += 1
+    if cur:
+        assert out
+        out[-1] += cur
+    return out
+
+
+def emit_piece(piece, tag, cond):
+    """One piece of dma_chunks behind a matrix instruction; cond: skipped on the last trip (s50 = 1), when the step it
+    would fill lies past the end of K."""
+    if cond:
+        emit("s_cmp_eq_u32 s50, 1")
+        emit(f"s_cbranch_scc1 Lnop{tag}%=")
+    lines.extend(piece)
+    if cond:
+        emit(f"Lnop{tag}%=:")
 
 
 def copies_per_part():
@@ -400,6 +440,7 @@ def step(c):
         emit(f"v_add_u32 {SRD}, s55, {SRD0}")
         if BROW:
             emit(f"v_add_u32 v{SRDB}, s55, v{SRDB0}")
+    pieces = []                  # copies waiting for their slot behind a matrix instruction: (piece, tag, skipped on the last trip)
     read_frag(WFB[par(c, 1)], RB0, RB1, boff + 2048)
     # LDS queue now: wf0, af0..3, wf1 = 12 reads
     if PINGPONG:
@@ -422,7 +463,7 @@ def step(c):
         # last read of the first half, so those rows and the activation rows can be requested again right after it.
         handback = EARLY and nb == NB // 2 - 1
         if handback:
-            assert nb + 1 < NB
+            assert nb + 1 < NB and not pieces
             wait_copies(c, False, " lgkmcnt(0)")
             emit("s_barrier")
         if nb + 1 < NB:
@@ -437,6 +478,7 @@ def step(c):
         if nb + 1 == NB:
             if flip:
                 # every wave has read all of this stage and its share of the next stage has landed
+                assert not pieces                # the waits count every copy of the mid-step part as issued
                 if EARLY:
                     wait_copies(c, True, " lgkmcnt(0)")
                 elif NSTAGE == 2:
@@ -481,23 +523,33 @@ def step(c):
             if handback and mb == 0:
                 # the activation rows and the first weight half of the step after the next, into the rows just freed
                 cond = c + NSTAGE >= 4 if ROT else c + 1 + KSUB >= 4
-                if cond:
-                    emit("s_cmp_eq_u32 s50, 1")
-                    emit(f"s_cbranch_scc1 Lnodmam{c}%=")
-                dma(stage, "mid")
-                if cond:
-                    emit(f"Lnodmam{c}%=:")
+                if SPREAD:
+                    pieces += [(pc, f"m{c}_{i}", cond) for i, pc in enumerate(dma_chunks(stage, "mid"))]
+                else:
+                    if cond:
+                        emit("s_cmp_eq_u32 s50, 1")
+                        emit(f"s_cbranch_scc1 Lnodmam{c}%=")
+                    dma(stage, "mid")
+                    if cond:
+                        emit(f"Lnodmam{c}%=:")
             if nb + 1 == NB:
                 read_frag(AF + 8 * mb, RA0, RA1, naoff + mb * 2048)
                 if mb == 0 and flip:
                     # copies for the K blocks after the next stage overwrite the stage just finished
                     cond = NSTAGE == 4 or (c + NSTAGE >= 4 if ROT else c + 1 + KSUB >= 4)
-                    if cond:
-                        emit("s_cmp_eq_u32 s50, 1")
-                        emit(f"s_cbranch_scc1 Lnodma{c}%=")
-                    dma(stage, "end" if EARLY else "all")
-                    if cond:
-                        emit(f"Lnodma{c}%=:")
+                    if SPREAD:
+                        assert not pieces
+                        pieces += [(pc, f"e{c}_{i}", cond) for i, pc in enumerate(dma_chunks(stage, "end"))]
+                        assert len(pieces) <= MB
+                    else:
+                        if cond:
+                            emit("s_cmp_eq_u32 s50, 1")
+                            emit(f"s_cbranch_scc1 Lnodma{c}%=")
+                        dma(stage, "end" if EARLY else "all")
+                        if cond:
+                            emit(f"Lnodma{c}%=:")
+            if pieces:
+                emit_piece(*pieces.pop(0))
         if WIDE and not HW:
             # the folds of block nb follow (in the next block's shadow): if it is the first block in the second
             # weight-scale block, they and all later ones use that row's products
@@ -506,6 +558,7 @@ def step(c):
             for mb in range(MB):
                 emit(f"v_mov_b32 v{SC + mb}, v{SC2 + mb}")
             emit(f"Lsw{c}_{nb}%=:")
+    assert not pieces
     # fold of the last block: the 12 folds of mb 0..2 separate the last MFMA from the read of its result
     for mb in range(MB):
         fold(NB - 1, mb, c)
@@ -657,6 +710,7 @@ def generate():
 
 
 PP = os.environ.get("LP_GEN_PINGPONG", "1") == "1"
+SPREAD_ON = os.environ.get("LP_GEN_SPREAD", "1") == "1"
 
 
 def main():
