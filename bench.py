@@ -37,12 +37,25 @@ sys.path.insert(0, os.path.join(ROOT, "g-core-gh_amd"))
 SETTLE_MS = 40.0             # untimed graph replays before every timed region (see time_launches)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA
-# Bytes per launch of the headline GEMM kernel between its L2s and the memory side (Infinity Cache / HBM): reads from
-# the request-size counters (32 / 64 / 128-byte TCC->EA reads, exact; the derived FETCH_SIZE prices the 128-byte
-# requests of LDS-direct and non-temporal loads at 64) plus WRITE_SIZE.  Counters cannot be read from inside this process:
-# the figures are those of rocprofv3 --pmc runs of this script (profiles/gemm_kernels_mfma_lds_hbm_counters.txt), not of this run.
-GEMM_BIG_TRAFFIC_BYTES = 430.0e6     # gemm_asm<256,256,1> on 16384 weight rows: 362.9 MB read + 67.1 MB written
-GEMM_WIDE_TRAFFIC_BYTES = 461.2e6    # gemm_asm_wide<false> on the whole problem: 376.5 MB read + 84.7 MB written
+# Bytes per launch between a kernel's L2s and the memory side (Infinity Cache / HBM) cannot be read from inside this
+# process: `roofline.traffic` comes from profiles/traffic.json, which profile_summary.py writes from rocprofv3 --pmc
+# runs of this script (reads from the request-size counters, 32 / 64 / 128-byte TCC->EA reads, exact -- the derived
+# FETCH_SIZE prices the 128-byte requests of LDS-direct and non-temporal loads at 64 -- plus WRITE_SIZE).  A kernel the
+# file does not list reports null.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(kernel, grid_threads):
+    """read + write bytes per launch of `kernel` at that grid size from the committed counter summary, or None."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            table = json.load(f)["kernels"]
+    except (OSError, ValueError, KeyError):
+        return None
+    for row in table:
+        if row["kernel"].startswith(kernel) and row["grid_threads"] == grid_threads:
+            return row["read_bytes"] + row["write_bytes"]
+    return None
 
 
 def main():
@@ -66,11 +79,13 @@ def main():
         sys.exit("bench.py: no GPU visible")
     import gcore_lowp  # noqa: F401  (fails loudly if the HIP library is missing)
     from gcore_lowp import _abi as A
-    from tests._inputs import zipf_m_splits        # the grouped problem's rows per expert: one recipe for tests and bench
+    from gcore_lowp import _probe_abi as PA            # bare-stream / matrix-pipe / copy-path probes (liblowp_probe.so)
+    from tests._inputs import zipf_m_splits_with_idle_expert as zipf_m_splits   # the grouped problem's rows per expert: one recipe for tests and bench
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     L = A.lib()
+    LP = PA.lib()
     E4M3, E8M0 = torch.float8_e4m3fn, torch.float8_e8m0fnu
 
     def stream():
@@ -256,7 +271,7 @@ def main():
         probe = {}
         for tag, ptr in (("zero_operands", None), ("random_e4m3_operands", rnd.data_ptr())):
             for k in (0, 4, 8):
-                ms_p, _ = time_launches([lambda k=k, ptr=ptr: chk(L.lp_probe_mfma(k, iters, ptr, wgs, stream()))], 6, 2)
+                ms_p, _ = time_launches([lambda k=k, ptr=ptr: PA.check(LP.lp_probe_mfma(k, iters, ptr, wgs, stream()))], 6, 2)
                 probe[f"{tag}_{k}_fmas_per_instruction"] = {"ms": ms_p, "tflops": fl_p / ms_p / 1e9, "mfma_frac": fl_p / ms_p / 1e9 / FP8_PEAK_TFLOPS}
         extras["matrix_pipe_probe_registers_only"] = probe
         # what a CU's copy path out of the L2 delivers in the loops' request shape (1 KB per wave and request, rows 7168 bytes
@@ -271,7 +286,7 @@ def main():
         for tag, to_lds, waves, per_cu in (("to_lds_8_waves_1_wg_per_cu", 1, 8, 1), ("to_lds_4_waves_2_wg_per_cu", 1, 4, 2),
                                            ("to_registers_8_waves_1_wg_per_cu", 0, 8, 1)):
             wg = cus * per_cu
-            ms_c, _ = time_launches([lambda to_lds=to_lds, waves=waves, wg=wg: chk(L.lp_probe_copy(
+            ms_c, _ = time_launches([lambda to_lds=to_lds, waves=waves, wg=wg: PA.check(LP.lp_probe_copy(
                 to_lds, waves, steps_c, rows_src.data_ptr(), rows_src.numel(), 7168, sink.data_ptr(), wg, stream()))], 6, 2)
             by = float(wg) * waves * steps_c * 8192
             cp[tag] = {"ms": ms_c, "TB/s": by / ms_c / 1e9, "bytes_per_ns_per_cu": by / ms_c / 1e6 / cus}
@@ -326,9 +341,9 @@ def main():
         # a bare stream of the same bytes: read 32 MiB + write 16 MiB (the quantiser's traffic) and the reverse
         probes = {}
         for wgs in (512, 1024, 2048, 4096):
-            fq = [(lambda i=i: chk(L.lp_probe_stream(xs[i].data_ptr(), R * C * 2, qs[i].data_ptr(), R * C, wgs, stream())))
+            fq = [(lambda i=i: PA.check(LP.lp_probe_stream(xs[i].data_ptr(), R * C * 2, qs[i].data_ptr(), R * C, wgs, stream())))
                   for i in range(sets)]
-            fd = [(lambda i=i: chk(L.lp_probe_stream(qs[i].data_ptr(), R * C, outs[i].data_ptr(), R * C * 2, wgs, stream())))
+            fd = [(lambda i=i: PA.check(LP.lp_probe_stream(qs[i].data_ptr(), R * C, outs[i].data_ptr(), R * C * 2, wgs, stream())))
                   for i in range(sets)]
             probes[f"read32MiB_write16MiB_{wgs}_workgroups_us"] = time_launches(fq, 48, 12)[0] * 1e3
             probes[f"read16MiB_write32MiB_{wgs}_workgroups_us"] = time_launches(fd, 48, 12)[0] * 1e3
@@ -342,48 +357,51 @@ def main():
         torch.cuda.empty_cache()
 
     if want("c3"):
-        # -------------------------------------------------------------- config 3: skinny GEMM
-        M3, N3, K3 = 64, 4096, 7168
-        sets = 12                                   # 12 x 29 MB of weights > 256 MB
-        a3 = randn(M3, K3)
-        a3q = torch.empty(M3, K3, dtype=torch.uint8, device=dev)
-        a3s = torch.empty(M3, K3 // 128, dtype=torch.float32, device=dev)
+        # -------------------------------------------------------------- config 3: skinny GEMM, and the same 64 tokens
+        # against config 2's 18432 weight rows (a 132 MB weight stream, long enough to amortise launch and first bytes)
+        K3 = 7168
+        a3 = randn(64, K3)
+        a3q = torch.empty(64, K3, dtype=torch.uint8, device=dev)
+        a3s = torch.empty(64, K3 // 128, dtype=torch.float32, device=dev)
         quant_into(a3, 1, 128, a3q, a3s)
-        w3q, w3s = [], []
-        for _ in range(sets):
-            w = randn(N3, K3, std=0.02)
-            q = torch.empty(N3, K3, dtype=torch.uint8, device=dev)
-            s = torch.empty(N3 // 128, K3 // 128, dtype=torch.float32, device=dev)
-            quant_into(w, 128, 128, q, s)
-            w3q.append(q)
-            w3s.append(s)
-        c3 = torch.empty(M3, N3, dtype=torch.bfloat16, device=dev)
-        nws = L.lp_gemm_workspace_bytes(M3, N3, K3)
-        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
-        fns = [(lambda i=i: chk(L.lp_gemm_fp8_block(a3q.data_ptr(), a3s.data_ptr(), w3q[i].data_ptr(), w3s[i].data_ptr(), A.F32,
-                                                    M3, N3, K3, c3.data_ptr(), A.BF16, ws.data_ptr(), nws, stream())))
-               for i in range(sets)]
-        ms3, _ = time_launches(fns, 48, 12)
-        bytes3 = N3 * K3 + (N3 // 128) * (K3 // 128) * 4 + M3 * K3 + M3 * (K3 // 128) * 4 + M3 * N3 * 2
-        extras["c3_skinny_gemm"] = {"ms": ms3, "GB/s": bytes3 / ms3 / 1e6, "hbm_frac": bytes3 / ms3 / 1e6 / HBM_PEAK_GBS,
-                                    "weight_GB/s": N3 * K3 / ms3 / 1e6, "tflops": 2.0 * M3 * N3 * K3 / ms3 / 1e9,
-                                    "bytes": bytes3}
-        # what the box takes for an empty launch and for a bare stream of the same bytes (rotating buffers like above)
-        ms_empty, _ = time_launches([lambda: chk(L.lp_probe_stream(None, 0, None, 0, 256, stream()))], 48, 12)
+        ms_empty, _ = time_launches([lambda: PA.check(LP.lp_probe_stream(None, 0, None, 0, 256, stream()))], 48, 12)
         sink = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
-        wbytes = N3 * K3
-        probes = {"empty_launch_us": ms_empty * 1e3}
-        for wgs in (256, 512, 1024, 2048):
-            fns = [(lambda i=i: chk(L.lp_probe_stream(w3q[i].data_ptr(), wbytes, sink.data_ptr(), 4096 * wgs // 256, wgs, stream())))
+        for tag, probe_tag, M3, N3, sets in (("c3_skinny_gemm", "c3_floor_probe", 64, 4096, 12),
+                                             ("decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", 64, 18432, 4)):
+            w3q, w3s = [], []                           # sets x N3 x 7168 bytes of weights > 256 MB
+            for _ in range(sets):
+                w = randn(N3, K3, std=0.02)
+                q = torch.empty(N3, K3, dtype=torch.uint8, device=dev)
+                sc = torch.empty(N3 // 128, K3 // 128, dtype=torch.float32, device=dev)
+                quant_into(w, 128, 128, q, sc)
+                w3q.append(q)
+                w3s.append(sc)
+                del w
+            c3 = torch.empty(M3, N3, dtype=torch.bfloat16, device=dev)
+            nws = L.lp_gemm_workspace_bytes(M3, N3, K3)
+            ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+            fns = [(lambda i=i: chk(L.lp_gemm_fp8_block(a3q.data_ptr(), a3s.data_ptr(), w3q[i].data_ptr(), w3s[i].data_ptr(), A.F32,
+                                                        M3, N3, K3, c3.data_ptr(), A.BF16, ws.data_ptr(), nws, stream())))
                    for i in range(sets)]
-            msp, _ = time_launches(fns, 48, 12)
-            probes[f"read_29MB_{wgs}_workgroups_us"] = msp * 1e3
-        best = min(v for k, v in probes.items() if k.startswith("read_"))
-        probes["read_29MB_best_GB/s"] = wbytes / best / 1e3
-        probes["skinny_gemm_over_bare_read"] = ms3 * 1e3 / best
-        extras["c3_floor_probe"] = probes
-        del w3q, w3s, sink
-        torch.cuda.empty_cache()
+            ms3, _ = time_launches(fns, 48, 12)
+            bytes3 = N3 * K3 + (N3 // 128) * (K3 // 128) * 4 + M3 * K3 + M3 * (K3 // 128) * 4 + M3 * N3 * 2
+            extras[tag] = {"ms": ms3, "GB/s": bytes3 / ms3 / 1e6, "hbm_frac": bytes3 / ms3 / 1e6 / HBM_PEAK_GBS,
+                           "weight_GB/s": N3 * K3 / ms3 / 1e6, "tflops": 2.0 * M3 * N3 * K3 / ms3 / 1e9, "bytes": bytes3}
+            # what the box takes for an empty launch and for a bare stream of the same weight bytes (rotating buffers like above)
+            wbytes = N3 * K3
+            probes = {"empty_launch_us": ms_empty * 1e3}
+            for wgs in (256, 512, 1024, 2048):
+                fns = [(lambda i=i: PA.check(LP.lp_probe_stream(w3q[i].data_ptr(), wbytes, sink.data_ptr(), 4096 * wgs // 256, wgs, stream())))
+                       for i in range(sets)]
+                msp, _ = time_launches(fns, 48, 12)
+                probes[f"read_{wbytes // 1000000}MB_{wgs}_workgroups_us"] = msp * 1e3
+            best = min(v for k, v in probes.items() if k.startswith("read_"))
+            probes["bare_read_best_GB/s"] = wbytes / best / 1e3
+            probes["gemm_over_bare_read"] = ms3 * 1e3 / best
+            extras[probe_tag] = probes
+            del w3q, w3s, c3, ws
+            torch.cuda.empty_cache()
+        del sink
 
     if want("c5"):
         # -------------------------------------------------------------- config 5: FP4 -> FP8 (fused), whole MoE layer
@@ -634,7 +652,7 @@ def main():
             ex["c3_skinny_gemm_weight_GB/s"] = 4096 * K / t3 / 1e9
             # config 4 on 4 experts (ranks 9 .. 12 by rows, about 1000 rows each; gate_up; their weights are the first
             # 4 x 4096 rows of the config-2 weight), scaled to the whole problem by flops
-            ms4 = zipf_m_splits(256, 8192, 8, seed=4321).tolist()
+            ms4 = zipf_m_splits(256, 8192, 8, seed=4321).tolist()        # (one of the 256 experts has no rows)
             sub = sorted(range(256), key=lambda e: -ms4[e])[8:12]
             rows_sub = [ms4[e] for e in sub]
             x4c = torch.randn(sum(rows_sub), K, generator=g).to(torch.bfloat16)
@@ -663,12 +681,13 @@ def main():
         "config": {"workload": "C2 dense block-FP8 GEMM: A[2048,7168] 1x128 e4m3 x B[18432,7168] 128x128 e4m3, fp32 scales -> bf16 [2048,18432]",
                    "M": M, "N": N, "K": K, "operands": "pre-quantised, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_WIDE_TRAFFIC_BYTES,
+                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": measured_traffic("gemm_asm_wide<false>", 512 * 512),
+                     "traffic_source": "profiles/traffic.json (rocprofv3 --pmc runs of this script, summarised by profile_summary.py)",
                      "kernel": "gemm_asm_wide<false>: the whole problem in one launch, 512 tiles of 256x288 (two full rounds of 256 CUs)",
                      "launch_ms": ms, "flops_per_launch": flops, "wall_ms_per_step": wall_ms,
                      "tiles_256x256_alone": {"kernel": "gemm_asm<256,256,1>: M=2048, weight rows 0..16383 of 18432, K=7168 (512 tiles)",
                                          "launch_ms": big_ms, "flops_per_launch": big_flops, "tflops": big_tflops,
-                                         "frac": big_tflops / FP8_PEAK_TFLOPS, "traffic": GEMM_BIG_TRAFFIC_BYTES}},
+                                         "frac": big_tflops / FP8_PEAK_TFLOPS, "traffic": measured_traffic("gemm_asm<256, 256, 1, false, 2>", 512 * 512)}},
         "cpu_baseline": cpu,
         "extras": extras,
     }

@@ -69,3 +69,12 @@ def zipf_m_splits(experts=256, tokens=8192, topk=8, seed=4321, exponent=1.1):
     choice = torch.multinomial(pop.expand(tokens, experts), topk, replacement=False, generator=g)
     return torch.bincount(choice.flatten(), minlength=experts)
 
+
+
+def zipf_m_splits_with_idle_expert(experts=256, tokens=8192, topk=8, seed=4321, exponent=1.1):
+    """The grouped-GEMM benchmark problem as it is timed and tested: the Zipf law over experts - 1 experts and one
+    expert in the middle of the list that no token chose (per-expert rows then range from 0 upwards, and the kernels'
+    empty-expert path is part of the measured launch).  Same total: tokens * topk rows."""
+    m = zipf_m_splits(experts - 1, tokens, topk, seed, exponent)
+    mid = experts // 2
+    return torch.cat([m[:mid], torch.zeros(1, dtype=m.dtype), m[mid:]])

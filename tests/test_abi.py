@@ -17,10 +17,19 @@ def lib():
     return _abi
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "lowp.h")).read()
+def _declared(header="lowp.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(lp_[a-z0-9_]+)\s*\(", text)))
+
+
+def _declarations_with_comments(header="lowp.h"):
+    """(name, text of the comment block right in front of the declaration) for every entry point of a header."""
+    text = open(os.path.join(ROOT, "include", header)).read()
+    out = []
+    for m in re.finditer(r"/\*((?:(?!\*/).)*)\*/\s*(?:const\s+char\s*\*|int64_t|int)\s*(lp_[a-z0-9_]+)\s*\(", text, flags=re.S):
+        out.append((m.group(2), m.group(1)))
+    return out
 
 
 def test_every_declared_symbol_is_exported_and_bound(lib):
@@ -32,6 +41,45 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
         assert n in lib.PROTOTYPES, f"{n} has no ctypes prototype"
     assert sorted(lib.PROTOTYPES) == names
     assert L.lp_version() >= 100
+
+
+def test_drop_in_header_lists_only_reference_interfaces(lib):
+    """include/lowp.h is the drop-in ABI: every entry point's comment cites the reference interface it stands in for
+    (a file:line in the reference tree), or is one of the plumbing calls of the library itself (version, error text,
+    workspace / scratch sizes), or says that it has no counterpart and whom it is for (the entry point that allocates
+    nothing).  Measurement aids and self tests live in include/lowp_probe.h and in a library of their own."""
+    plumbing = {"lp_version", "lp_last_error", "lp_gemm_workspace_bytes", "lp_gemm_static_scratch_bytes"}
+    cite = re.compile(r"[A-Za-z0-9_/]+\.py:\d+")
+    decls = _declarations_with_comments()
+    names = {n for n, _ in decls}
+    assert names | plumbing >= set(_declared()), sorted(set(_declared()) - names - plumbing)
+    for name, comment in decls:
+        if name in plumbing:
+            continue
+        assert "probe" not in name and "selftest" not in name and "debug" not in name, name
+        assert cite.search(comment) or "no counterpart in the reference" in comment, f"{name}: no reference citation"
+    probe = _declared("lowp_probe.h")
+    assert not set(probe) & set(_declared()), "an entry point is declared in both headers"
+
+
+def test_probe_header_matches_probe_library(lib):
+    from gcore_lowp import _probe_abi as P
+    if not os.path.exists(P.LIB_PATH):
+        pytest.fail(f"{P.LIB_PATH} missing: run `python g-core-gh_amd/build.py`")
+    names = _declared("lowp_probe.h")
+    L = P.lib()
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/lowp_probe.h but not exported"
+    assert sorted(P.PROTOTYPES) == names
+    # the product library exports none of them, and does not depend on the probe library
+    prod = lib.lib()
+    for n in names:
+        assert not hasattr(prod, n), f"{n} is exported by the product library"
+    one = ctypes.c_void_p(16)
+    assert L.lp_probe_mfma(3, 10, None, 16, None) == -1 and b"FMAs" in L.lp_probe_last_error()
+    assert L.lp_probe_stream(one, 15, one, 16, 8, None) == -1
+    assert L.lp_selftest(9, one, None) == -1
+    assert L.lp_debug_cast(0, None, None, 0, None) == 0
 
 
 def test_host_side_validation(lib):

@@ -89,11 +89,12 @@ def test_prefill_gemm_at_benchmark_shape(G, pow2, shape):
 @pytest.mark.parametrize("proj,N,K", [("gate_up", 4096, 7168), ("down", 7168, 2048)])
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_grouped_gemm_at_benchmark_shape(G, proj, N, K, pow2):
-    """256 experts with the benchmark's rows per expert (Zipf 1.1, top-8 of 8192 tokens) and a 257th expert without
-    rows; every expert's rows are checked against its own fp32 dequantise-then-matmul."""
-    m_splits = I.zipf_m_splits().tolist() + [0]
+    """The benchmark's 256 experts and rows per expert (Zipf 1.1, top-8 of 8192 tokens, one expert without rows in the
+    middle of the list) and a 257th expert without rows at the end; every expert's rows are checked against its own
+    fp32 dequantise-then-matmul."""
+    m_splits = I.zipf_m_splits_with_idle_expert().tolist() + [0]
     E, Mt = len(m_splits), sum(m_splits)
-    assert Mt == 65536 and min(m_splits[:-1]) > 0
+    assert Mt == 65536 and E == 257 and m_splits.count(0) == 2 and m_splits[128] == 0
     x = _randn(Mt, K, 1.0, 21)
     xq, xs = (G.quant_fp8_e4m3_scale_e8m0(x, (1, 128)) if pow2 else G.quant_act(x))
     del x

@@ -65,9 +65,9 @@ def test_zero_rows_gemm_and_grouped_linear():
 
 
 def test_measurement_probes_launch_and_reject_bad_arguments():
-    """The measurement aids of the library (bare stream, register-only matrix-pipe loop, L2-to-LDS copy loop) are what the benchmark's
+    """The measurement aids of the probe library (bare stream, register-only matrix-pipe loop, L2-to-LDS copy loop) are what the benchmark's
     floor figures come from: they must launch for every variant the benchmark uses and refuse what they do not implement."""
-    from gcore_lowp import _abi as A
+    from gcore_lowp import _probe_abi as A
     L = A.lib()
     st = torch.cuda.current_stream().cuda_stream
     src = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")

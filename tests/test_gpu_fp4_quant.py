@@ -56,9 +56,9 @@ def check(Q, x, block=(1, 32)):
 def test_hardware_encode_matches_software():
     """v_cvt_scalef32_pk_fp4_f32 plus the tie adjustment == round-to-nearest with ties to the smaller
     magnitude, over every finite fp32 at three scales."""
-    from gcore_lowp import ops
+    from gcore_lowp import _probe_abi as probe
     say("selftest 4")
-    assert ops.selftest(4) == 0
+    assert probe.selftest(4) == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])

@@ -38,30 +38,30 @@ def G():
 def test_hardware_conversions_match_software(G, which):
     """v_cvt_pk_fp8_f32 over all |x| <= 448, v_cvt_pk_f32_fp8 over all codes, fp32->bf16 over all
     non-NaN fp32, e2m1 decode over all bytes: zero mismatches against the library's software casts."""
-    from gcore_lowp import ops
+    from gcore_lowp import _probe_abi as probe
     say("selftest", which)
-    assert ops.selftest(which) == 0
+    assert probe.selftest(which) == 0
 
 
 def test_software_casts_match_oracle(G, corc):
-    from gcore_lowp import ops
+    from gcore_lowp import _probe_abi as probe
     rng = np.random.default_rng(1)
     u = np.concatenate([np.arange(0, 1 << 32, 1 << 10, dtype=np.uint64).astype(np.uint32),
                         rng.integers(0, 1 << 32, 1 << 22, dtype=np.uint64).astype(np.uint32)])
     f = torch.from_numpy(u.view(np.float32).copy())
     isnan = np.isnan(f.numpy())
     say("debug_cast e4m3 sw")
-    got = ops.debug_cast(0, f).numpy()
+    got = probe.debug_cast(0, f).numpy()
     want = corc.f32_to_e4m3fn(f.numpy())
     assert np.array_equal(got[~isnan], want[~isnan]) and ((got[isnan] & 0x7F) == 0x7F).all()
     say("debug_cast e4m3 hw (clamped)")
-    got = ops.debug_cast(1, f).numpy()
+    got = probe.debug_cast(1, f).numpy()
     want = corc.f32_to_e4m3fn(np.clip(f.numpy(), -448, 448))
     assert np.array_equal(got[~isnan], want[~isnan])
     say("debug_cast e8m0")
-    assert np.array_equal(ops.debug_cast(2, f).numpy(), corc.f32_to_e8m0(f.numpy()))
+    assert np.array_equal(probe.debug_cast(2, f).numpy(), corc.f32_to_e8m0(f.numpy()))
     say("debug_cast bf16")
-    got = ops.debug_cast(3, f).numpy().view(np.uint16)
+    got = probe.debug_cast(3, f).numpy().view(np.uint16)
     assert np.array_equal(got[~isnan], corc.f32_to_bf16(f.numpy())[~isnan])
 
 
