@@ -1,4 +1,5 @@
-"""Builds the gfx950 C-ABI library in-tree: csrc/*.hip + api.cpp -> gcore_lowp/_lib/liblowp.so.
+"""Builds the gfx950 C-ABI library in-tree: csrc/*.hip + api.cpp -> gcore_lowp/_lib/liblowp.so, and the
+measurement / self-test aids of include/lowp_probe.h as a second library: csrc/probe/*.hip -> liblowp_probe.so.
 
 Usage: python g-core-gh_amd/build.py [--force]
 hipcc cross-compiles without a GPU.  The library links against the HIP runtime
@@ -17,6 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "gcore_lowp", "_lib")
 LIB = os.path.join(LIBDIR, "liblowp.so")
+PROBE_LIB = os.path.join(LIBDIR, "liblowp_probe.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 COMMON = [
@@ -31,14 +33,19 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cpp")))
 
 
+def probe_sources():
+    return sorted(os.path.join("probe", f) for f in os.listdir(os.path.join(CSRC, "probe")) if f.endswith(".hip"))
+
+
 def _headers_mtime():
     paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".inc"))]
-    paths.append(os.path.join(HERE, "..", "include", "lowp.h"))
+    paths += [os.path.join(CSRC, "probe", f) for f in os.listdir(os.path.join(CSRC, "probe")) if f.endswith(".inc")]
+    paths += [os.path.join(HERE, "..", "include", h) for h in ("lowp.h", "lowp_probe.h")]
     return max(os.path.getmtime(p) for p in paths)
 
 
 def _compile(src: str, force: bool) -> str:
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    obj = os.path.join(OBJ, os.path.splitext(src)[0].replace(os.sep, "_") + ".o")
     spath = os.path.join(CSRC, src)
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(spath), _headers_mtime()):
         return obj
@@ -75,15 +82,22 @@ def build(force: bool = False) -> str:
     _generate()
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(8, len(sources()))) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force), sources()))
+    srcs, psrcs = sources(), probe_sources()
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs) + len(psrcs))) as ex:
+        all_objs = list(ex.map(lambda s: _compile(s, force), srcs + psrcs))
+    objs, pobjs = all_objs[:len(srcs)], all_objs[len(srcs):]
     if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
         _audit_asm_operands()
-        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"link failed:\n{r.stderr}")
+        _link(LIB, objs)
+    if force or not os.path.exists(PROBE_LIB) or any(os.path.getmtime(o) > os.path.getmtime(PROBE_LIB) for o in pobjs):
+        _link(PROBE_LIB, pobjs)
     return LIB
+
+
+def _link(lib, objs):
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link of {os.path.basename(lib)} failed:\n{r.stderr}")
 
 
 if __name__ == "__main__":

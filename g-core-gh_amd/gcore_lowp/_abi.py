@@ -47,11 +47,6 @@ PROTOTYPES = {
     "lp_quant_fp8_colwise_t": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _i64, _i32, _p, _p, _i32, _p]),
     "lp_gemm_fp8_grouped": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
-    "lp_probe_stream": (_i32, [_p, _i64, _p, _i64, _i32, _p]),
-    "lp_probe_mfma": (_i32, [_i32, _i32, _p, _i32, _p]),
-    "lp_probe_copy": (_i32, [_i32, _i32, _i32, _p, _i64, _i64, _p, _i32, _p]),
-    "lp_selftest": (_i32, [_i32, _p, _p]),
-    "lp_debug_cast": (_i32, [_i32, _p, _p, _i64, _p]),
 }
 
 _lib = None
