@@ -325,6 +325,16 @@ def test_quant_colwise_t_matches_oracle(G):
     m_splits = [300, 0, 128, 1, 77, 513]
     x = I.act_like(sum(m_splits), 384, 21)
     x[5, 7] = 0.0
+    # columns of the first block whose maxima sit on, just above and just below 448 * 2^k (where the scale exponent
+    # steps), an all-zero column, maxima below the smallest normal float and near the largest
+    edge = [3584.0, 3600.0, 3568.0, 0.0, 2.0 ** -130, 1.75 * 2.0 ** -126, 1.7578125 * 2.0 ** -126, 3.0e38,
+            448.0 * 2.0 ** -20, 450.0 * 2.0 ** -20, 2.0 ** -133]
+    for c, v in enumerate(edge):
+        x[:128, c] *= 2.0 ** -140 if v < 1e-30 else min(1.0, abs(v) * 0.01)
+        if v == 0.0:
+            x[:128, c] = 0.0
+        else:
+            x[(7 * c + 3) % 128, c] = -v if c % 2 else v
     offs = torch.zeros(len(m_splits) + 1, dtype=torch.int32)
     offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
     for dt in (torch.bfloat16, torch.float32):
