@@ -545,6 +545,31 @@ def main():
                                                     offs_d.data_ptr(), E4, Mt, N4, K4, c4.data_ptr(), A.BF16, stream()))
             ms48, _ = time_launches([fn8], 5, 2)
             res4[name + "_e8m0_scales"] = {"ms": ms48, "tflops": fl / ms48 / 1e9, "mfma_frac": fl / ms48 / 1e9 / FP8_PEAK_TFLOPS}
+            if name == "gate_up":
+                # the data gradient of the same layer, dX_e = dY_e W_e on the stored [N4, K4] weights (layout NN,
+                # gpatch_v4/models/deepseek_v4/fp8.py:301-313): the kernel that turns the weight operand on its way out of
+                # LDS, beside a transposed copy of all weights followed by the forward kernel (what the wrapper did before)
+                dyq = torch.randint(0, 120, (Mt, N4), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+                dys8 = torch.randint(118, 128, (Mt, N4 // 128), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+                dx = torch.empty(Mt, K4, dtype=torch.bfloat16, device=dev)
+                fnn = lambda: chk(L.lp_gemm_fp8_grouped_nn(dyq.data_ptr(), dys8.data_ptr(), w4q.data_ptr(), w4s8.data_ptr(), A.E8M0,  # noqa: E731
+                                                           offs_d.data_ptr(), E4, Mt, K4, N4, dx.data_ptr(), A.BF16, stream()))
+                ms_nn, _ = time_launches([fnn], 5, 2)
+                wT = torch.empty(E4, K4, N4, dtype=torch.uint8, device=dev)
+                wsT = torch.empty(E4, K4 // 128, N4 // 128, dtype=torch.uint8, device=dev)
+
+                def f_transposed():
+                    wT.copy_(w4q.view(E4, N4, K4).transpose(1, 2))
+                    wsT.copy_(w4s8.view(E4, N4 // 128, K4 // 128).transpose(1, 2))
+                    chk(L.lp_gemm_fp8_grouped(dyq.data_ptr(), dys8.data_ptr(), wT.data_ptr(), wsT.data_ptr(), A.E8M0,
+                                              offs_d.data_ptr(), E4, Mt, K4, N4, dx.data_ptr(), A.BF16, stream()))
+                ms_tr, _ = time_launches([f_transposed], 3, 1)
+                fl_d = 2.0 * Mt * N4 * K4
+                dgrad_res = {"ms": ms_nn, "tflops": fl_d / ms_nn / 1e9, "mfma_frac": fl_d / ms_nn / 1e9 / FP8_PEAK_TFLOPS,
+                             "over_forward_gate_up_e8m0": ms_nn / ms48,
+                             "with_a_transposed_copy_of_the_weights_ms": ms_tr,
+                             "kernel": "gemm_asm_grouped_mixed<true, true>: weights read as stored [4096, 7168], operand turned by ds_read_b64_tr_b8"}
+                del dyq, dys8, dx, wT, wsT
             del x4q, x4s, w4q, w4s, c4, x4s8, w4s8
             torch.cuda.empty_cache()
         extras["c4_grouped_gemm"] = res4
@@ -596,6 +621,7 @@ def main():
         flg = 2.0 * 4096 * 7168 * pbw * 128
         del aT, bT, saT, sbT, dW, tabs
         extras["grouped_linear_backward"] = {
+            "dgrad_grouped_256_experts_65536x4096_to_7168": dgrad_res,
             "wgrad_grouped_256_experts_4096x7168": {"ms": msg, "rows_padded_to": padw, "tflops_on_padded_rows": flg / msg / 1e9,
                                                     "mfma_frac": flg / msg / 1e9 / FP8_PEAK_TFLOPS,
                                                     "output_GB": E4 * 4096 * 7168 * 2 / 1e9,

@@ -97,6 +97,9 @@ bool mid_asm_ok(const void *As, const void *Bs, int scale_dtype, int64_t M, int6
 int launch_mid_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                    int64_t K, void *C, int64_t ldc, int out_dtype, hipStream_t st);
 bool big_grouped_ok(const void *As, const void *Bs, int scale_dtype, int64_t M_total, int64_t N, int64_t K);
+bool grouped_nn_ok(const void *As, const void *Bs, int scale_dtype, int E, int64_t M_total, int64_t N, int64_t K);
+int launch_grouped_nn(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,
+                      int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype, hipStream_t st);
 int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
                        const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype,
                        hipStream_t st);

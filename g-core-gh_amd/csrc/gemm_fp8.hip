@@ -596,6 +596,24 @@ extern "C" int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *B
     return check_launch("lp_gemm_fp8_grouped");
 }
 
+extern "C" int lp_gemm_fp8_grouped_nn(const void *Aq, const void *As, const void *Wq, const void *Ws, int scale_dtype,
+                                      const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C,
+                                      int out_dtype, lp_stream_t stream)
+{
+    LP_REQUIRE(E >= 0, "lp_gemm_fp8_grouped_nn: negative expert count");
+    int rc = check_gemm_args("lp_gemm_fp8_grouped_nn", Aq, As, Wq, Ws, scale_dtype, M_total, N, K, C, out_dtype);
+    if (rc) return rc > 0 ? LP_OK : rc;
+    if (E == 0) return LP_OK;
+    LP_REQUIRE(m_offsets, "lp_gemm_fp8_grouped_nn: null m_offsets");
+    LP_REQUIRE(scale_dtype == LP_E8M0, "lp_gemm_fp8_grouped_nn: power-of-two (LP_E8M0) scales only");
+    if (!gemm::grouped_nn_ok(As, Ws, scale_dtype, E, M_total, N, K))
+        return fail(LP_ERR_UNSUPPORTED,
+                    "lp_gemm_fp8_grouped_nn: needs N %% 512 == 0, K %% 512 == 0, 4-byte aligned scale tables, at most 512 experts and "
+                    "operands below 4 GiB (got E=%d M=%lld N=%lld K=%lld): transpose the weights and call lp_gemm_fp8_grouped",
+                    E, (long long)M_total, (long long)N, (long long)K);
+    return gemm::launch_grouped_nn(Aq, As, Wq, Ws, m_offsets, E, M_total, N, K, C, out_dtype, (hipStream_t)stream);
+}
+
 // ---------------------------------------------------------------------------------------------
 // lp_gemm_fp8_block for callers that cannot allocate device memory: the K-split partial sums go to a buffer that is
 // part of the library's device image instead of a caller workspace.  Each GPU the process uses holds its own copy

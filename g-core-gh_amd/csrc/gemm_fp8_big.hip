@@ -48,6 +48,11 @@ constexpr int THREADS = 512;
 __device__ __forceinline__ int lds_row(int r) { return (r & ~15) | ((r & 7) << 1) | ((r >> 3) & 1); }
 __device__ __forceinline__ int tile_row(int p) { return (p & ~15) | ((p >> 1) & 7) | ((p & 1) << 3); }
 __device__ __forceinline__ int swz(int r, int chunk) { return chunk ^ (r & 7); }
+// Weights stored [K, N]: a stage holds 128 contraction rows of 256 bytes; chunk c (16 columns) of row k sits in slot
+// c ^ nn_swz(k).  ds_read_b64_tr_b8 takes, per 16 lanes, 8 consecutive rows of one chunk (lane pairs on its two halves):
+// the low three bits spread those rows over the 8 slots of a 128-byte half, bit 5 of the row puts the four 16-lane
+// groups of an instruction (rows 32 apart) alternately on the two halves (measured conflict free).
+__device__ __forceinline__ int nn_swz(int k) { return (k & 7) | (((k >> 5) & 1) << 3); }
 
 // NB = 16-column blocks per wave; TN = 2 * 16 * NB
 template <int SDT, int NB>
@@ -223,6 +228,13 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bs_u), [bsptr2] "s"(bs2_u), [m0base] "s"(m0base), \
         [trips] "s"(trips), [flags] "s"(flags), [splitnb] "s"(splitnb), [bextra] "s"(bextra), [bstride] "s"(bstride),       \
         [g4] "s"(g4), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
+#define LP_ASM_INPUTS_NN                                                                                                  \
+    [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
+        [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
+        [ard0] "v"(ard0), [ard1] "v"(ard1), [brdn0] "v"(brdn[0]), [brdn1] "v"(brdn[1]), [brdn2] "v"(brdn[2]),             \
+        [brdn3] "v"(brdn[3]), [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u), [bsptr] "s"(bsn_u),                    \
+        [m0base] "s"(m0base), [trips] "s"(trips), [flags] "s"(flags), [bsstride] "s"(bsstride), [bsbfe] "s"(bsbfe),       \
+        [bstep] "s"(bstep), [amask0] "s"(amask[0]), [amask1] "s"(amask[1]), [amask2] "s"(amask[2]), [amask3] "s"(amask[3])
 #define LP_ASM_INPUTS                                                                                                     \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [boff1] "v"(boff[1]), [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [soff] "v"(soff), [srd] "v"(srd),               \
@@ -300,7 +312,7 @@ struct AsmTile {
 // check_asm_operands.py verifies both on the generated assembly at build time.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false, int WN = 2>
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false, int WN = 2, bool NN = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
@@ -308,6 +320,10 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     using T = AsmTile<TM, TN, KSUB, NST, WN>;
     constexpr int WAVES = T::WAVES, NBW = T::NBW;
     static_assert(WN == 2 || (WN == 4 && TM == 128 && TN == 256 && KSUB == 1 && !DUAL && NST == 3 && !BROW), "four waves along N: the 128 x 256 tile, three stages");
+    // NN: Bq is the weight as stored for C = A W, [K, N] row-major (row pitch N), Bs its [K / 128, N / 128] scale bytes:
+    // the 256-row and the flat tile with e8m0 scales (the data gradient of the grouped linear)
+    static_assert(!NN || (HWS && TN == 256 && KSUB == 1 && !DUAL && !BROW && ((TM == 256 && WN == 2 && NST == 2) || (TM == 128 && WN == 4 && NST == 3))),
+                  "weights stored [K, N]: hardware-scaled 256 x 256 and 128 x 256 tiles");
     static_assert(!DUAL || (TM == 128 && TN == 128), "the K split inside a workgroup is built for the 128 x 128 tile");
     static_assert(NST == 2 || (NST == 3 && WN == 4) || (NST == 4 && TM == 128 && TN == 128 && KSUB == 1 && !DUAL), "three stages: flat tile, four: 128 x 128 tile");
     static_assert(!BROW || (HWS && TM == 128 && TN == 128 && KSUB == 1 && !DUAL && NST == 2), "row-scaled weights: hardware-scaled 128 x 128 loop");
@@ -354,6 +370,12 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         const int64_t n = n0 + row < N ? n0 + row : N - 1;          // i = 3 is unused when there are three copies
         aoff[i] = (uint32_t)(m * K + swz(row, ld_slot) * 16);
         boff[i] = (uint32_t)(n * K + swz(row, ld_slot) * 16);
+        if constexpr (NN) {
+            // a copy moves 4 contraction rows of 256 bytes: lane -> row 4 (wave + WAVES i) + lane / 16 of the K step,
+            // slot lane % 16, which holds chunk slot ^ nn_swz(row) of the row (columns n0 + 16 chunk ..)
+            const int krow = 4 * (wave + WAVES * i) + (lane >> 4);
+            boff[i] = (uint32_t)((int64_t)krow * N + n0 + (((lane & 15) ^ nn_swz(krow)) << 4));
+        }
     }
     (void)NBC;
     // activation scales travel in groups of four K steps through LDS: the first TM / 64 waves copy one row per lane
@@ -410,6 +432,24 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t ard1 = lds0 + lds_row(arow_l) * KB + swz(arow_l, 2 * lq + 1) * 16;
     const uint32_t brd0 = lds0 + T::B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq) * 16;
     const uint32_t brd1 = lds0 + T::B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq + 1) * 16;
+    // NN: fragment address per block of 16 columns: lane 16 q + s of a transposing read points at half s & 1 of chunk
+    // (wn NBW + b) of contraction row 32 q + s / 2 (+ 8 per instruction of the fragment, in the offset field)
+    uint32_t brdn[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (NN) {
+        const int krow = 32 * lq + (l16 >> 1);
+#pragma unroll
+        for (int b = 0; b < NBW; ++b)
+            brdn[b] = lds0 + T::B_LDS + krow * 256 + (((wn * NBW + b) ^ nn_swz(krow)) << 4) + 8 * (l16 & 1);
+    }
+    // NN: the wave's weight scales are column (n0 + its first column) / 128 of the [K / 128, N / 128] byte table, one row per
+    // K step: the loop loads the aligned dword around each byte (rows are a multiple of 4 bytes apart, checked on the
+    // host, so the byte's place in the dword is the same for every step)
+    const uint64_t bsn_addr = (uint64_t)(uintptr_t)Bs + (uint64_t)(wcol0 >> 7);
+    const uint64_t bsn_u = uniform((const void *)(uintptr_t)(bsn_addr & ~(uint64_t)3));
+    const uint32_t bsbfe = __builtin_amdgcn_readfirstlane((uint32_t)((bsn_addr & 3) * 8) | (8u << 16));
+    const uint32_t bsstride = __builtin_amdgcn_readfirstlane((uint32_t)(N >> 7));
+    const uint32_t bstep = __builtin_amdgcn_readfirstlane((uint32_t)(128 * N));
+    (void)bsn_u; (void)bsbfe; (void)bsstride; (void)bstep;
     // scale staging: 16 bytes per activation row (fp32, four K steps), or 4 bytes per row in 1 KB per copying wave (e8m0)
     const uint32_t srd = HWS ? lds0 + T::S_LDS + wm * 1024 + l16 * 4 : lds0 + T::S_LDS + arow_l * 16;
     // row-scaled weights: their dwords live behind the two activation halves, 1 KB per copying wave like those
@@ -440,6 +480,24 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4;
         accs[5] = acc5; accs[6] = acc6; accs[7] = acc7; accs[8] = acc8;
+    } else if constexpr (NN && WN == 4) {
+        f32x16v acc0, acc1, acc2, acc3;
+        asm volatile(
+#include "gemm_flat_hw_nn_loop.inc"
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3)
+            : LP_ASM_INPUTS_NN
+            : LP_ASM_CLOBBERS, "s64", "s65", "s66", "s89", "s90", "s91", "s92");
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+    } else if constexpr (NN) {
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
+        asm volatile(
+#include "gemm_big_hw_nn_loop.inc"
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
+            : LP_ASM_INPUTS_NN, [brdn4] "v"(brdn[4]), [brdn5] "v"(brdn[5]), [brdn6] "v"(brdn[6]), [brdn7] "v"(brdn[7])
+            : LP_ASM_CLOBBERS, "s64", "s65", "s66");
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+        accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
     } else if constexpr (WN == 4) {
         // the early hand-back of this loop splits the weight copies by wave: the first four copy each wave column's first half
         f32x16v acc0, acc1, acc2, acc3;
@@ -824,7 +882,9 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm_grouped(const uint8_t *__rest
 // be re-used out of one L2.
 constexpr int kMixedMaxExperts = 512;
 
-template <bool HWS>
+// NN: expert e's weight is stored [K, N] (the layer's own [out, in] weight read for the data gradient dX = dY W: K = out
+// features = the contraction, N = in features = the columns of C), its scale bytes [K / 128, N / 128].
+template <bool HWS, bool NN = false>
 __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                               const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
                                                               const int32_t *__restrict__ m_offsets, int E, int64_t M_total,
@@ -962,9 +1022,9 @@ __global__ __launch_bounds__(512) void gemm_asm_grouped_mixed(const uint8_t *__r
             const uint8_t *bq_e = Bq + (int64_t)e * N * K;
             __syncthreads();                            // every wave is done with the previous tile's use of the stage memory
             if (ex >> 30)
-                tile_asm<256, 256, 1, HWS, false, 2, false, true>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
+                tile_asm<256, 256, 1, HWS, false, 2, false, true, 2, NN>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
             else
-                tile_asm<128, 256, 1, HWS, false, 3, false, true, 4>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
+                tile_asm<128, 256, 1, HWS, false, 3, false, true, 4, NN>(smem, Aq, As, bq_e, bs_e, m0, row_end, n0, N, K, C, N, out_dtype);
         }
     }
 }
@@ -1232,6 +1292,26 @@ static int compute_units()
         cached[dev] = n > 0 ? n : -1;
     }
     return cached[dev] > 0 ? cached[dev] : 0;
+}
+
+// The data gradient of the grouped linear on the stored weights (no transposed copy): e8m0 scales, N a multiple of 256,
+// K of 512, the scale table's rows a multiple of 4 bytes apart and 4-byte aligned, at most kMixedMaxExperts experts.
+bool grouped_nn_ok(const void *As, const void *Bs, int scale_dtype, int E, int64_t M_total, int64_t N, int64_t K)
+{
+    return scale_dtype == LP_E8M0 && E <= kMixedMaxExperts && N % 256 == 0 && (N / 128) % 4 == 0 && ((uintptr_t)Bs & 3) == 0 &&
+           asm_shape_ok(As, Bs, M_total, N, K, LP_E8M0);
+}
+
+int launch_grouped_nn(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *m_offsets, int E,
+                      int64_t M_total, int64_t N, int64_t K, void *C, int out_dtype, hipStream_t st)
+{
+    int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;
+    if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_grouped_nn: problem too large");
+    const int cus = compute_units();
+    if (cus >= 8 && grid > cus) grid = cus / 8 * 8;            // one workgroup per CU walks the tile slots, as in the forward launch
+    hipLaunchKernelGGL((gemm_asm_grouped_mixed<true, true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq,
+                       (const float *)As, (const uint8_t *)Bq, (const float *)Bs, m_offsets, E, M_total, N, K, C, out_dtype, 4);
+    return check_launch("lp_gemm_fp8_grouped_nn");
 }
 
 int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,

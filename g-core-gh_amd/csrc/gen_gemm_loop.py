@@ -35,12 +35,12 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False, pingpong=False):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False, pingpong=False, nn=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
-    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP, SPREAD
+    global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP, SPREAD, NN, BF, RBN
     # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
     # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
     WITH_IDLE, IDLE = idle, False
@@ -53,10 +53,25 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # flat 128 x 256 loop of the grouped kernel gains nothing and keeps one body.
     PINGPONG, GRP = pingpong, 0
     HW = hw
+    # nn: the weights are stored with the contraction index as their row index ([K, N] row-major: the data gradient of a
+    # linear layer on the stored weight, C = A W).  A stage then holds 128 contraction rows of tn bytes each, copied as
+    # stored (a copy instruction moves 4 rows of 256 bytes), and the matrix instruction's weight operand -- 32
+    # consecutive contraction bytes of one column per lane -- is gathered by ds_read_b64_tr_b8, which hands lane
+    # (i, p) of every 16 the bytes i of the eight 8-byte rows 2 j + p that the 16 lanes address: with lane pairs on
+    # the two halves of 16 bytes of one contraction row, eight rows per instruction, a lane receives column i + 8 p
+    # of 8 consecutive contraction rows, and four instructions fill the 32 bytes of a K step.  Every block of 16
+    # columns has its own address register (the 16-byte chunks of a row are XOR-swizzled by the row, so a block is not
+    # an offset away from the next).  All of a stage's weight rows are read until the end of a step: the early
+    # hand-back returns the activation rows only, every weight copy waits for the end of the step.  The weight scale
+    # of a K step is one byte of a row of the [K / 128, N / 128] table: four strided loads per group, put together
+    # with scalar instructions.  Hardware-scaled loops only.
+    NN = nn
+    assert not nn or (hw and early and not wide and not brow and ksub == 1 and tn == 256)
+    BF = 4 if nn else 2                                    # LDS instructions per weight fragment
     # A wave column of 64 weight rows is one copy of eight waves: its first half (the 32 rows the first two blocks read)
     # is then what waves 0 .. 3 copy and its second half what waves 4 .. 7 copy, so the early hand-back splits the
     # weight copies by wave (s87 = 1 for the first half of the waves) instead of by copy index.
-    HALFSPLIT = early and tn // waves_n == 64 and waves_m * waves_n == 8
+    HALFSPLIT = early and tn // waves_n == 64 and waves_m * waves_n == 8 and not nn
     # one copy behind each matrix instruction instead of runs of copies (see dma_chunks); the flat tile, whose weight
     # copies are split by wave behind one branch, keeps its runs
     SPREAD = early and not HALFSPLIT and SPREAD_ON
@@ -104,6 +119,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     SCL_LDS = nstage * ksub * (A_BYTES + B_BYTES)          # activation-scale buffer: 2 halves x tm rows x 16 bytes
     SCL_HALF = tm * 16        # (the e8m0 variant uses 4 of every 16 bytes: one wave writes 64 rows x 4 bytes per KB)
     NB = tn // waves_n // 16
+    RBN = [f"v{96 + b}" for b in range(NB)]               # nn: fragment read address of block b (the fp32 loops' result registers are free)
     # a wave whose columns are not a multiple of 128 wide can straddle two weight-scale blocks: two scale rows
     # are loaded and each pair of 16-column blocks takes the one the set-up code selected for it
     SPLIT = (tn // waves_n) % 128 != 0 and (tn // waves_n) > 64 and not wide
@@ -184,6 +200,9 @@ def dma(stage, part="all"):
             if WIDE:
                 if part != "all" and WIDE_PART[i] != part:
                     continue
+            elif NN:
+                if part == "mid":
+                    continue
             elif not HALFSPLIT and ((part == "mid" and i % 2) or (part == "end" and i % 2 == 0)):
                 continue
             partial = WIDE and (i + 1) * WAVES * 1024 > B_BYTES       # only the first waves have rows left for this copy
@@ -216,7 +235,7 @@ def dma(stage, part="all"):
         if part in ("all", "end"):
             for i in range(ncopies if WIDE else 1):
                 lo = int(WB_EXTRA[i][2:4])
-                emit(f"s_add_u32 s{lo}, s{lo}, 128")
+                emit(f"s_add_u32 s{lo}, s{lo}, {'s66' if NN else 128}")      # nn: 128 rows of the stored weight further on
                 emit(f"s_addc_u32 s{lo + 1}, s{lo + 1}, 0")
 
 
@@ -260,6 +279,8 @@ def emit_piece(piece, tag, cond):
 def copies_per_part():
     """Requests of one wave in the mid-step part and in the end-of-step part of a stage (early hand-back)."""
     a, b = A_BYTES // 1024 // WAVES, B_BYTES // 1024 // WAVES
+    if NN:
+        return a, b
     if WIDE:
         # waves 0 .. 3 issue a third request in the end part; counting two makes their waits one request stricter
         return a + 2, 2
@@ -277,7 +298,10 @@ def younger_requests(c, at_end, last_trip):
     issued in the order mid(j), end(j), mid(j + 1) ...; on the last trip a part of step j exists only if the step it
     fills, j + NSTAGE, is still inside the trip (steps of earlier trips, j < 0, always do)."""
     mid, end = copies_per_part()
-    need = ("mid", c - NSTAGE + 1) if at_end else ("end", c - NSTAGE)
+    # nn: every block of a step reads all of the stage's weight rows, so the whole stage -- the activation rows asked for
+    # mid-step and the weight rows asked for at the end of the same step -- must have landed when the step begins: the
+    # end-of-step wait covers both, the mid-step wait has nothing to wait for (wait_copies leaves it out)
+    need = (("end", c - NSTAGE + 1) if NN else ("mid", c - NSTAGE + 1)) if at_end else ("end", c - NSTAGE)
     upto = ("mid", c) if at_end else ("end", c - 1)
     parts = []
     for j in range(need[1], c + 1):
@@ -293,6 +317,9 @@ def wait_copies(c, at_end, extra=""):
     """Early hand-back: wait until the requests this point depends on have landed.  Requests return in order, so it
     is enough to bound how many younger ones may still be out (c = step within the trip, s50 = 1 on the last trip,
     on which nothing is requested for steps past the end)."""
+    if NN and not at_end:
+        emit(f"s_waitcnt{extra}")
+        return
     steady, last = younger_requests(c, at_end, False), younger_requests(c, at_end, True)
     tag = f"{'e' if at_end else 'm'}{c}"
     if last != steady:
@@ -327,6 +354,13 @@ def weight_scale_load():
     """The four weight scales of the next group into s[60:63] (and those of the second scale row into s[68:71])."""
     if BROW:
         return                                            # they travel with the activation scales, see scale_group_copy
+    if NN:
+        # one byte per K step, a table row (s64 bytes) apart: the aligned dword around each, taken apart at the top of the loop
+        for i in range(4):
+            emit(f"s_load_dword s{60 + i}, s[46:47], 0x0")
+            emit("s_add_u32 s46, s46, s64")
+            emit("s_addc_u32 s47, s47, 0")
+        return
     if HW:
         emit("s_load_dword s60, s[46:47], 0x0")          # four e8m0 bytes = four K steps
         emit("s_add_u32 s46, s46, 4")
@@ -348,6 +382,15 @@ def weight_scale_load():
 def read_frag(dst, addr0, addr1, off):
     emit(f"ds_read_b128 {vr(dst, 4)}, {addr0} offset:{off}")
     emit(f"ds_read_b128 {vr(dst + 4, 4)}, {addr1} offset:{off}")
+
+
+def read_bfrag(dst, nb, stage_off):
+    """The weight fragment of block nb (16 columns x 128 bytes of K) into v[dst : dst + 7]."""
+    if NN:
+        for t in range(4):
+            emit(f"ds_read_b64_tr_b8 {vr(dst + 2 * t, 2)}, {RBN[nb]} offset:{stage_off + 2048 * t}")
+    else:
+        read_frag(dst, RB0, RB1, stage_off + nb * 2048)
 
 
 def read_scales(col):
@@ -441,12 +484,12 @@ def step(c):
         if BROW:
             emit(f"v_add_u32 v{SRDB}, s55, v{SRDB0}")
     pieces = []                  # copies waiting for their slot behind a matrix instruction: (piece, tag, skipped on the last trip)
-    read_frag(WFB[par(c, 1)], RB0, RB1, boff + 2048)
-    # LDS queue now: wf0, af0..3, wf1 = 12 reads
+    read_bfrag(WFB[par(c, 1)], 1, boff)
+    # LDS queue now: wf0, af0..3, wf1 = 12 reads (16 with four instructions per weight fragment)
     if PINGPONG:
         emit(f"s_setprio {(c * NB + GRP + 1) & 1}")
     for mb in range(MB):
-        emit(f"s_waitcnt lgkmcnt({8 - 2 * mb})")
+        emit(f"s_waitcnt lgkmcnt({(3 - mb) * 2 + BF})")
         mfma(0, mb, c)
     read_scales((c + 1) & 3)
     for nb in range(1, NB):
@@ -467,14 +510,14 @@ def step(c):
             wait_copies(c, False, " lgkmcnt(0)")
             emit("s_barrier")
         if nb + 1 < NB:
-            read_frag(WFB[par(c, nb + 1)], RB0, RB1, boff + (nb + 1) * 2048)
+            read_bfrag(WFB[par(c, nb + 1)], nb + 1, boff)
         if nb == 1:
             pending = 4 if (not HW or c == 3) else 0                # scale reads issued after block 0
             if BROW and c == 3:
                 pending += NB
-            emit(f"s_waitcnt lgkmcnt({pending + (2 if NB > 2 else 0)})")        # those and wf2 may still be outstanding
+            emit(f"s_waitcnt lgkmcnt({pending + (BF if NB > 2 else 0)})")        # those and wf2 may still be outstanding
         elif nb + 1 < NB:
-            emit("s_waitcnt lgkmcnt(2)")
+            emit(f"s_waitcnt lgkmcnt({BF})")
         if nb + 1 == NB:
             if flip:
                 # every wave has read all of this stage and its share of the next stage has landed
@@ -512,11 +555,15 @@ def step(c):
                     emit("s_cselect_b32 s90, 0, s90")
                     emit(f"v_add_u32 {RA0}, s89, %[ard0]")
                     emit(f"v_add_u32 {RA1}, s89, %[ard1]")
-                    emit(f"v_add_u32 {RB0}, s90, %[brd0]")
-                    emit(f"v_add_u32 {RB1}, s90, %[brd1]")
+                    if NN:
+                        for b in range(NB):
+                            emit(f"v_add_u32 {RBN[b]}, s90, %[brdn{b}]")
+                    else:
+                        emit(f"v_add_u32 {RB0}, s90, %[brd0]")
+                        emit(f"v_add_u32 {RB1}, s90, %[brd1]")
             else:
                 emit("s_waitcnt lgkmcnt(0)")
-            read_frag(WFB[par(c + 1, 0)], RB0, RB1, nboff)
+            read_bfrag(WFB[par(c + 1, 0)], 0, nboff)
         for mb in range(MB):
             mfma(nb, mb, c)
             fold(nb - 1, mb, c)
@@ -573,6 +620,17 @@ def loop_body():
         if BROW:
             for nb in range(NB):
                 emit(f"v_mov_b32 v{WSN + nb}, v{WSC + nb}")
+        elif NN:
+            # byte (address & 3) of each of the four dwords -> the four scale bytes of this group in one register
+            for i in range(4):
+                emit(f"s_bfe_u32 s{60 + i}, s{60 + i}, s65")
+            emit("s_lshl_b32 s61, s61, 8")
+            emit("s_lshl_b32 s62, s62, 16")
+            emit("s_lshl_b32 s63, s63, 24")
+            emit("s_or_b32 s60, s60, s61")
+            emit("s_or_b32 s62, s62, s63")
+            emit("s_or_b32 s60, s60, s62")
+            emit(f"v_mov_b32 {WS1}, s60")
         else:
             emit(f"v_mov_b32 {WS1}, s60")
             if WIDE:
@@ -630,8 +688,16 @@ def generate():
     emit("s_mov_b32 s54, 0")
     emit("s_mov_b32 s55, 0")
     for reg, name in ((RA0, "ard0"), (RA1, "ard1"), (RB0, "brd0"), (RB1, "brd1"), (SRD0, "srd"), (SRD, "srd")):
+        if NN and name.startswith("brd"):
+            continue
         if not reg.startswith("%"):
             emit(f"v_mov_b32 {reg}, %[{name}]")
+    if NN:
+        for b in range(NB):
+            emit(f"v_mov_b32 {RBN[b]}, %[brdn{b}]")
+        emit("s_mov_b32 s64, %[bsstride]")                 # bytes between two rows of the weight-scale table
+        emit("s_mov_b32 s65, %[bsbfe]")                    # s_bfe_u32 operand: 8 bits from bit 8 * (table address & 3)
+        emit("s_mov_b32 s66, %[bstep]")                    # bytes between two K steps of the stored weight
     if BROW:
         emit("s_mov_b32 s51, %[sdst]")
         emit(f"v_mov_b32 v{SRDB0}, %[srdb]")
@@ -675,7 +741,7 @@ def generate():
         for nb in range(NB):
             emit(f"ds_read_b32 v{WSC + nb}, v{SRDB} offset:{nb * 64}")
     emit("s_waitcnt lgkmcnt(0)")
-    read_frag(WFB[0], RB0, RB1, 0)
+    read_bfrag(WFB[0], 0, 0)
     for mb in range(MB):
         read_frag(AF + 8 * mb, RA0, RA1, mb * 2048)
     # ---- main loop: one trip = four K steps = one group of scales
@@ -724,7 +790,9 @@ def main():
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
                       ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
-                      ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True, True))):
+                      ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True, True)),
+                      ("gemm_big_hw_nn_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True, PP, True)),
+                      ("gemm_flat_hw_nn_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True, False, True))):
         configure(*cfg)
         generate()
         write(here, name)

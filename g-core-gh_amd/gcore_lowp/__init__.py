@@ -14,7 +14,8 @@ from .dsv4_kernels import (  # noqa: F401
 )
 from .mygemm_fp8 import gemm_fp8_block_scaling_impl, gemm_impl  # noqa: F401
 from .grouped_gemm_fp8 import (  # noqa: F401
-    MyTeGroupedLinearFp8, gemm_fp8_rowscale, gemm_fp8_rowscale_grouped, grouped_gemm_fp8, m_grouped_gemm_fp8_fp8_bf16_nt_contiguous,
+    MyTeGroupedLinearFp8, gemm_fp8_rowscale, gemm_fp8_rowscale_grouped, grouped_gemm_fp8, grouped_gemm_fp8_nn,
+    m_grouped_gemm_fp8_fp8_bf16_nt_contiguous,
     quant_fp8_colwise_t,
 )
 from .fp8_tensor import Fp8TensorAg, Fp8TensorTrain  # noqa: F401

@@ -46,6 +46,7 @@ PROTOTYPES = {
     "lp_gemm_fp8_rowscale_grouped": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _i32, _i32, _i64, _i64, _p, _i32, _p]),
     "lp_quant_fp8_colwise_t": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _i64, _i32, _p, _p, _i32, _p]),
     "lp_gemm_fp8_grouped": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
+    "lp_gemm_fp8_grouped_nn": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _i32, _p]),
     "lp_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
 }
 

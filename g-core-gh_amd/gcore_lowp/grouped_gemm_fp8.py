@@ -13,8 +13,8 @@ import torch
 from . import _abi as A
 from . import ops
 
-__all__ = ["grouped_gemm_fp8", "m_grouped_gemm_fp8_fp8_bf16_nt_contiguous", "MyTeGroupedLinearFp8", "quant_fp8_colwise_t",
-           "gemm_fp8_rowscale"]
+__all__ = ["grouped_gemm_fp8", "grouped_gemm_fp8_nn", "m_grouped_gemm_fp8_fp8_bf16_nt_contiguous", "MyTeGroupedLinearFp8",
+           "quant_fp8_colwise_t", "gemm_fp8_rowscale"]
 
 
 def _scale_arg(s, dev):
@@ -37,8 +37,10 @@ def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor 
     """xq [M,K] e4m3fn, xs [M,K/128], wq [E,N,K] e4m3fn, ws [E,N/128,K/128],
     m_offsets integer [E+1] (rows of expert e: m_offsets[e]..m_offsets[e+1]-1, non-decreasing from 0, last <= M).
     Rows at or beyond m_offsets[E] belong to no expert: a freshly allocated `out` has them zeroed, a caller's `out`
-    keeps them.  total_rows: m_offsets[E] when the caller knows it on the host (saves reading it back);
-    validate: check the offsets on the host (one device read-back)."""
+    keeps them.  A table that breaks the contract (does not start at 0, decreases) leaves the rows that fall outside
+    every expert's range of a freshly allocated `out` undefined.  total_rows: m_offsets[E] when the caller knows it on
+    the host (saves reading it back); validate: check the offsets, and total_rows against them, on the host (one device
+    read-back)."""
     M, K = xq.shape
     E, N, K2 = wq.shape
     assert K == K2 and K % 128 == 0 and N % 128 == 0
@@ -54,6 +56,8 @@ def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor 
         o = offs.cpu()
         if int(o[0]) != 0 or bool((o[1:] < o[:-1]).any()) or int(o[-1]) > M:
             raise ValueError(f"grouped_gemm_fp8: m_offsets must start at 0, never decrease and end at or below M = {M}")
+        if total_rows is not None and E > 0 and int(o[-1]) != total_rows:
+            raise ValueError(f"grouped_gemm_fp8: total_rows = {total_rows} but m_offsets ends at {int(o[-1])}")
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=dev)
         if total_rows is None:
@@ -66,6 +70,42 @@ def grouped_gemm_fp8(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor 
             xq.contiguous().data_ptr(), sa.data_ptr(), wq.contiguous().data_ptr(), sb.data_ptr(), ca,
             offs.data_ptr(), E, M, N, K, out.data_ptr(),
             A.BF16 if out.dtype == torch.bfloat16 else A.F32, A.stream_ptr()))
+    return out
+
+
+def grouped_gemm_fp8_nn(xq, xs, wq, ws, m_offsets: torch.Tensor, out: torch.Tensor | None = None,
+                        out_dtype=torch.bfloat16, total_rows: int | None = None) -> torch.Tensor:
+    """out_e = x_e W_e on weights stored [E, K, N] (K = the contraction): the data gradient of the grouped linear on the
+    layer's own [out, in] weights, general_grouped_gemm(..., layout="NN") at gpatch_v4/models/deepseek_v4/fp8.py:301-313.
+    xq [M, K] e4m3fn with xs [M, K/128], wq [E, K, N] e4m3fn with ws [E, K/128, N/128], all scales e8m0.
+    The kernel turns the weight operand while it reads it out of LDS; shapes it does not take (N or K not a multiple of
+    512, more than 512 experts) go through a transposed copy of the weights and grouped_gemm_fp8."""
+    M, K = xq.shape
+    E, K2, N = wq.shape
+    assert K == K2 and K % 128 == 0 and N % 128 == 0
+    assert tuple(xs.shape) == (M, K // 128) and tuple(ws.shape) == (E, K // 128, N // 128)
+    assert xs.dtype == ops.E8M0 and ws.dtype == ops.E8M0, "grouped_gemm_fp8_nn: power-of-two (e8m0) scales"
+    dev = xq.device
+    assert dev.type == "cuda", "grouped_gemm_fp8_nn takes GPU tensors"
+    offs = _check_offsets(m_offsets, E, dev, "grouped_gemm_fp8_nn")
+    fresh = out is None
+    if fresh:
+        out = torch.empty((M, N), dtype=out_dtype, device=dev)
+        if total_rows is None:
+            total_rows = int(offs[-1].item()) if E > 0 else 0
+        if total_rows < M:
+            out[total_rows:].zero_()
+    assert out.is_contiguous() and tuple(out.shape) == (M, N) and out.dtype in (torch.bfloat16, torch.float32)
+    wqc, wsc, xsc = wq.contiguous(), ws.contiguous(), xs.contiguous()
+    with torch.cuda.device(dev):
+        rc = A.lib().lp_gemm_fp8_grouped_nn(
+            xq.contiguous().data_ptr(), xsc.data_ptr(), wqc.data_ptr(), wsc.data_ptr(), A.E8M0, offs.data_ptr(), E, M, N, K,
+            out.data_ptr(), A.BF16 if out.dtype == torch.bfloat16 else A.F32, A.stream_ptr())
+    if rc == -2:            # LP_ERR_UNSUPPORTED: a shape the transposing-read kernel does not take
+        wt = wqc.view(torch.uint8).transpose(1, 2).contiguous().view(ops.E4M3)
+        wst = wsc.view(torch.uint8).transpose(1, 2).contiguous().view(ops.E8M0)
+        return grouped_gemm_fp8(xq, xs, wt, wst, offs, out=out)
+    A.check(rc)
     return out
 
 
@@ -178,8 +218,9 @@ def _offsets(m_splits, dev):
 class _GroupedGemmFp8(torch.autograd.Function):
     """gpatch_v4/models/deepseek_v4/fp8.py:180-343 without TransformerEngine, Float8BlockScaling with power-of-two
     scales: forward y_e = x_e W_e^T on 1 x 128 activations and 128 x 128 weights; backward
-      dgrad  dx_e = dY_e W_e      (layout NN): dY quantised 1 x 128 along N, the weight's codes and scales transposed
-                                  (a 128 x 128 block scaling is its own transpose);
+      dgrad  dx_e = dY_e W_e      (layout NN): dY quantised 1 x 128 along N, on the stored weight codes and scales: the
+                                  kernel turns the weight operand while it reads it out of LDS (a 128 x 128 block
+                                  scaling is its own transpose, its table is read by column); no transposed copy;
       wgrad  dW_e = dY_e^T X_e    (layout NT over column-wise operands): dY and X quantised per (column, 128 rows of
                                   the expert), transposed, all experts' row-scaled GEMMs in one launch (two when some experts'
                                   padded row counts are not multiples of 512) straight into dW.
@@ -215,10 +256,8 @@ class _GroupedGemmFp8(torch.autograd.Function):
         dgrad = wgrad = None
         if ctx.need_dgrad:
             dyq, dys = quant_fp8_e4m3_scale_e8m0(dy, block_size=(1, 128))
-            wt = wq.transpose(1, 2).contiguous().view(ops.E4M3)
-            wst = ws.transpose(1, 2).contiguous().view(ops.E8M0)
-            dgrad = grouped_gemm_fp8(dyq, dys, wt, wst, offs, out_dtype=ctx.out_dtype,
-                                     total_rows=sum(ctx.m_splits)).view(ctx.inp_shape)
+            dgrad = grouped_gemm_fp8_nn(dyq, dys, wq.view(ops.E4M3), ws.view(ops.E8M0), offs, out_dtype=ctx.out_dtype,
+                                        total_rows=sum(ctx.m_splits)).view(ctx.inp_shape)
         if ctx.need_wgrad:
             xtq, xts = ctx.saved_tensors[3:5]
             dtq, dts, nblk = quant_fp8_colwise_t(dy, offs, ctx.m_splits, ctx.pad_rows)       # padded like X^T in the forward

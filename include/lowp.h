@@ -267,6 +267,20 @@ int lp_gemm_fp8_grouped(const void *Aq, const void *As, const void *Bq, const vo
                         void *C, int out_dtype, lp_stream_t stream);
 
 /*
+ * The same grouped GEMM on weights stored for the other product: C_e = A_e W_e with W [E,K,N] row-major (K = the
+ * contraction) and its 128 x 128 scales Ws [E,K/128,N/128], scales e8m0 on both operands.  This is the data gradient
+ * of the grouped linear, dX_e = dY_e W_e on the layer's own [out, in] weight (K = out features, N = in features),
+ * without a transposed copy of the weights: the matrix cores' operand is turned while it is read out of LDS.
+ * Aq [M_total,K], As [M_total,K/128] (dY quantised 1 x 128 along K), C [M_total,N].  Needs N % 512 == 0, K % 512 == 0,
+ * Ws 4-byte aligned, E <= 512; LP_ERR_UNSUPPORTED otherwise (transpose and call lp_gemm_fp8_grouped).
+ * Replaces the dgrad of _MyTeGroupedLinear.backward, general_grouped_gemm(..., layout="NN")
+ * (gpatch_v4/models/deepseek_v4/fp8.py:301-313).
+ */
+int lp_gemm_fp8_grouped_nn(const void *Aq, const void *As, const void *Wq, const void *Ws, int scale_dtype,
+                           const int32_t *m_offsets, int E, int64_t M_total, int64_t N, int64_t K, void *C,
+                           int out_dtype, lp_stream_t stream);
+
+/*
  * Block-scaled FP8 GEMM with a scale per row and 128-wide K group on BOTH operands:
  * C[m, n] = sum_kb (Aq[m, kb] . Bq[n, kb]) * As[m, kb] * Bs[n, kb], Bs [N, K/128].
  * Same shapes, dtypes and checks as lp_gemm_fp8_block otherwise.  This is the weight-gradient GEMM of

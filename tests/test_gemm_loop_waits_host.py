@@ -19,6 +19,9 @@ LOOPS = {
     "big 256x256": ((256, 256, 4, 2, 1, False, 2, False, True), [(4 + 2, 2)]),
     "wide 256x288": ((256, 288, 4, 2, 1, False, 2, False, True, True), [(4 + 2, 3), (4 + 2, 2)]),        # waves 0..3 copy a fifth group
     "flat 128x256, three stages": ((128, 256, 2, 4, 1, False, 3, False, True), [(2 + 4, 0), (2, 4)]),    # first / second half of the waves
+    # weights stored [K, N]: the activation rows mid-step, every weight row at the end of the step
+    "big 256x256, weights stored [K, N]": ((256, 256, 4, 2, 1, True, 2, False, True, False, True, True, True), [(4, 4)]),
+    "flat 128x256, three stages, weights stored [K, N]": ((128, 256, 2, 4, 1, True, 3, False, True, False, True, False, True), [(2, 4)]),
 }
 
 
@@ -36,13 +39,20 @@ def test_waits_cover_what_is_read(name, trips):
         for step in range(steps):
             c, last = step % 4, step // 4 == trips - 1
             for at_end in (False, True):
-                allowed = gen.younger_requests(c, at_end, last)
+                if gen.NN and not at_end:
+                    needs = []                        # the mid-step wait of these loops waits for no copy
+                    allowed = len(issued)
+                else:
+                    allowed = gen.younger_requests(c, at_end, last)
+                    # weights stored [K, N]: a step reads all of its stage from its first block on, so both parts of the
+                    # next step's stage must have landed at the end of this one
+                    needs = ([("mid", step + 1), ("end", step + 1)] if gen.NN else [("mid", step + 1)]) if at_end else [("end", step)]
                 landed = issued[:len(issued) - allowed] if allowed else issued
-                need = ("mid", step + 1) if at_end else ("end", step)
-                if need[1] < steps:
-                    n_need = sum(1 for r in issued if r == need)
-                    assert n_need == (mid if need[0] == "mid" else end)
-                    assert sum(1 for r in landed if r == need) == n_need, (name, step, at_end, allowed)
+                for need in needs:
+                    if need[1] < steps:
+                        n_need = sum(1 for r in issued if r == need)
+                        assert n_need == (mid if need[0] == "mid" else end)
+                        assert sum(1 for r in landed if r == need) == n_need, (name, step, at_end, allowed)
                 # after the wait and the barrier this wave requests the freed part for the step nst ahead
                 if step + nst < steps:
                     issued += [("mid" if not at_end else "end", step + nst)] * (mid if not at_end else end)

@@ -420,6 +420,52 @@ def test_gemm_rowscale_grouped_equals_per_problem_launches(G, out_dtype):
         before += kb
 
 
+@pytest.mark.parametrize("case", [([300, 0, 128, 1, 77, 513], 512, 512), ([2048, 16, 700], 1024, 2048), ([64, 64, 64, 64], 2048, 512),
+                                  ([1000, 5, 0, 260, 129], 512, 4096)],
+                         ids=lambda c: "E%d_N%d_K%d" % (len(c[0]), c[1], c[2]))
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_gemm_grouped_nn_equals_transposed_weights(G, case, out_dtype):
+    """The data gradient's GEMM on the stored weights, out_e = x_e W_e with W [E, K, N] (layout NN,
+    gpatch_v4/models/deepseek_v4/fp8.py:301-313): the kernel that turns the weight operand on its way out of LDS gives the
+    bits of the NT kernel on a transposed copy of the weights (same products, same order of accumulation), and both are
+    the fp32 dequantise-then-matmul within the GEMM tolerance."""
+    m_splits, N, K = case
+    E, M = len(m_splits), sum(m_splits)
+    say("grouped NN", m_splits, N, K, out_dtype)
+    g = torch.Generator().manual_seed(N + K + M)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(E, K, N, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    xq, xs = G.quant_fp8_e4m3_scale_e8m0(x, (1, 128))
+    wq, ws = G.quant_fp8_e4m3_scale_e8m0(w, (128, 128))
+    offs = torch.zeros(E + 1, dtype=torch.int32)
+    offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    G.grouped_gemm_fp8_nn(xq, xs, wq, ws, offs.cuda(), out=out)
+    wt = wq.view(torch.uint8).transpose(1, 2).contiguous().view(torch.float8_e4m3fn)
+    wst = ws.view(torch.uint8).transpose(1, 2).contiguous().view(torch.float8_e8m0fnu)
+    want = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    G.grouped_gemm_fp8(xq, xs, wt, wst, offs.cuda(), out=want)
+    assert torch.equal(out.view(torch.int16 if out_dtype == torch.bfloat16 else torch.int32),
+                       want.view(torch.int16 if out_dtype == torch.bfloat16 else torch.int32))
+    xd = T.dequant_act_f32(xq, xs.float())
+    off = 0
+    for e, m in enumerate(m_splits):
+        if m:
+            wd = T.dequant_weight_f32(wq[e], ws[e].float())
+            check(out[off:off + m], xd[off:off + m] @ wd, f"grouped NN expert {e}")
+        off += m
+    # a shape the kernel does not take (N not a multiple of 512) goes through the transposed copy inside the wrapper
+    if N == 512:
+        w2 = w[:, :, :384].contiguous()
+        wq2, ws2 = G.quant_fp8_e4m3_scale_e8m0(w2, (128, 128))
+        got = G.grouped_gemm_fp8_nn(xq, xs, wq2, ws2, offs.cuda(), out_dtype=out_dtype, total_rows=M)
+        off = 0
+        for e, m in enumerate(m_splits):
+            if m:
+                check(got[off:off + m], xd[off:off + m] @ T.dequant_weight_f32(wq2[e], ws2[e].float()), f"grouped NN fallback expert {e}")
+            off += m
+
+
 @pytest.mark.parametrize("m_splits", [[8192, 16, 2048, 256], [32, 1, 2000, 323], [100, 0, 31, 200], [2048, 1024, 0, 4096]],
                          ids=["even", "uneven", "empty", "pad512"])
 def test_grouped_linear_backward(G, m_splits):
