@@ -84,7 +84,7 @@ int64_t skinny_workspace_bytes(int64_t N, int splits);
 int launch_skinny(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                   int64_t K, void *C, int out_dtype, float *ws, int splits, int per, hipStream_t st);
 
-int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int64_t M,
+int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int max_k_blocks, int64_t M,
                                 int64_t N, void *C, int out_dtype, hipStream_t st);
 int launch_nt_unit_scales(const void *A, const void *B, const void *ones, int64_t M, int64_t N, int64_t K, void *C, int out_dtype,
                           hipStream_t st);

@@ -222,14 +222,16 @@ template <int SDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_rowscale_grouped(
     const uint8_t *__restrict__ Aq, const void *__restrict__ As, const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
     int scale_dtype, const int32_t *__restrict__ groups, int64_t M, int64_t N, int64_t tiles_m, int64_t tiles_n, int64_t per_group,
-    void *__restrict__ C, int out_dtype)
+    void *__restrict__ C, int out_dtype, int max_k_blocks)
 {
     __shared__ Smem sm;
     const int64_t g = blockIdx.x / per_group, local = blockIdx.x - g * per_group;
     int64_t tm, tn;
     if (!tile_coords(local, tiles_m, tiles_n, tm, tn)) return;
     const int64_t slot = groups[4 * g], kb = groups[4 * g + 1], before = groups[4 * g + 2];
-    if (kb <= 0) return;
+    // an entry that breaks the caller's promise (more K blocks than max_k_blocks, on which the host checked the operand
+    // sizes; a negative slot or offset) writes nothing
+    if (kb <= 0 || kb > max_k_blocks || slot < 0 || before < 0) return;
     const int64_t ssz = SDT == LP_F32 ? 4 : 1;
     TileArgs ta;
     ta.Aq = Aq + M * 128 * before; ta.As = (const char *)As + M * before * ssz;
@@ -472,16 +474,16 @@ extern "C" int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, cons
     hipStream_t st = (hipStream_t)stream;
     // every problem's K a multiple of 512 (promised by the caller: k_blocks_multiple), e8m0 scales: the hand-scheduled loop
     if (k_blocks_multiple % 4 == 0 && gemm::rowscale_asm_ok(As, Bs, scale_dtype, M, N, (int64_t)max_k_blocks * 128))
-        return gemm::launch_rowscale_grouped_asm(Aq, As, Bq, Bs, groups, G, M, N, C, out_dtype, st);
+        return gemm::launch_rowscale_grouped_asm(Aq, As, Bq, Bs, groups, G, max_k_blocks, M, N, C, out_dtype, st);
     const int64_t tiles_m = M / TM, tiles_n = N / TN;
     const int64_t per_group = padded_grid(tiles_m, tiles_n), grid = per_group * G;
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_rowscale_grouped: problem too large");
     if (scale_dtype == LP_F32)
         hipLaunchKernelGGL(gemm_rowscale_grouped<LP_F32>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype, max_k_blocks);
     else
         hipLaunchKernelGGL(gemm_rowscale_grouped<LP_E8M0>, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
-                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+                           (const uint8_t *)Bq, Bs, scale_dtype, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype, max_k_blocks);
     return check_launch("lp_gemm_fp8_rowscale_grouped");
 }
 
@@ -656,7 +658,9 @@ extern "C" int lp_gemm_fp8_block_static(const void *Aq, const void *As, const vo
     if (rc) return rc > 0 ? LP_OK : rc;
     // Only the K-split pair uses scratch (fp32 partial tiles, every one of them written before the reduction reads
     // it, so the buffer's previous contents never matter and nothing is cleared).
-    const int64_t need = split_bytes(M, N, K);
+    // (decode shapes are served by the single-launch kernels before the K split is considered: no scratch, never refused)
+    static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;
+    const int64_t need = !no_thin && gemm::thin_ok(M, N, K) ? 0 : split_bytes(M, N, K);
     LP_REQUIRE(need <= kStaticScratchBytes,
                "lp_gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of K-split scratch, the built-in buffer holds %lld; "
                "call lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes()",

@@ -790,14 +790,17 @@ __global__ __launch_bounds__(256) void gemm_asm_rowscale_grouped(const uint8_t *
                                                                  const uint8_t *__restrict__ Bq, const float *__restrict__ Bs,
                                                                  const int32_t *__restrict__ groups, int64_t M, int64_t N,
                                                                  int64_t tiles_m, int64_t tiles_n, int64_t per_group,
-                                                                 void *__restrict__ C, int out_dtype)
+                                                                 void *__restrict__ C, int out_dtype, int max_k_blocks)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<128, 128, 1>::LDS_BYTES + 4096];
     const int64_t g = blockIdx.x / per_group, local = blockIdx.x - g * per_group;
     int64_t tm, tn;
     if (!gemm::tile_coords(local, tiles_m, tiles_n, tm, tn)) return;
     const int64_t slot = groups[4 * g], kb = groups[4 * g + 1], before = groups[4 * g + 2];
-    if (kb <= 0) return;
+    // an entry that breaks the caller's promise writes nothing: more K blocks than max_k_blocks (on which the host checked
+    // that the operands fit 32-bit offsets), a count that is not a multiple of four (the loop works in groups of four
+    // K blocks and would silently drop the rest), a negative slot or offset
+    if (kb <= 0 || kb > max_k_blocks || (kb & 3) || slot < 0 || before < 0) return;
     char *c = (char *)C + slot * M * N * (out_dtype == LP_BF16 ? 2 : 4);
     tile_asm<128, 128, 1, true, false, 2, true, true>(smem, Aq + M * 128 * before, (const float *)((const char *)As + M * before),
                                                       Bq + N * 128 * before, (const float *)((const char *)Bs + N * before), tm * 128, M,
@@ -1261,14 +1264,14 @@ int launch_rowscale_asm(const void *Aq, const void *As, const void *Bq, const vo
     return check_launch("lp_gemm_fp8_rowscale(asm)");
 }
 
-int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int64_t M,
+int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int max_k_blocks, int64_t M,
                                 int64_t N, void *C, int out_dtype, hipStream_t st)
 {
     const int64_t tiles_m = (M + 127) / 128, tiles_n = N / 128;
     const int64_t per_group = gemm::padded_grid(tiles_m, tiles_n), grid = per_group * G;
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_rowscale_grouped: problem too large");
     hipLaunchKernelGGL(gemm_asm_rowscale_grouped, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, (const float *)As,
-                       (const uint8_t *)Bq, (const float *)Bs, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype);
+                       (const uint8_t *)Bq, (const float *)Bs, groups, M, N, tiles_m, tiles_n, per_group, C, out_dtype, max_k_blocks);
     return check_launch("lp_gemm_fp8_rowscale_grouped(asm)");
 }
 

@@ -306,6 +306,22 @@ def test_gemm_impl(G, shape, kind):
             assert ((ci - wi).abs() <= 1).float().mean() > 0.9999
 
 
+def test_gemm_impl_compile_and_profiler(G):
+    """gemm_impl.compile(...).get_profiler().do_bench() as the reference's benchmark drives it
+    (tests/test_gfused/test_my_gemm_fp8.py:141-163): a callable fixed to one shape, and a positive latency."""
+    say("gemm_impl.compile / do_bench")
+    k = G.gemm_impl.compile(M=256, N=256, K=512, dtype=torch.float8_e4m3fn, out_dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(5)
+    a = torch.randint(-3, 4, (256, 512), generator=g).float().to(torch.float8_e4m3fn).cuda()
+    b = torch.randint(-3, 4, (256, 512), generator=g).float().to(torch.float8_e4m3fn).cuda()
+    c = k(a, b)
+    assert torch.equal(c.float(), (a.float() @ b.float().T).to(torch.bfloat16).float())        # small integers: exact
+    ms = k.get_profiler().do_bench(warmup=1, rep=2)
+    assert ms > 0.0
+    with pytest.raises(AssertionError):
+        k(a[:128], b)
+
+
 def test_gemm_impl_errors_and_cpu_inputs(G):
     a = torch.randn(64, 256).to(torch.bfloat16)
     b = torch.randn(32, 256).to(torch.bfloat16)
@@ -418,6 +434,18 @@ def test_gemm_rowscale_grouped_equals_per_problem_launches(G, out_dtype):
             T.dequant_act_f32(bq[:, sl].cuda(), b_s[:, before:before + kb].float().cuda()).T
         check(out[e], ref, f"rowscale grouped problem {e} kb={kb}")
         before += kb
+    # A table that breaks the caller's promises: an entry with more K blocks than max_k_blocks, one whose count is not a
+    # multiple of the promised 4, a negative slot.  The table is device memory, so the host cannot refuse it: such an entry
+    # must compute and write nothing (its output keeps its contents), and the entries beside it are served as usual.
+    from gcore_lowp import _abi as A
+    table = torch.tensor([[0, 4, 0, 0], [1, 16, 0, 0], [2, 3, 4, 0], [-1, 4, 0, 0], [3, 8, 5, 0]], dtype=torch.int32, device="cuda")
+    out2 = torch.full((4, M, N), 7.0, dtype=out_dtype, device="cuda")
+    A.check(A.lib().lp_gemm_fp8_rowscale_grouped(aqf.data_ptr(), asf.data_ptr(), bqf.data_ptr(), bsf.data_ptr(), A.E8M0, table.data_ptr(), 5, 8, 4,
+                                                 M, N, out2.data_ptr(), A.BF16 if out_dtype == torch.bfloat16 else A.F32, A.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(out2[0], out[0])                      # problem 0: 4 blocks from block 0
+    assert bool((out2[1] == 7).all()) and bool((out2[2] == 7).all())           # 16 > max_k_blocks; 3 is not a multiple of 4
+    assert torch.equal(out2[3], out[3])                      # problem 3: 8 blocks behind the 5 of problems 0 .. 2
 
 
 @pytest.mark.parametrize("case", [([300, 0, 128, 1, 77, 513], 512, 512), ([2048, 16, 700], 1024, 2048), ([64, 64, 64, 64], 2048, 512),

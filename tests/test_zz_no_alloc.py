@@ -37,6 +37,11 @@ def test_static_scratch_gemm_equals_workspace_gemm(pow2):
     for M, N, K in ((384, 1024, 7168), (200, 256, 4096)):
         need = L.lp_gemm_workspace_bytes(M, N, K)
         assert 0 < need <= L.lp_gemm_static_scratch_bytes(), (M, N, K, need)
+        # the workspace also holds fp32 copies of e8m0 scales (a tuning aid): what is left must be the K split's partial
+        # sums, or this shape would not touch the built-in buffer at all
+        r256 = lambda x: (x + 255) // 256 * 256
+        scale_copies = r256(M * (K // 128) * 4) + r256((N // 128) * (K // 128) * 4) if M > 64 and K % 512 == 0 else 0
+        assert need - scale_copies > 0 and (need - scale_copies) % (M * N * 4) == 0, (need, scale_copies)
         xq, xs, wq, ws = _problem(M, N, K, M + N + K, pow2)
         ref = T.gemm_fp8_block_scaling_ref(xq, xs.float(), wq, ws.float())
         xq, xs, wq, ws = (t.to(dev).contiguous() for t in (xq, xs, wq, ws))
@@ -52,7 +57,36 @@ def test_static_scratch_gemm_equals_workspace_gemm(pow2):
                                                    got.data_ptr(), code, A.stream_ptr()))
             torch.cuda.synchronize()
             assert torch.equal(got, want), (got.float() - want.float()).abs().max().item()
+            # nothing is allocated by the call: the device's free memory is the same after three more calls
+            free0 = torch.cuda.mem_get_info()[0]
+            with torch.cuda.device(dev):
+                for _ in range(3):
+                    A.check(L.lp_gemm_fp8_block_static(xq.data_ptr(), xs.data_ptr(), wq.data_ptr(), ws.data_ptr(), sdt, M, N, K,
+                                                       got.data_ptr(), code, A.stream_ptr()))
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free0
+            assert torch.equal(got, want)
             o = got.float().cpu()
             rel = (o - ref).abs().max().item() / ref.abs().max().item()
             cos = torch.nn.functional.cosine_similarity(o.flatten().double(), ref.flatten().double(), dim=0).item()
             assert rel <= 2e-2 and cos >= 0.9999, (rel, cos)
+
+
+def test_static_scratch_entry_takes_shapes_without_a_k_split():
+    """Shapes that never use scratch are served whatever their size: a decode shape whose K split would need more than
+    the built-in buffer if it were taken (it is not: the single-launch decode kernel runs), and a prefill shape."""
+    from gcore_lowp import _abi as A
+    L = A.lib()
+    dev = A.require_gpu()
+    for M, N, K in ((16, 4096, 7168), (512, 2048, 512)):
+        xq, xs, wq, ws = _problem(M, N, K, M + N + K, False)
+        ref = T.gemm_fp8_block_scaling_ref(xq, xs.float(), wq, ws.float())
+        xq, xs, wq, ws = (t.to(dev).contiguous() for t in (xq, xs, wq, ws))
+        got = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        say("static-scratch gemm without a split", (M, N, K))
+        with torch.cuda.device(dev):
+            A.check(L.lp_gemm_fp8_block_static(xq.data_ptr(), xs.data_ptr(), wq.data_ptr(), ws.data_ptr(), A.F32, M, N, K,
+                                               got.data_ptr(), A.BF16, A.stream_ptr()))
+        torch.cuda.synchronize()
+        o = got.float().cpu()
+        assert (o - ref).abs().max().item() / ref.abs().max().item() <= 2e-2
