@@ -644,7 +644,12 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
                     // panels in the L2 (config 2 +1-2 %, the grouped launches 1-2 %, the weight gradient's 15 GB of output 3 %).
                     // Only here, where a store instruction writes whole 128-byte lines: the direct stores below write 4 to 16
                     // bytes per lane, and with the hint the unscaled 4096^3 GEMM (4-byte e4m3 stores) took 83 us instead of 55.
-                    __builtin_nontemporal_store(v, (u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n));
+                    // Not for the 288-column tile: a wave's rows are 288 bytes there and start in the middle of a 128-byte
+                    // line, so neighbouring waves and tiles complete each other's lines, and a line that is pushed out
+                    // half written costs the memory side a partial write (config 2 with e8m0 scales, same box: 179.6 us
+                    // with plain stores, 182 - 191 with the hint; with no stores at all 173.4).
+                    if constexpr (TN == 288) *(u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n) = v;
+                    else __builtin_nontemporal_store(v, (u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n));
                 }
             }
             return;
