@@ -65,7 +65,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
-    ap.add_argument("--only", default="", help="comma list of extra sections to run: deep,copy,c2q,c1,c3,c5,c4 (default: all)")
+    ap.add_argument("--only", default="", help="comma list of extra sections to run: deep,vendor,copy,c2q,c1,c3,c5,c4 (default: all)")
     ap.add_argument("--only-gemm", action="store_true", help="extras: only the skinny and the grouped GEMM (counter runs)")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches (for counter-collection runs)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="rough budget of the CPU baseline sample")
@@ -293,6 +293,25 @@ def main():
         extras["l2_to_cu_copy_probe"] = cp
         del rows_src, sink
 
+    if want("vendor"):
+        # -------------------------------------------------------------- the vendor library on the same silicon: hipBLASLt's
+        # fp8 GEMM through torch._scaled_mm with one scale per tensor (no block scaling: what an unscaled or e8m0-scaled
+        # loop is to be read against, not a replacement for the path) on config 2's shape and on the deep-K shape
+        vend = {}
+        for tag, (Mv, Nv, Kv) in (("c2_2048x18432x7168", (2048, 18432, 7168)), ("deep_k_4096x7168x18432", (4096, 7168, 18432))):
+            try:
+                av = [torch.randn(Mv, Kv, generator=gen, device=dev).to(E4M3) for _ in range(2)]
+                bv = [(torch.randn(Nv, Kv, generator=gen, device=dev)).to(E4M3) for _ in range(2)]
+                one = torch.ones((), device=dev)
+                fns = [(lambda i=i: torch._scaled_mm(av[i], bv[i].t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)) for i in range(2)]
+                msv, _ = time_launches(fns, 10, 3)
+                vend[tag] = {"ms": msv, "tflops": 2.0 * Mv * Nv * Kv / msv / 1e9, "mfma_frac": 2.0 * Mv * Nv * Kv / msv / 1e9 / FP8_PEAK_TFLOPS}
+                del av, bv
+            except Exception as e:                  # a torch build without the fp8 path: reported, not fatal
+                vend[tag] = {"error": repr(e)[:200]}
+            torch.cuda.empty_cache()
+        extras["hipblaslt_fp8_tensorwise_scaled_mm"] = vend
+
     if want("copy"):
         # -------------------------------------------------------------- calibration: a plain device copy of known size
         # (what a streaming read+write kernel reaches on this box; also the reference kernel for scaling the
@@ -435,6 +454,22 @@ def main():
         extras["c5_fp4_to_fp8_fused"] = {"ms_total": total_ms5, "GB/s": bytes5 / total_ms5 / 1e6,
                                          "hbm_frac": bytes5 / total_ms5 / 1e6 / HBM_PEAK_GBS, "elements": elems,
                                          "bytes": bytes5, "variant": "fused, bf16 intermediate not written"}
+
+        # a bare stream of the same mix: per tensor read its packed bytes and write its FP8 bytes (17/32 of the kernel's
+        # reads: the 1 x 32 scale bytes are left out, so the probe moves slightly less than the kernel)
+        probes5 = {}
+        for wgs in (2048, 8192, 32768):
+            def c5_stream(i, wgs=wgs):
+                def run():
+                    for (packed, sc, q, so, rows, cc) in bufs[i]:
+                        PA.check(LP.lp_probe_stream(packed.data_ptr(), rows * cc // 2, q.data_ptr(), rows * cc, wgs, stream()))
+                return run
+            msb, _ = time_launches([c5_stream(i) for i in range(n_chunksets)], max(n_chunks, 4), 2)
+            probes5[f"read_half_write_one_byte_per_element_{wgs}_workgroups_ms"] = msb * n_chunks
+        best5 = min(probes5.values())
+        probes5["bare_stream_hbm_frac"] = (elems // 2 + elems) / best5 / 1e6 / HBM_PEAK_GBS
+        probes5["fused_over_bare_stream"] = total_ms5 / best5
+        extras["c5_floor_probe"] = probes5
 
         def c5_rebase(i):
             def run():
@@ -707,7 +742,7 @@ def main():
         "config": {"workload": "C2 dense block-FP8 GEMM: A[2048,7168] 1x128 e4m3 x B[18432,7168] 128x128 e4m3, fp32 scales -> bf16 [2048,18432]",
                    "M": M, "N": N, "K": K, "operands": "pre-quantised, resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": measured_traffic("gemm_asm_wide<false>", 512 * 512),
+                     "frac": tflops / FP8_PEAK_TFLOPS, "traffic": measured_traffic("gemm_asm_wide<false, 288>", 512 * 512),
                      "traffic_source": "profiles/traffic.json (rocprofv3 --pmc runs of this script, summarised by profile_summary.py)",
                      "kernel": "gemm_asm_wide<false>: the whole problem in one launch, 512 tiles of 256x288 (two full rounds of 256 CUs)",
                      "launch_ms": ms, "flops_per_launch": flops, "wall_ms_per_step": wall_ms,

@@ -401,13 +401,15 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     const uint32_t sel1 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 32) >> 7) != (wcol0 >> 7)));
     const uint32_t sel2 = __builtin_amdgcn_readfirstlane((uint32_t)(((wcol0 + 64) >> 7) != (wcol0 >> 7)));
     (void)bs2_u; (void)sel1; (void)sel2;
-    // 256 x 288 tile: first 16-column block of this wave that lies in the second weight-scale block, whether this wave has
-    // a fifth weight copy (36 groups of 8 rows over 8 waves) and which group that copy moves (16, 17 for waves 0, 1 and
-    // 34, 35 for waves 2, 3, as group g4 + wave), bytes between two groups of weight rows
+    // 256 x 288 and 256 x 224 tiles: first 16-column block of this wave that lies in the second weight-scale block (past
+    // the wave's last block when all its columns lie in one), whether this wave has the one weight copy more that the
+    // first four waves have (36 or 28 groups of 8 rows over 8 waves), which group the copy moves whose group depends on
+    // the wave (as group g4 + wave; 288: the fifth copy, groups 16, 17 for waves 0, 1 and 34, 35 for waves 2, 3; 224: the
+    // third copy, groups 8 .. 13 for waves 0 .. 5 and 22, 23 for waves 6, 7), bytes between two groups of weight rows
     const uint32_t splitnb = __builtin_amdgcn_readfirstlane((uint32_t)(((((wcol0 >> 7) + 1) << 7) - wcol0) >> 4));
     const uint32_t bextra = __builtin_amdgcn_readfirstlane(wave < (TN / 8) % WAVES ? 1u : 0u);
     const uint32_t bstride = __builtin_amdgcn_readfirstlane((uint32_t)(8 * K));
-    const uint32_t g4 = __builtin_amdgcn_readfirstlane(wave < 2 ? 16u : 32u);
+    const uint32_t g4 = __builtin_amdgcn_readfirstlane(TN == 224 ? (wave < 6 ? 8u : 16u) : (wave < 2 ? 16u : 32u));
     // A wave none of whose 64 activation rows exist (the tail of M, or an expert's short tile) runs the loop's
     // copy-and-barrier skeleton only, in the loops generated with that second body (256-row and flat tiles).
     const uint32_t idle = __builtin_amdgcn_readfirstlane((int64_t)wm * 64 >= M - m0 ? 1u : 0u);
@@ -480,6 +482,25 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4;
         accs[5] = acc5; accs[6] = acc6; accs[7] = acc7; accs[8] = acc8;
+    } else if constexpr (TN == 224) {
+        static_assert(TM == 256 && KSUB == 1 && !DUAL && NST == 2 && !BROW, "the 224-column tile exists for the 256-row kernel only");
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6;
+        if constexpr (HWS) {
+            asm volatile(
+#include "gemm_wide224_hw_loop.inc"
+                : "=&{v[112:127]}"(acc0), "=&{v[128:143]}"(acc1), "=&{v[144:159]}"(acc2), "=&{v[160:175]}"(acc3),
+                  "=&{v[176:191]}"(acc4), "=&{v[192:207]}"(acc5), "=&{v[208:223]}"(acc6)
+                : LP_ASM_INPUTS_WIDE
+                : LP_ASM_CLOBBERS_WIDE);
+        } else {
+            asm volatile(
+#include "gemm_wide224_loop.inc"
+                : "=&{v[112:127]}"(acc0), "=&{v[128:143]}"(acc1), "=&{v[144:159]}"(acc2), "=&{v[160:175]}"(acc3),
+                  "=&{v[176:191]}"(acc4), "=&{v[192:207]}"(acc5), "=&{v[208:223]}"(acc6)
+                : LP_ASM_INPUTS_WIDE
+                : LP_ASM_CLOBBERS_WIDE);
+        }
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3; accs[4] = acc4; accs[5] = acc5; accs[6] = acc6;
     } else if constexpr (NN && WN == 4) {
         f32x16v acc0, acc1, acc2, acc3;
         asm volatile(
@@ -644,11 +665,11 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
                     // panels in the L2 (config 2 +1-2 %, the grouped launches 1-2 %, the weight gradient's 15 GB of output 3 %).
                     // Only here, where a store instruction writes whole 128-byte lines: the direct stores below write 4 to 16
                     // bytes per lane, and with the hint the unscaled 4096^3 GEMM (4-byte e4m3 stores) took 83 us instead of 55.
-                    // Not for the 288-column tile: a wave's rows are 288 bytes there and start in the middle of a 128-byte
-                    // line, so neighbouring waves and tiles complete each other's lines, and a line that is pushed out
-                    // half written costs the memory side a partial write (config 2 with e8m0 scales, same box: 179.6 us
-                    // with plain stores, 182 - 191 with the hint; with no stores at all 173.4).
-                    if constexpr (TN == 288) *(u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n) = v;
+                    // Not for the 288- and 224-column tiles: a wave's rows are 288 or 224 bytes there and start in the middle
+                    // of a 128-byte line, so neighbouring waves and tiles complete each other's lines, and a line that is
+                    // pushed out half written costs the memory side a partial write (config 2 with e8m0 scales, same box:
+                    // 179.6 us with plain stores, 182 - 191 with the hint; with no stores at all 173.4).
+                    if constexpr (TN == 288 || TN == 224) *(u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n) = v;
                     else __builtin_nontemporal_store(v, (u32x4 *)((uint16_t *)C + (row_base + row) * ldc + n));
                 }
             }
@@ -724,16 +745,17 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
 }
 
 // 256 x 288 tiles: N = 18432 is 64 of them, so a 2048-row problem is 512 tiles, exactly two rounds on 256 CUs.
-template <bool HWS>
+// 256 x 224 tiles: N = 7168 is 32 of them, so 4096 rows are 512 tiles where 256 x 256 tiles make 448 (1.75 rounds).
+template <bool HWS, int TN = 288>
 __global__ __launch_bounds__(512) void gemm_asm_wide(const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                                      const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t M,
                                                      int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
                                                      void *__restrict__ C, int64_t ldc, int out_dtype)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<256, 288, 1>::LDS_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<256, TN, 1>::LDS_BYTES];
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
-    tile_asm<256, 288, 1, HWS, false, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 256, M, tn * 288, N, K, C, ldc, out_dtype);
+    tile_asm<256, TN, 1, HWS, false, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 256, M, tn * TN, N, K, C, ldc, out_dtype);
 }
 
 // 128 x 128 tile with the K split inside the workgroup (see tile_asm): 8 waves, two sets of LDS stages.
@@ -1137,27 +1159,36 @@ bool nt_unit_scales_ok(const void *ones, int64_t M, int64_t N, int64_t K)
     return !no_asm && asm_shape_ok(ones, ones, M, N, K, LP_E8M0);
 }
 
-// 256 x 288 tiles when they divide N and fill the last round of tiles better than 256 x 256 tiles would; false when
-// the shape does not fit (the caller goes on with the other kernels).
+// 256 x 288 or 256 x 224 tiles when they divide N and fill the last round of tiles better than 256 x 256 tiles would
+// (of the two, the one that fills it better; 288 when they tie); false when the shape does not fit (the caller goes on
+// with the other kernels).  LP_GEMM_WIDE = 0 switches the route off, 288 or 224 forces that width where it divides N.
 bool launch_wide(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                  void *C, int64_t ldc, int out_dtype, hipStream_t st, int *rc)
 {
-    static const bool off = getenv("LP_GEMM_NO_ASM") != nullptr || (getenv("LP_GEMM_WIDE") && atoi(getenv("LP_GEMM_WIDE")) == 0);
-    static const bool force = getenv("LP_GEMM_WIDE") && atoi(getenv("LP_GEMM_WIDE")) == 1;             // tuning aid
-    if (off || (scale_dtype != LP_F32 && scale_dtype != LP_E8M0) || N % 288 || !asm_shape_ok(As, Bs, M, N, K, scale_dtype)) return false;
-    const int64_t tiles_m = (M + 255) / 256, wide = tiles_m * (N / 288), big = tiles_m * ((N + 255) / 256);
+    static const int knob = getenv("LP_GEMM_WIDE") ? atoi(getenv("LP_GEMM_WIDE")) : -1;             // tuning aid
+    static const bool off = getenv("LP_GEMM_NO_ASM") != nullptr || knob == 0;
+    if (off || (scale_dtype != LP_F32 && scale_dtype != LP_E8M0) || !asm_shape_ok(As, Bs, M, N, K, scale_dtype)) return false;
+    const int64_t tiles_m = (M + 255) / 256, big = tiles_m * ((N + 255) / 256);
     // fraction of CU slots used over whole rounds of 256 tiles
-    const double fill_wide = (double)wide / (double)((wide + 255) / 256 * 256), fill_big = (double)big / (double)((big + 255) / 256 * 256);
-    if (!force && !(fill_wide >= 0.9 && fill_wide > fill_big + 0.05)) return false;
-    const int64_t grid = gemm::padded_grid(tiles_m, N / 288);
+    auto fill = [](int64_t tiles) { return (double)tiles / (double)((tiles + 255) / 256 * 256); };
+    int width = 0;
+    for (int w : {288, 224}) {
+        if (N % w) continue;
+        if (knob == w) { width = w; break; }
+        if (knob > 0) continue;
+        const double f = fill(tiles_m * (N / w));
+        if (f >= 0.9 && f > fill(big) + 0.05 && (!width || f > fill(tiles_m * (N / width)))) width = w;
+    }
+    if (!width) return false;
+    const int64_t tiles_n = N / width, grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return false;
-    if (scale_dtype == LP_E8M0)
-        hipLaunchKernelGGL((gemm_asm_wide<true>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
-                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, N / 288, C, ldc, out_dtype);
-    else
-        hipLaunchKernelGGL((gemm_asm_wide<false>), dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As,
-                           (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, N / 288, C, ldc, out_dtype);
-    *rc = check_launch("lp_gemm_fp8_block(asm 256x288)");
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(512), 0, st, (const uint8_t *)Aq, (const float *)As, (const uint8_t *)Bq,
+                           (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
+    };
+    if (width == 288) scale_dtype == LP_E8M0 ? go(gemm_asm_wide<true, 288>) : go(gemm_asm_wide<false, 288>);
+    else scale_dtype == LP_E8M0 ? go(gemm_asm_wide<true, 224>) : go(gemm_asm_wide<false, 224>);
+    *rc = check_launch(width == 288 ? "lp_gemm_fp8_block(asm 256x288)" : "lp_gemm_fp8_block(asm 256x224)");
     return true;
 }
 

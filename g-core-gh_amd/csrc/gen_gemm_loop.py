@@ -41,6 +41,7 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
     global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP, SPREAD, NN, BF, RBN
+    global WIDE_GROUP, WIDE_PART
     # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
     # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
     WITH_IDLE, IDLE = idle, False
@@ -76,15 +77,18 @@ def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, ea
     # copies are split by wave behind one branch, keeps its runs
     SPREAD = early and not HALFSPLIT and SPREAD_ON
     # wide: a wave owns 64 x 144 columns (nine 16-column blocks), e.g. the 256 x 288 tile that cuts 18432 weight rows
-    # into exactly 64 tile columns.  144 columns always straddle two weight-scale blocks, at a 16-column boundary known
-    # only at run time (s74 = first block that takes the second scale row): the folds read one set of scale products,
-    # which is switched to the second row's products when the loop reaches that block.  The accumulators take 144
-    # registers, so the plan below moves everything down; fragment read addresses and the scale buffer base are used
-    # straight from the asm operands, and the weight copies share one per-lane offset (the tile's weight rows are
-    # never clamped: N is a multiple of the tile width) with one scalar base per copy.
+    # into exactly 64 tile columns, or 64 x 112 columns (seven blocks): the 256 x 224 tile that cuts 7168 weight rows
+    # into 32.  144 columns always straddle two weight-scale blocks and 112 mostly do, at a 16-column boundary known
+    # only at run time (s74 = first block that takes the second scale row; past the last block if there is none): the
+    # folds read one set of scale products, which is switched to the second row's products when the loop reaches that
+    # block.  The accumulators take up to 144 registers, so the plan below moves everything down; fragment read
+    # addresses and the scale buffer base are used straight from the asm operands, and the weight copies share one
+    # per-lane offset (the tile's weight rows are never clamped: N is a multiple of the tile width) with one scalar
+    # base per copy.
     WIDE = wide
     if wide:
-        assert tm == 256 and tn == 288 and waves_m == 4 and waves_n == 2 and ksub == 1 and nstage == 2 and not brow
+        assert tm == 256 and tn in WIDE_PLANS and waves_m == 4 and waves_n == 2 and ksub == 1 and nstage == 2 and not brow
+        WIDE_GROUP, WIDE_PART = WIDE_PLANS[tn]
         ACC, P, AF, WFB = 112, 80, 48, (32, 40)
         SAN, SC, SC2, SRD = 24, 28, 20, "v19"
         WS1, WS2, WSCUR = "v20", "v21", "v22"            # hardware-scaled variant: weight-scale bytes of row 1, row 2, in use
@@ -143,13 +147,18 @@ SCP = (44, 224, 228)        # scale products per pair of 16-column blocks when a
 SRDB0, SRDB = 37, 38        # row-scaled weights: LDS address of the lane's weight-scale dwords (half 0, half in use)
 WSN, WSC = 96, 100          # ... the dwords of this group / of the next one, one per 16-row block
 WB_EXTRA = ("s[42:43]", "s[78:79]", "s[80:81]", "s[82:83]", "s[84:85]")     # wide: weight base per copy
-# wide: the 36 groups of 8 weight rows are dealt to the waves so that the early hand-back can request the first 64 rows of
-# both wave columns (groups 0..7 and 18..25: the rows blocks 0..3 read) half way through a step and the other 80 rows of
-# each at its end.  Copy i of wave w moves group WIDE_GROUP[i] + w; the fifth copy exists for waves 0..3 only and moves
-# groups 16, 17 (waves 0, 1) and 34, 35 (waves 2, 3): its group comes in s88 (as an LDS offset) and its base in s[84:85].
-# All group numbers have the parity of w, so one per-lane source offset (row 8 w + lane / 8, swizzled chunk) serves all.
-WIDE_GROUP = (0, 18, 8, 26, None)
-WIDE_PART = ("mid", "mid", "end", "end", "end")
+# wide, 288 columns: the 36 groups of 8 weight rows are dealt to the waves so that the early hand-back can request the
+# first 64 rows of both wave columns (groups 0..7 and 18..25: the rows blocks 0..3 read) half way through a step and the
+# other 80 rows of each at its end.  Copy i of wave w moves group WIDE_GROUP[i] + w; the fifth copy exists for waves 0..3
+# only and moves groups 16, 17 (waves 0, 1) and 34, 35 (waves 2, 3): its group (less w) comes from the set-up code, in
+# s88 as an LDS offset, and its base in the copy's own register pair.  All group numbers have the parity of w, so one
+# per-lane source offset (row 8 w + lane / 8, swizzled chunk) serves all.
+# 224 columns: 28 groups, wave columns of 14.  Mid-step: groups 0..7 and 14..21 (blocks 0..3 of both wave columns); at
+# the end of the step the third copy moves groups 8..13 (waves 0..5) and 22, 23 (waves 6, 7) -- the set-up code's group --
+# and the fourth, of waves 0..3 only, groups 24..27.
+WIDE_PLANS = {288: ((0, 18, 8, 26, None), ("mid", "mid", "end", "end", "end")),
+              224: ((0, 14, None, 24), ("mid", "mid", "end", "end"))}
+WIDE_GROUP, WIDE_PART = WIDE_PLANS[288]
 
 _uid = 0
 
@@ -282,8 +291,9 @@ def copies_per_part():
     if NN:
         return a, b
     if WIDE:
-        # waves 0 .. 3 issue a third request in the end part; counting two makes their waits one request stricter
-        return a + 2, 2
+        # waves 0 .. 3 issue one more request in the end part than the others; counting without it makes their waits
+        # one request stricter
+        return a + WIDE_PART.count("mid"), B_BYTES // 1024 // WAVES - WIDE_PART.count("mid")
     if HALFSPLIT:
         # a wave issues its weight copies in one of the two parts; either way the two parts together are a + b
         # requests, and counting none for the end part only makes the last trip's waits stricter
@@ -504,7 +514,7 @@ def step(c):
         # Early hand-back: the barrier sits in front of the first read of the second weight half (block NB / 2, read
         # one block ahead), so that half is known to have landed before anyone reads it, and behind every wave's
         # last read of the first half, so those rows and the activation rows can be requested again right after it.
-        handback = EARLY and nb == NB // 2 - 1
+        handback = EARLY and nb == (3 if WIDE else NB // 2 - 1)      # wide: blocks 0..3 are the first part whatever NB
         if handback:
             assert nb + 1 < NB and not pieces
             wait_copies(c, False, " lgkmcnt(0)")
@@ -671,7 +681,7 @@ def generate():
         emit("s_mov_b32 s86, %[bextra]")
         # weight base of copy i: WIDE_GROUP[i] groups of 8 rows further on (%[bstride] = bytes per group); the fifth
         # copy's group comes from the set-up code (%[g4])
-        for i in range(1, len(WB_EXTRA)):
+        for i in range(1, len(WIDE_GROUP)):
             lo = int(WB_EXTRA[i][2:4])
             if WIDE_GROUP[i] is None:
                 emit("s_mul_i32 s87, %[bstride], %[g4]")
@@ -787,6 +797,8 @@ def main():
                       ("gemm_mid_hw_loop.inc", (128, 128, 2, 2, 1, True, 2, False, True)),
                       ("gemm_wide_loop.inc", (256, 288, 4, 2, 1, False, 2, False, True, True, True, PP)),
                       ("gemm_wide_hw_loop.inc", (256, 288, 4, 2, 1, True, 2, False, True, True, True, PP)),
+                      ("gemm_wide224_loop.inc", (256, 224, 4, 2, 1, False, 2, False, True, True, True, PP)),
+                      ("gemm_wide224_hw_loop.inc", (256, 224, 4, 2, 1, True, 2, False, True, True, True, PP)),
                       ("gemm_flat_loop.inc", (128, 256, 2, 4, 1, False, 3, False, True, False, True)),
                       ("gemm_flat_hw_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True)),
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),

@@ -18,6 +18,7 @@ spec.loader.exec_module(gen)
 LOOPS = {
     "big 256x256": ((256, 256, 4, 2, 1, False, 2, False, True), [(4 + 2, 2)]),
     "wide 256x288": ((256, 288, 4, 2, 1, False, 2, False, True, True), [(4 + 2, 3), (4 + 2, 2)]),        # waves 0..3 copy a fifth group
+    "wide 256x224": ((256, 224, 4, 2, 1, False, 2, False, True, True), [(4 + 2, 2), (4 + 2, 1)]),        # waves 0..3 copy a fourth group
     "flat 128x256, three stages": ((128, 256, 2, 4, 1, False, 3, False, True), [(2 + 4, 0), (2, 4)]),    # first / second half of the waves
     # weights stored [K, N]: the activation rows mid-step, every weight row at the end of the step
     "big 256x256, weights stored [K, N]": ((256, 256, 4, 2, 1, True, 2, False, True, False, True, True, True), [(4, 4)]),

@@ -610,17 +610,19 @@ def test_gemm_column_split_one_launch_equals_two_launches(G):
     assert len(theirs) == 2 * len(shapes) and theirs == digests(), (theirs, r.stdout[-800:])
 
 
-def test_gemm_wide_tile_forced_on_other_shapes(G):
-    """The 256 x 288 tile kernel is chosen by itself only where it fills whole rounds of CUs; LP_GEMM_WIDE=1 (read once
-    per process, hence the child) sends every prefill-sized problem whose N is a multiple of 288 to it: few tile
-    columns, ragged M, tile origins at all four offsets inside a weight-scale block, both scale types; with
+@pytest.mark.parametrize("width,shapes", [(288, ((2048, 4608, 512), (1000, 13824, 512), (333, 27648, 1024))),
+                                          (224, ((2048, 3584, 512), (1000, 10752, 512), (333, 21504, 1024)))])
+def test_gemm_wide_tile_forced_on_other_shapes(G, width, shapes):
+    """The 256 x 288 and 256 x 224 tile kernels are chosen by themselves only where they fill whole rounds of CUs;
+    LP_GEMM_WIDE=288 or 224 (read once per process, hence the child) sends every prefill-sized problem whose N is a
+    multiple of that width to it: few tile columns, ragged M, tile origins at every offset inside a weight-scale block
+    (wave columns that straddle two blocks and, for 224, wave columns inside one), both scale types; with
     power-of-two scales the result must equal the default kernels' bit for bit (same order of summation)."""
     import hashlib
     import os
     import subprocess
     import sys
-    say("gemm 256 x 288 tiles forced (LP_GEMM_WIDE=1 in a child process)")
-    shapes = ((2048, 4608, 512), (1000, 13824, 512), (333, 27648, 1024))
+    say(f"gemm 256 x {width} tiles forced (LP_GEMM_WIDE={width} in a child process)")
     mine = []
     for (M, N, K) in shapes:
         xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + K, pow2=True)
@@ -634,7 +636,7 @@ def test_gemm_wide_tile_forced_on_other_shapes(G):
         "for (M, N, K) in %r:\n"
         "    for pow2 in (False, True):\n"
         "        xq, xs, wq, ws = t.quantized_problem(M, N, K, seed=M + K, pow2=pow2)\n"
-        "        print('[case] 256 x 288 tiles', M, N, K, pow2, flush=True)\n"
+        "        print('[case] wide tiles', M, N, K, pow2, flush=True)\n"
         "        c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())\n"
         "        wide = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), out_dtype=torch.float32)\n"
         "        assert torch.equal(c, wide.to(torch.bfloat16))\n"
@@ -642,7 +644,7 @@ def test_gemm_wide_tile_forced_on_other_shapes(G):
         "        if pow2:\n"
         "            print('md5', hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest(), flush=True)\n"
     ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), shapes)
-    env = dict(os.environ, LP_GEMM_WIDE="1", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    env = dict(os.environ, LP_GEMM_WIDE=str(width), PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
     theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
