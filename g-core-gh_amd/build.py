@@ -61,9 +61,10 @@ def _compile(src: str, force: bool) -> str:
 
 
 def _generate():
-    """Run the generator of the hand-scheduled GEMM loops: it rewrites exactly those of its outputs (csrc/gemm_*_loop.inc)
+    """Run the generators of the hand-scheduled GEMM loops: they rewrite exactly those of its outputs (csrc/gemm_*_loop.inc)
     whose content differs from what it generates, so a stale or hand-edited file never reaches the compiler."""
     subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_gemm_loop.py")])
+    subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_gemm_quad_loop.py")])
 
 
 def _audit_asm_operands():

@@ -97,6 +97,26 @@ def asm_blocks(asm_text: str):
     return out
 
 
+def accumulation_registers_outside_asm(asm_text: str, kernel_substr: str) -> list[str]:
+    """Lines of the kernels whose symbol contains kernel_substr that name an accumulation register (a0 .. a255) outside the
+    inline-asm expansions.  The four-wave loop keeps its accumulators there across two asm statements; the compiler is
+    told they are clobbered, and must not put anything of its own (a spill, say) into them in between."""
+    out, kernel, inside = [], "", False
+    for line in asm_text.splitlines():
+        m = re.match(r"^(\w+):", line)
+        if m and not inside:
+            kernel = m.group(1)
+        if "ASMSTART" in line:
+            inside = True
+        elif "ASMEND" in line:
+            inside = False
+        elif not inside and kernel_substr in kernel:
+            code = line.split(";")[0].strip()
+            if code and not code.startswith(".") and re.search(r"\ba(?:\d+|\[\d+:\d+\])", code):
+                out.append(f"{kernel}: {code}")
+    return out
+
+
 def audit(quiet: bool = False) -> int:
     templates = {f: load_template(os.path.join(HERE, f)) for f in sorted(os.listdir(HERE)) if f.endswith("_loop.inc")}
     with tempfile.TemporaryDirectory() as tmp:
@@ -106,8 +126,12 @@ def audit(quiet: bool = False) -> int:
             sys.stderr.write(r.stderr)
             return 2
         with open(out) as f:
-            blocks = asm_blocks(f.read())
+            asm_text = f.read()
+        blocks = asm_blocks(asm_text)
     bad = checked = 0
+    for line in accumulation_registers_outside_asm(asm_text, "gemm_asm_quad"):
+        print(f"FAIL accumulation register used outside the asm statements: {line}")
+        bad += 1
     declared = declared_registers(os.path.join(HERE, "gemm_fp8_big.hip"))
     for name, (_, literal) in templates.items():
         if name not in declared:

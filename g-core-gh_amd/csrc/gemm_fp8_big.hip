@@ -40,6 +40,7 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int BM = 256;             // tile rows (activations)
 constexpr int KB = 128;             // bytes per row per step
 constexpr int THREADS = 512;
+constexpr int QUAD_DEFAULT = 0;    // the four-wave 256 x 256 loop is opt-in (LP_GEMM_QUAD=1)
 
 #define LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
 #define GLB_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
@@ -222,6 +223,31 @@ typedef float f32x16v __attribute__((ext_vector_type(16)));
         "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60",   \
         "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77",   \
         "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s98", "s99"
+#define LP_ASM_CLOBBERS_QUAD                                                                                              \
+    "memory", "scc", "m0", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84",     \
+        "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95", "v96", "v97", "v98", "v99",          \
+        "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109", "v110", "v111", "v112",           \
+        "v113", "v114", "v115", "v116", "v117", "v118", "v119", "v120", "v121", "v122", "v123", "v124", "v125",           \
+        "v126", "v127", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52",        \
+        "s53", "s54", "s55", "s56", "s57", "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11",      \
+        "a12", "a13", "a14", "a15", "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26",          \
+        "a27", "a28", "a29", "a30", "a31", "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41",          \
+        "a42", "a43", "a44", "a45", "a46", "a47", "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56",          \
+        "a57", "a58", "a59", "a60", "a61", "a62", "a63", "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71",          \
+        "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", "a80", "a81", "a82", "a83", "a84", "a85", "a86",          \
+        "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", "a96", "a97", "a98", "a99", "a100", "a101",        \
+        "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", "a112", "a113", "a114",           \
+        "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127",           \
+        "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140",           \
+        "a141", "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153",           \
+        "a154", "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166",           \
+        "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179",           \
+        "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192",           \
+        "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205",           \
+        "a206", "a207", "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218",           \
+        "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231",           \
+        "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244",           \
+        "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
 #define LP_ASM_INPUTS_WIDE                                                                                                \
     [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [boff0] "v"(boff[0]),         \
         [soff] "v"(soff), [srd] "v"(srd), [ard0] "v"(ard0), [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1),         \
@@ -730,6 +756,133 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
     }
 }
 
+
+// The 256 x 256 tile on four waves of 128 x 128 with the accumulators in a[0:255] (gen_gemm_quad_loop.py): e8m0 scales,
+// whole tiles only (M and N multiples of 256, K of 512).  The loop statement leaves the accumulators of the wave's first
+// 64 rows in v[128:255], laid out like tile_asm's (block nb of 16 columns at v[128 + 16 nb : +15], register 4 mb + r of
+// lane (l16, lq) = row 16 mb + l16, column 16 nb + 4 lq + r); a second statement fetches the other 64 rows.  The compiler
+// is told that the loop clobbers every accumulation register, and nothing between the two statements may use one: the
+// build audit fails if the kernel's assembly names an accumulation register outside the statements.
+__device__ __forceinline__ void tile_quad(uint8_t *smem, const uint8_t *__restrict__ Aq, const uint8_t *__restrict__ As,
+                                          const uint8_t *__restrict__ Bq, const uint8_t *__restrict__ Bs, int64_t m0, int64_t n0,
+                                          int64_t M, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    constexpr int WAVES = 4, A_BYTES = 256 * KB, B_LDS = 2 * A_BYTES, S_LDS = 4 * A_BYTES;
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    const int lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const uint32_t kblocks = (uint32_t)(K / KB);
+    const uint32_t trips = kblocks / 4;
+    auto uniform = [](const void *p) -> uint64_t {
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)p);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)p >> 32));
+        return ((uint64_t)hi << 32) | lo;
+    };
+    const int64_t wcol0 = n0 + wn * 128;
+    const uint64_t a_u = uniform(Aq), b_u = uniform(Bq), s_u = uniform(As), bs_u = uniform(Bs + (wcol0 >> 7) * kblocks);
+    // copy i of this wave moves the 8 LDS rows 8 (wave + 4 i) ..: lane -> row lane / 8 of them, 16-byte slot lane % 8
+    const int ld_row = lane >> 3, ld_slot = lane & 7;
+    uint32_t aoff[8], boff[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = tile_row(8 * (wave + WAVES * i) + ld_row);
+        aoff[i] = (uint32_t)((m0 + row) * K + swz(row, ld_slot) * 16);
+        boff[i] = (uint32_t)((n0 + row) * K + swz(row, ld_slot) * 16);
+    }
+    // scale bytes of a group of four K steps: each wave copies the dwords of 64 activation rows (one per lane) and its own
+    // weight-scale dword into every lane's slot
+    const uint32_t soff = (uint32_t)((m0 + wave * 64 + lane) * kblocks);
+    uint32_t zero = 0;
+    asm volatile("" : "+v"(zero));
+    const uint32_t lds0 = (uint32_t)(uintptr_t)LDS_PTR(smem);
+    const uint32_t m0base = __builtin_amdgcn_readfirstlane(lds0 + wave * 1024);
+    const uint32_t s0base = __builtin_amdgcn_readfirstlane(lds0 + S_LDS + wave * 256);
+    const int arow_l = wm * 128 + l16, brow_l = wn * 128 + l16;
+    const uint32_t ard0 = lds0 + lds_row(arow_l) * KB + swz(arow_l, 2 * lq) * 16;
+    const uint32_t ard1 = lds0 + lds_row(arow_l) * KB + swz(arow_l, 2 * lq + 1) * 16;
+    const uint32_t brd0 = lds0 + B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq) * 16;
+    const uint32_t brd1 = lds0 + B_LDS + lds_row(brow_l) * KB + swz(brow_l, 2 * lq + 1) * 16;
+    const uint32_t srd = lds0 + S_LDS + arow_l * 4;
+    const uint32_t wsrd = lds0 + S_LDS + 1024 + wave * 256 + lane * 4;
+
+    f32x16v accs[8];
+    {
+        f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
+        asm volatile(
+#include "gemm_quad_hw_loop.inc"
+            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
+            : [aoff0] "v"(aoff[0]), [aoff1] "v"(aoff[1]), [aoff2] "v"(aoff[2]), [aoff3] "v"(aoff[3]), [aoff4] "v"(aoff[4]),
+              [aoff5] "v"(aoff[5]), [aoff6] "v"(aoff[6]), [aoff7] "v"(aoff[7]), [boff0] "v"(boff[0]), [boff1] "v"(boff[1]),
+              [boff2] "v"(boff[2]), [boff3] "v"(boff[3]), [boff4] "v"(boff[4]), [boff5] "v"(boff[5]), [boff6] "v"(boff[6]),
+              [boff7] "v"(boff[7]), [soff] "v"(soff), [zero] "v"(zero), [srd] "v"(srd), [wsrd] "v"(wsrd), [ard0] "v"(ard0),
+              [ard1] "v"(ard1), [brd0] "v"(brd0), [brd1] "v"(brd1), [abase] "s"(a_u), [bbase] "s"(b_u), [sbase] "s"(s_u),
+              [bsptr] "s"(bs_u), [m0base] "s"(m0base), [s0base] "s"(s0base), [trips] "s"(trips)
+            : LP_ASM_CLOBBERS_QUAD);
+        accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+        accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+    }
+    using E = StagedEpilogue<128>;
+    static_assert(WAVES * E::WAVE_BYTES <= S_LDS, "the waves' staging regions must fit the stage memory");
+    __syncthreads();                                      // every wave is done with the stage memory
+    uint8_t *stage = smem + wave * E::WAVE_BYTES;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        if (half == 1) {
+            f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
+            asm volatile(
+#include "gemm_quad_tail_loop.inc"
+                : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+                  "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
+                :
+                : "memory");
+            accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
+            accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
+        }
+        const int64_t row_base = m0 + wm * 128 + half * 64;
+        if (out_dtype == LP_BF16) {
+            // through LDS, so that a store instruction writes whole 128-byte lines (see tile_asm); a wave reads back only
+            // what it wrote, in a region of its own
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb) {
+#pragma unroll
+                for (int nb = 0; nb < 8; ++nb) {
+                    const u32x2 o = {pack_bf16(accs[nb][mb * 4], accs[nb][mb * 4 + 1]), pack_bf16(accs[nb][mb * 4 + 2], accs[nb][mb * 4 + 3])};
+                    *(u32x2 *)(stage + E::write_offset(mb, nb, l16, lq)) = o;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int p = 0; p < E::PASSES; ++p) {
+                const int row = E::read_row(p, lane), chunk = E::read_chunk(p, lane);
+                const u32x4 v = *(const u32x4 *)(stage + E::read_offset(row, chunk));
+                __builtin_nontemporal_store(v, (u32x4 *)((uint16_t *)C + (row_base + row) * ldc + wcol0 + chunk * 8));
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the other half's staging writes follow
+            continue;
+        }
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+            const int64_t row = row_base + mb * 16 + l16;
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) {
+                const int64_t n = wcol0 + nb * 16 + 4 * lq;
+                const float v0 = accs[nb][mb * 4], v1 = accs[nb][mb * 4 + 1], v2 = accs[nb][mb * 4 + 2], v3 = accs[nb][mb * 4 + 3];
+                if (out_dtype == LP_E4M3) {
+                    auto sat = [](float x) { const float c = __builtin_fminf(__builtin_fmaxf(x, -kE4M3Max), kE4M3Max); return x != x ? x : c; };
+                    *(uint32_t *)((uint8_t *)C + row * ldc + n) = cvt4(sat(v0), sat(v1), sat(v2), sat(v3));
+                } else {
+                    u32x4 o = {f2u(v0), f2u(v1), f2u(v2), f2u(v3)};
+                    *(u32x4 *)((float *)C + row * ldc + n) = o;
+                }
+            }
+        }
+    }
+    (void)M; (void)N;
+}
+
 #pragma clang diagnostic pop
 
 template <int TM, int TN, int KSUB, bool HWS = false, int NST = 2>
@@ -756,6 +909,18 @@ __global__ __launch_bounds__(512) void gemm_asm_wide(const uint8_t *__restrict__
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
     tile_asm<256, TN, 1, HWS, false, 2, false, true>(smem, Aq, As, Bq, Bs, tm * 256, M, tn * TN, N, K, C, ldc, out_dtype);
+}
+
+// 256 x 256 tiles on four waves with the accumulators in the accumulation registers (tile_quad): e8m0 scales, whole tiles.
+__global__ __launch_bounds__(256) void gemm_asm_quad(const uint8_t *__restrict__ Aq, const uint8_t *__restrict__ As,
+                                                     const uint8_t *__restrict__ Bq, const uint8_t *__restrict__ Bs, int64_t M,
+                                                     int64_t N, int64_t K, int64_t tiles_m, int64_t tiles_n,
+                                                     void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * 256 * KB + 4096];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    tile_quad(smem, Aq, As, Bq, Bs, tm * 256, tn * 256, M, N, K, C, ldc, out_dtype);
 }
 
 // 128 x 128 tile with the K split inside the workgroup (see tile_asm): 8 waves, two sets of LDS stages.
@@ -1101,6 +1266,13 @@ int choose_big_tn(int64_t M, int64_t N)
     return best;
 }
 
+// Whole 256 x 256 tiles only: the four-wave loop copies and stores without masks.  LP_GEMM_QUAD = 0 / 1 (tuning aid).
+static bool quad_ok(int64_t M, int64_t N)
+{
+    static const int knob = getenv("LP_GEMM_QUAD") ? atoi(getenv("LP_GEMM_QUAD")) : QUAD_DEFAULT;
+    return knob != 0 && M % 256 == 0 && N % 256 == 0;
+}
+
 int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N,
                int64_t K, void *C, int64_t ldc, int out_dtype, int tn, hipStream_t st)
 {
@@ -1116,6 +1288,11 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
         const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
         const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
         if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: problem too large");
+        if (quad_ok(M, N)) {
+            hipLaunchKernelGGL(gemm_asm_quad, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, (const uint8_t *)As,
+                               (const uint8_t *)Bq, (const uint8_t *)Bs, M, N, K, tiles_m, tiles_n, C, ldc, out_dtype);
+            return check_launch("lp_gemm_fp8_block(asm e8m0, four waves)");
+        }
         hipLaunchKernelGGL((gemm_asm<256, 256, 1, true>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)Aq,
                            (const float *)As, (const uint8_t *)Bq, (const float *)Bs, M, N, K, tiles_m, tiles_n, C, ldc,
                            out_dtype);
@@ -1148,6 +1325,11 @@ int launch_nt_unit_scales(const void *A, const void *B, const void *ones, int64_
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_nt: problem too large");
+    if (quad_ok(M, N)) {
+        hipLaunchKernelGGL(gemm_asm_quad, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)A, (const uint8_t *)ones,
+                           (const uint8_t *)B, (const uint8_t *)ones, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+        return check_launch("lp_gemm_nt(asm, unit scales, four waves)");
+    }
     hipLaunchKernelGGL((gemm_asm<256, 256, 1, true>), dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)A, (const float *)ones,
                        (const uint8_t *)B, (const float *)ones, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
     return check_launch("lp_gemm_nt(asm, unit scales)");

@@ -824,6 +824,12 @@ def probe_bodies(here):
             for f in range(k):
                 lines.append(f"v_fmac_f32 v{64 + (j * 8 + f) % 64}, v{32 + 4 * src + f % 4}, v20")
         write(os.path.join(here, "probe"), f"probe_mfma_body{k}.inc")
+    # the hardware-scaled form, accumulating in place as the e8m0 loops do (unit scale bytes in v21)
+    lines = [f"v_mfma_scale_f32_16x16x128_f8f6f4 v[{32 + 4 * j}:{35 + 4 * j}], v[0:7], v[8:15], v[{32 + 4 * j}:{35 + 4 * j}], v21, v21 "
+             "op_sel:[0,0,0] op_sel_hi:[0,0,0]" for j in range(8)]
+    write(os.path.join(here, "probe"), "probe_mfma_body_scaled.inc")
+    lines = [f"v_mfma_f32_16x16x128_f8f6f4 v[{32 + 4 * j}:{35 + 4 * j}], v[0:7], v[8:15], v[{32 + 4 * j}:{35 + 4 * j}]" for j in range(8)]
+    write(os.path.join(here, "probe"), "probe_mfma_body_inplace.inc")
 
 
 def write(here, name):

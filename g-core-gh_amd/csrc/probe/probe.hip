@@ -178,11 +178,11 @@ __global__ __launch_bounds__(512) void probe_mfma(const uint8_t *__restrict__ op
     if (operands != nullptr)
         asm volatile("global_load_dwordx4 v[0:3], %0, off\n\tglobal_load_dwordx4 v[4:7], %0, off offset:16\n\t"
                      "global_load_dwordx4 v[8:11], %0, off offset:32\n\tglobal_load_dwordx4 v[12:15], %0, off offset:48\n\t"
-                     "s_waitcnt vmcnt(0)\n\tv_mov_b32 v20, 0x3f8ccccd" ::"v"(p) : "memory", LP_PROBE_CLOBBERS);
+                     "s_waitcnt vmcnt(0)\n\tv_mov_b32 v20, 0x3f8ccccd\n\tv_mov_b32 v21, 0x7f7f7f7f" ::"v"(p) : "memory", LP_PROBE_CLOBBERS);
     else
         asm volatile("v_mov_b32 v0, 0\n\tv_mov_b32 v1, 0\n\tv_mov_b32 v2, 0\n\tv_mov_b32 v3, 0\n\tv_mov_b32 v4, 0\n\tv_mov_b32 v5, 0\n\t"
                      "v_mov_b32 v6, 0\n\tv_mov_b32 v7, 0\n\tv_mov_b32 v8, 0\n\tv_mov_b32 v9, 0\n\tv_mov_b32 v10, 0\n\tv_mov_b32 v11, 0\n\t"
-                     "v_mov_b32 v12, 0\n\tv_mov_b32 v13, 0\n\tv_mov_b32 v14, 0\n\tv_mov_b32 v15, 0\n\tv_mov_b32 v20, 0" ::: LP_PROBE_CLOBBERS);
+                     "v_mov_b32 v12, 0\n\tv_mov_b32 v13, 0\n\tv_mov_b32 v14, 0\n\tv_mov_b32 v15, 0\n\tv_mov_b32 v20, 0\n\tv_mov_b32 v21, 0x7f7f7f7f" ::: LP_PROBE_CLOBBERS);
     for (int i = 0; i < iters; ++i) {
         if constexpr (FMAS == 0) asm volatile(
 #include "probe_mfma_body0.inc"
@@ -196,8 +196,14 @@ __global__ __launch_bounds__(512) void probe_mfma(const uint8_t *__restrict__ op
         else if constexpr (FMAS == 6) asm volatile(
 #include "probe_mfma_body6.inc"
             ::: LP_PROBE_CLOBBERS);
-        else asm volatile(
+        else if constexpr (FMAS == 8) asm volatile(
 #include "probe_mfma_body8.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else if constexpr (FMAS == -1) asm volatile(
+#include "probe_mfma_body_scaled.inc"
+            ::: LP_PROBE_CLOBBERS);
+        else asm volatile(
+#include "probe_mfma_body_inplace.inc"
             ::: LP_PROBE_CLOBBERS);
     }
 }
@@ -261,7 +267,8 @@ extern "C" int lp_probe_copy(int to_lds, int waves, int steps, const void *src, 
 extern "C" int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream)
 {
     LP_REQUIRE(fmas_per_instruction == 0 || fmas_per_instruction == 2 || fmas_per_instruction == 4 || fmas_per_instruction == 6 ||
-                   fmas_per_instruction == 8, "lp_probe_mfma: 0, 2, 4, 6 or 8 FMAs per matrix instruction");
+                   fmas_per_instruction == 8 || (fmas_per_instruction <= -1 && fmas_per_instruction >= -4),
+               "lp_probe_mfma: 0, 2, 4, 6 or 8 FMAs per matrix instruction, or -1 .. -4");
     LP_REQUIRE(iters >= 1 && iters <= (1 << 24), "lp_probe_mfma: 1 .. 2^24 iterations");
     LP_REQUIRE(workgroups >= 1 && workgroups <= (1 << 20), "lp_probe_mfma: 1 .. 2^20 workgroups");
     LP_REQUIRE((uintptr_t)operands % 16 == 0, "lp_probe_mfma: operands must be 16-byte aligned (4096 bytes, or NULL)");
@@ -272,6 +279,10 @@ extern "C" int lp_probe_mfma(int fmas_per_instruction, int iters, const void *op
     case 2: hipLaunchKernelGGL(probe_mfma<2>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
     case 4: hipLaunchKernelGGL(probe_mfma<4>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
     case 6: hipLaunchKernelGGL(probe_mfma<6>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case -1: hipLaunchKernelGGL(probe_mfma<-1>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case -2: hipLaunchKernelGGL(probe_mfma<-2>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
+    case -3: hipLaunchKernelGGL(probe_mfma<-1>, dim3((unsigned)workgroups), dim3(256), 0, st, ops, iters); break;
+    case -4: hipLaunchKernelGGL(probe_mfma<-2>, dim3((unsigned)workgroups), dim3(256), 0, st, ops, iters); break;
     default: hipLaunchKernelGGL(probe_mfma<8>, dim3((unsigned)workgroups), dim3(512), 0, st, ops, iters); break;
     }
     return check_launch("lp_probe_mfma");

@@ -51,7 +51,9 @@ int lp_probe_stream(const void *src, int64_t read_bytes, void *dst, int64_t writ
  * LDS, no memory traffic in the loop.  operands: 4096 bytes of e4m3 codes (64 per lane) for the matrix operands, or NULL
  * for zeros.  Flops = workgroups x 8 waves x iters x 8 x 2 x 16 x 16 x 128.  It shows the rate the matrix cores hold
  * with the arithmetic of an fp32-scaled GEMM loop (four FMAs per instruction) and nothing else: the ceiling the GEMM
- * kernels' fraction of peak is to be read against.  No reference counterpart.
+ * kernels' fraction of peak is to be read against.  Negative values select the accumulate-in-place forms without FMAs:
+ * -1 the hardware-scaled instruction (unit e8m0 scale bytes) and -2 the unscaled one with 512 threads per workgroup,
+ * -3 and -4 the same two with 256 threads (one wave per SIMD; flops then count 4 waves).  No reference counterpart.
  */
 int lp_probe_mfma(int fmas_per_instruction, int iters, const void *operands, int workgroups, lp_stream_t stream);
 

@@ -50,3 +50,11 @@ def test_template_matcher_reads_operands_back():
 @pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
 def test_no_operand_lands_in_a_loop_register(capsys):
     assert _load().audit(quiet=True) == 0, capsys.readouterr().out
+
+
+def test_accumulation_registers_outside_asm_are_reported():
+    C = _load()
+    text = "\n".join(["_Z13gemm_asm_quadv:", "\tv_mov_b32 v1, 0", "\t;;#ASMSTART", "\tv_accvgpr_write_b32 a0, 0", "\t;;#ASMEND",
+                      "\tv_accvgpr_write_b32 a17, v3 ; 4-byte Folded Spill", "\t.amdhsa_accum_offset 256", "_Z5otherv:",
+                      "\tv_accvgpr_read_b32 v0, a3"])
+    assert C.accumulation_registers_outside_asm(text, "gemm_asm_quad") == ["_Z13gemm_asm_quadv: v_accvgpr_write_b32 a17, v3"]

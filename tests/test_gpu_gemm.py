@@ -650,3 +650,50 @@ def test_gemm_wide_tile_forced_on_other_shapes(G, width, shapes):
     theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
     assert theirs == mine, (theirs, mine, r.stdout[-800:])
 
+
+
+def test_gemm_four_wave_loop_equals_the_eight_wave_loop(G):
+    """The opt-in 256 x 256 loop on four waves with the accumulators in the accumulation registers (LP_GEMM_QUAD=1, read
+    once per process, hence the child): e8m0 problems of whole tiles must give the default kernel's bits (same order of
+    summation), bf16 output must be the rounded fp32 output, and the unscaled NT route through it is checked against
+    an fp32 matmul for all three output types."""
+    import hashlib
+    import os
+    import subprocess
+    import sys
+    say("gemm four-wave loop (LP_GEMM_QUAD=1 in a child process)")
+    shapes = ((4096, 4096, 512), (2048, 8192, 1024), (2560, 5120, 1536), (4096, 7168, 2048))
+    mine = []
+    for (M, N, K) in shapes:
+        xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + K, pow2=True)
+        c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+        mine.append(hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest())
+    code = (
+        "import sys, hashlib, torch\n"
+        "import gcore_lowp as G\n"
+        "sys.path.insert(0, %r)\n"
+        "from tests import test_gpu_gemm as t\n"
+        "for (M, N, K) in %r:\n"
+        "    xq, xs, wq, ws = t.quantized_problem(M, N, K, seed=M + K, pow2=True)\n"
+        "    print('[case] four waves', M, N, K, flush=True)\n"
+        "    c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())\n"
+        "    wide = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), out_dtype=torch.float32)\n"
+        "    assert torch.equal(c, wide.to(torch.bfloat16))\n"
+        "    t.check(c, t.ref_gemm(xq, xs, wq, ws), 'four waves %%s' %% ((M, N, K),))\n"
+        "    print('md5', hashlib.md5(c.view(torch.int16).cpu().numpy().tobytes()).hexdigest(), flush=True)\n"
+        "g = torch.Generator(device='cuda').manual_seed(5)\n"
+        "a = torch.randn(4096, 1024, generator=g, device='cuda').to(torch.float8_e4m3fn)\n"
+        "b = torch.randn(4096, 1024, generator=g, device='cuda').to(torch.float8_e4m3fn)\n"
+        "ref = a.float() @ b.float().T\n"
+        "for od, tol in ((torch.bfloat16, 8e-3), (torch.float32, 1e-4), (torch.float8_e4m3fn, 7e-2)):\n"
+        "    print('[case] four waves, unscaled NT', od, flush=True)\n"
+        "    c = G.gemm_impl(a, b, dtype=torch.float8_e4m3fn, out_dtype=od)\n"
+        "    r = ref.clamp(-448, 448) if od == torch.float8_e4m3fn else ref\n"
+        "    err = (c.float() - r).abs().max().item() / r.abs().max().item()\n"
+        "    assert err < tol, (od, err)\n"
+    ) % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), shapes)
+    env = dict(os.environ, LP_GEMM_QUAD="1", LP_GEMM_WIDE="0", PYTHONPATH=os.pathsep.join(p for p in sys.path if p))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
+    theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
+    assert theirs == mine, (theirs, mine, r.stdout[-800:])
