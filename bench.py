@@ -273,6 +273,13 @@ def main():
             for k in (0, 4, 8):
                 ms_p, _ = time_launches([lambda k=k, ptr=ptr: PA.check(LP.lp_probe_mfma(k, iters, ptr, wgs, stream()))], 6, 2)
                 probe[f"{tag}_{k}_fmas_per_instruction"] = {"ms": ms_p, "tflops": fl_p / ms_p / 1e9, "mfma_frac": fl_p / ms_p / 1e9 / FP8_PEAK_TFLOPS}
+        # accumulating in place, as the e8m0 loops do: the hardware-scaled form and the plain one, with two waves and with one
+        # wave per SIMD (flops follow the wave count)
+        for k, waves, tag in ((-1, 8, "hardware_scaled_in_place_2_waves_per_simd"), (-2, 8, "unscaled_in_place_2_waves_per_simd"),
+                              (-3, 4, "hardware_scaled_in_place_1_wave_per_simd"), (-4, 4, "unscaled_in_place_1_wave_per_simd")):
+            ms_p, _ = time_launches([lambda k=k: PA.check(LP.lp_probe_mfma(k, iters, rnd.data_ptr(), wgs, stream()))], 6, 2)
+            fl = fl_p * waves / 8
+            probe[f"random_e4m3_operands_{tag}"] = {"ms": ms_p, "tflops": fl / ms_p / 1e9, "mfma_frac": fl / ms_p / 1e9 / FP8_PEAK_TFLOPS}
         extras["matrix_pipe_probe_registers_only"] = probe
         # what a CU's copy path out of the L2 delivers in the loops' request shape (1 KB per wave and request, rows 7168 bytes
         # apart, one step in flight behind a wait and a barrier; 2 MB per region, L2-resident): into LDS with one 8-wave

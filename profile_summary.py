@@ -4,6 +4,8 @@
 Inputs (each a directory that one rocprofv3 run wrote with `--output-format csv -d <dir> -o run`):
   --kernel-trace DIR   a `--kernel-trace --stats` run of `python3 bench.py --no-cpu` (graph replays, as the bench times them)
   --bench-json FILE    the JSON line that same run printed
+  --floor-json FILE    the JSON line of an untraced `python3 bench.py --no-cpu` run: its floor probes beside the kernels
+                       they bound -> floor_probes_matrix_pipe_bare_stream_empty_launch.txt
   --pmc DIR [DIR ...]  `--pmc` runs of `python3 bench.py --no-cpu --no-graph --steps 4 --warmup 1`, one counter set each;
                        the sets may be any of the ones named in COUNTER_SETS below (a missing set leaves its columns empty)
 Outputs (under --out, default profiles/):
@@ -141,14 +143,85 @@ def bench_lines(b):
     return "\n".join(L)
 
 
+def floor_summary(b):
+    """The floor probes of one untraced bench run beside the kernels they bound."""
+    ex = b["extras"]
+    L = ["Floor probes: what the box gives with nothing of the kernels' own in the way, beside the kernels, one MI355X",
+         "=" * 112,
+         "Command: python3 bench.py --no-cpu > <out>.json ; python3 profile_summary.py --floor-json <out>.json      (one untraced run, one",
+         "box; times are per launch, from HIP graph replays timed with events on the launching stream; the probes are the entry",
+         "points lp_probe_mfma, lp_probe_stream and lp_probe_copy of the probe library)", ""]
+    mp = ex.get("matrix_pipe_probe_registers_only")
+    if mp:
+        L.append("1. Matrix pipe, registers only (256 workgroups, the fp8 16x16x128 instruction into eight result buffers, no LDS and no")
+        L.append("   memory traffic in the loop; TFLOP/s and fraction of 5 PFLOP/s)")
+        L.append("   %-58s %12s %12s %12s" % ("into fresh registers, k fp32 FMAs behind each", "k = 0", "k = 4", "k = 8"))
+        for tag, label in (("zero_operands", "zeros"), ("random_e4m3_operands", "random e4m3 codes")):
+            L.append("   %-58s %12s %12s %12s" % (label, *["%.0f (%.2f)" % (mp[f"{tag}_{k}_fmas_per_instruction"]["tflops"],
+                                                                        mp[f"{tag}_{k}_fmas_per_instruction"]["mfma_frac"]) for k in (0, 4, 8)]))
+        for key, v in mp.items():
+            if "in_place" in key:
+                L.append("   %-58s %12s" % (key.replace("random_e4m3_operands_", "accumulating in place, ").replace("_", " "),
+                                            "%.0f (%.2f)" % (v["tflops"], v["mfma_frac"])))
+        d2 = ex.get("deep_k_gemm_4096x7168x18432_e8m0_scales", {})
+        L.append("   In the same run: config 2 with fp32 scales (four FMAs per instruction) %.0f TFLOP/s = %.3f of peak; with e8m0 scales %.0f;"
+                 % (b["value"], b["roofline"]["frac"], ex.get("c2_gemm_e8m0_scales", {}).get("tflops", float("nan"))))
+        L.append("   deep K 4096 x 7168 x 18432: %.0f / %.0f." % (ex.get("deep_k_gemm_4096x7168x18432_fp32_scales", {}).get("tflops", float("nan")),
+                                                                   d2.get("tflops", float("nan"))))
+        L.append("")
+    for n, (tag, ptag, what) in enumerate((("c3_skinny_gemm", "c3_floor_probe", "config 3: M = 64, N = 4096, K = 7168"),
+                                          ("decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", "M = 64, N = 18432, K = 7168")), 2):
+        if tag in ex and ptag in ex:
+            pr = ex[ptag]
+            L.append(f"{n}. Decode GEMM ({what}) against an empty launch and a bare read of its weight bytes")
+            L.append("   empty launch %37.2f us" % pr["empty_launch_us"])
+            for k, v in pr.items():
+                if k.startswith("read_"):
+                    L.append("   bare %-44s %6.2f us" % (k[:-3].replace("_", " "), v))
+            L.append("   the kernel %39.2f us = %.2f x the best bare read (%.0f GB/s)" % (ex[tag]["ms"] * 1e3, pr["gemm_over_bare_read"], pr["bare_read_best_GB/s"]))
+            L.append("")
+    if "c1_floor_probe" in ex:
+        c1 = ex["c1_floor_probe"]
+        L.append("4. 128 x 128 tile quantiser / dequantiser (config 1: 4096 x 4096, 32 MiB + 16 MiB) against a bare stream of the same bytes")
+        for w in (512, 1024, 2048, 4096):
+            L.append("   bare stream, %4d workgroups: read 32 MiB + write 16 MiB %6.2f us, read 16 MiB + write 32 MiB %6.2f us"
+                     % (w, c1[f"read32MiB_write16MiB_{w}_workgroups_us"], c1[f"read16MiB_write32MiB_{w}_workgroups_us"]))
+        L.append("   quant_tile128    %6.2f us = %.2f x the best bare stream (%.3f of 8 TB/s; the bare stream %.3f)"
+                 % (ex["c1_quant_128x128"]["ms"] * 1e3, c1["quant_over_bare_stream"], ex["c1_quant_128x128"]["hbm_frac"], c1["bare_stream_hbm_frac"]["read32_write16"]))
+        L.append("   dequant_fp8_fast %6.2f us = %.2f x the best bare stream (%.3f of 8 TB/s; the bare stream %.3f)"
+                 % (ex["c1_dequant_128x128"]["ms"] * 1e3, c1["dequant_over_bare_stream"], ex["c1_dequant_128x128"]["hbm_frac"], c1["bare_stream_hbm_frac"]["read16_write32"]))
+        L.append("")
+    if "c5_floor_probe" in ex:
+        c5 = ex["c5_floor_probe"]
+        L.append("5. FP4 -> FP8 fused over a whole MoE layer (config 5) against a bare stream of the same mix (0.5 byte read, 1 byte")
+        L.append("   written per element; the kernel also reads 1/32 byte of scales per element)")
+        for k, v in c5.items():
+            if k.endswith("_workgroups_ms"):
+                L.append("   bare stream, %6s workgroups %8.3f ms" % (k.split("_")[-3], v))
+        L.append("   fp4_amax (three launches)     %8.3f ms = %.3f x the best bare stream (%.3f of 8 TB/s; the bare stream %.3f)"
+                 % (ex["c5_fp4_to_fp8_fused"]["ms_total"], c5["fused_over_bare_stream"], ex["c5_fp4_to_fp8_fused"]["hbm_frac"], c5["bare_stream_hbm_frac"]))
+        L.append("")
+    if "l2_to_cu_copy_probe" in ex:
+        L.append("6. Operand copies out of the L2 alone (every wave issues eight 1 KB requests per step, 8 rows x 128 bytes with rows 7168")
+        L.append("   bytes apart, one step in flight behind a wait and a workgroup barrier; 2 MB per region, L2-resident after the first pass)")
+        for k, v in ex["l2_to_cu_copy_probe"].items():
+            L.append("   %-46s %6.1f B/ns per CU = %5.1f TB/s over the chip" % (k.replace("_", " "), v["bytes_per_ns_per_cu"], v["TB/s"]))
+        L.append("   What the GEMM loops ask of that path: the 256 x 288 tile 68 KB per %.2f us step = %.0f B/ns per CU (config 2)."
+                 % (b["roofline"]["launch_ms"] * 1e3 / 112, 68 * 1024 / (b["roofline"]["launch_ms"] * 1e3 / 112) / 1e3))
+    return "\n".join(L) + "\n"
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--kernel-trace")
     ap.add_argument("--bench-json")
+    ap.add_argument("--floor-json")
     ap.add_argument("--pmc", nargs="*", default=[])
     ap.add_argument("--out", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles"))
     args = ap.parse_args()
     os.makedirs(args.out, exist_ok=True)
+    if args.floor_json:
+        open(os.path.join(args.out, "floor_probes_matrix_pipe_bare_stream_empty_launch.txt"), "w").write(floor_summary(json.load(open(args.floor_json))))
     pmc = read_pmc(args.pmc)
     per, stats = read_trace(args.kernel_trace) if args.kernel_trace else ({}, [])
 
