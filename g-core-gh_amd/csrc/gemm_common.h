@@ -77,6 +77,9 @@ int launch_rowscale_asm(const void *Aq, const void *As, const void *Bq, const vo
 constexpr int kSkinnyBlocks = 7;          // K blocks one workgroup handles
 // at most 16 activation rows: one workgroup per 16 weight rows over all of K (gemm_thin.hip)
 bool thin_ok(int64_t M, int64_t N, int64_t K);
+bool thin_rows_ok(int64_t M, int64_t N, int64_t K);
+int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
+                     void *C, int out_dtype, hipStream_t st);
 int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                 void *C, int out_dtype, hipStream_t st);
 void skinny_plan(int64_t N, int64_t K, int &splits, int &per);

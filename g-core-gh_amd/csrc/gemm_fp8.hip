@@ -512,6 +512,7 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     // the single-launch kernels above and the 128-row tile kernel exist it is level with them or behind (two launches).
     static const bool no_skinny = getenv("LP_GEMM_SKINNY") == nullptr || getenv("LP_GEMM_NO_SKINNY") != nullptr;
     static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;           // tuning aid
+    if (!no_thin && gemm::thin_rows_ok(M, N, K)) return gemm::launch_thin_rows(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, st);
     if (!no_thin && gemm::thin_ok(M, N, K)) return gemm::launch_thin(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, out_dtype, st);
     if (M <= 64 && !no_skinny) {
         // decode-sized: the weight-streaming kernel, when the caller gave scratch for its K ranges and one range
@@ -660,7 +661,7 @@ extern "C" int lp_gemm_fp8_block_static(const void *Aq, const void *As, const vo
     // it, so the buffer's previous contents never matter and nothing is cleared).
     // (decode shapes are served by the single-launch kernels before the K split is considered: no scratch, never refused)
     static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;
-    const int64_t need = !no_thin && gemm::thin_ok(M, N, K) ? 0 : split_bytes(M, N, K);
+    const int64_t need = !no_thin && (gemm::thin_ok(M, N, K) || gemm::thin_rows_ok(M, N, K)) ? 0 : split_bytes(M, N, K);
     LP_REQUIRE(need <= kStaticScratchBytes,
                "lp_gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of K-split scratch, the built-in buffer holds %lld; "
                "call lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes()",

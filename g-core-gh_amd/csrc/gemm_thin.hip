@@ -440,6 +440,224 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// 17 to 64 activation rows against many weight rows (more than one group of 16 per CU): a workgroup owns 8 R weight
+// rows (R = 4 .. 10: N / (8 R) workgroups, e.g. 256 of 72 rows for N = 18432) over the whole of K, so the 64 activation
+// rows a workgroup pulls through its CU's copy path are shared by 4 R / 8 times the weight bytes of the 16-row cut.
+// Same scheme as gemm_thin_ring2 otherwise: the 8 waves take runs of PER K blocks, wave-private rings fed by LDS-direct
+// loads (a request = 8 rows x 128 bytes), hand-counted waits, no barrier inside the loop, partial sums added through LDS
+// in wave order.  A K block of a wave is R weight requests (one block in flight: R KB) and two activation units of 32
+// rows (4 requests each, two units in flight), 144 KB per workgroup at R = 10.  The rows are cut into (R + 1) / 2 blocks
+// of 16 for the matrix instruction; with odd R the last block's upper 8 rows are never loaded and its upper 8 columns
+// never stored (a column of the result depends on its own weight row only).  8 R is not a multiple of 128, so a
+// block of 16 rows can straddle two weight-scale blocks: every lane takes the scale of its own four columns.
+template <int PER, int R>
+struct RowsPlan {
+    int a_end[PER * 2];          // requests issued up to and including activation unit u
+    int b_end[PER];              // ... weight block j
+    int before[PER * 2];         // requests issued before the wait of step u
+    constexpr RowsPlan() : a_end{}, b_end{}, before{}
+    {
+        int n = R;
+        b_end[0] = n;
+        for (int u = 0; u < 2; ++u) { n += 4; a_end[u] = n; }
+        for (int u = 0; u < PER * 2; ++u) {
+            before[u] = n;
+            if (u + 2 < PER * 2) { n += 4; a_end[u + 2] = n; }
+            if (u % 2 == 0 && u / 2 + 1 < PER) { n += R; b_end[u / 2 + 1] = n; }
+        }
+    }
+};
+
+template <int SDT, int PER, int R>
+__global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
+                                                                  const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
+                                                                  int M, int64_t N, int64_t K, void *__restrict__ C,
+                                                                  int out_dtype)
+{
+    constexpr int MB = 4, NBK = (R + 1) / 2, UNITS = PER * 2;
+    constexpr int SV = (16 * MB * kThinWaves * kThinRun + 64 * kThinWaves - 1) / (64 * kThinWaves);      // table entries per lane
+    constexpr int WAVE_LDS = R * 1024 + 2 * 4096;
+    constexpr RowsPlan<PER, R> plan{};
+    __shared__ __attribute__((aligned(1024))) uint8_t ring[kThinWaves * WAVE_LDS];       // per wave: R KB of weights, two activation units
+    __shared__ float sSa[SV * 64 * kThinWaves];          // activation scales, [row][K block] as in memory
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int kblocks = (int)(K / 128);
+    const int64_t n0 = (int64_t)blockIdx.x * (8 * R);
+    const int kb0 = wave * PER;
+
+    uint32_t sv[SV];
+#pragma unroll
+    for (int q = 0; q < SV; ++q) {
+        const int i = t + 64 * kThinWaves * q;
+        const int last = M * kblocks - 1;
+        const int idx = i < last ? i : last;
+        if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
+        else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
+    }
+
+    const int ld_row = lane >> 3, chunk = (lane & 7) ^ ld_row;
+    uint8_t *wb = ring + wave * WAVE_LDS, *wa = wb + R * 1024;
+    // weight rows past the end of the matrix (last workgroup) are read from the last row and never stored
+    uint32_t boff[R];                                    // N K < 2^32 (checked on the host)
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int64_t row = n0 + 8 * i + ld_row;
+        boff[i] = (uint32_t)((row < N ? row : N - 1) * K + chunk * 16);
+    }
+    auto request_b = [&](int j) {
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+#pragma unroll
+        for (int i = 0; i < R; ++i)              // read once by the whole launch: streamed past the L2's resident lines
+            __builtin_amdgcn_global_load_lds(GLB_PTR(Bq + boff[i] + (uint32_t)kb * 128u), LDS_PTR(wb + i * 1024), 16, 0, 2);
+    };
+    auto request_a = [&](int u) {                        // unit u: rows 32 (u % 2) .. + 31 of block u / 2
+        const int j = u / 2, v = u % 2;
+        const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+        uint8_t *dst = wa + v * 4096;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = 32 * v + 8 * i + ld_row;
+            const uint8_t *src = Aq + (int64_t)(row < M ? row : M - 1) * K + chunk * 16 + (int64_t)kb * 128;
+            __builtin_amdgcn_global_load_lds(GLB_PTR(src), LDS_PTR(dst + i * 1024), 16, 0, 0);
+        }
+    };
+    request_b(0);
+    request_a(0);
+    request_a(1);
+
+    // weight scales of the lane's own four columns of every block of 16
+    float sb[NBK][PER];
+    const int64_t last_blk = (N >> 7) - 1;
+#pragma unroll
+    for (int nb = 0; nb < NBK; ++nb) {
+        int64_t blk = (n0 + 16 * nb + 4 * lq) >> 7;
+        if (blk > last_blk) blk = last_blk;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+            sb[nb][j] = gemm::scale_at<SDT>(Bs, blk * kblocks + kb);
+        }
+    }
+    const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R + 8) : "memory");          // the table requests are the oldest
+#pragma unroll
+    for (int q = 0; q < SV; ++q) {
+        asm volatile("" : "+v"(sv[q]));
+        if (SDT != LP_F32) sv[q] = sv[q] == 0u ? 0x00400000u : (sv[q] == 0xFFu ? 0x7FC00000u : sv[q] << 23);       // e8m0 -> fp32 bits
+        asm volatile("ds_write_b32 %0, %1" ::"v"(ssa0 + 4 * (t + 64 * kThinWaves * q)), "v"(sv[q]) : "memory");
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float sa[MB][PER];
+#pragma unroll
+    for (int g = 0; g < MB; ++g) {
+        const int m = 16 * g + l16 < M ? 16 * g + l16 : M - 1;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
+            asm volatile("ds_read_b32 %0, %1" : "=v"(sa[g][j]) : "v"(ssa0 + 4 * (m * kblocks + kb)));
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < MB; ++g)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sa[g][j])::"memory");
+            if (kb0 + j >= kblocks) sa[g][j] = 0.0f;     // a K block past the end (the last wave's run) adds nothing
+        }
+    // the weight scales are in their registers before the loop: inside it every wait on the request counter is counted by hand
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int nb = 0; nb < NBK; ++nb)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) asm volatile("" : "+v"(sb[nb][j]));
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint32_t rdo0 = l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rdo1 = l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
+    const uint32_t wb0 = (uint32_t)(uintptr_t)LDS_PTR(wb), wa0 = (uint32_t)(uintptr_t)LDS_PTR(wa);
+    f32x4v acc[MB][NBK];
+#pragma unroll
+    for (int g = 0; g < MB; ++g)
+#pragma unroll
+        for (int nb = 0; nb < NBK; ++nb) acc[g][nb] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+    const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    i32x8 wf[NBK];                                       // weight fragments of the current block, kept over its two units
+    auto step = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, j = u / 2, v = u % 2;
+        constexpr int need = (v == 0 && plan.b_end[j] > plan.a_end[u]) ? plan.b_end[j] : plan.a_end[u];
+        wait_requests<plan.before[u] - need>();
+        const uint32_t ao = wa0 + v * 4096;
+        u32x4 x0 = lds_read16(ao + rdo0), x1 = lds_read16(ao + rdo1);
+        u32x4 y0 = lds_read16(ao + 2048 + rdo0), y1 = lds_read16(ao + 2048 + rdo1);
+        u32x4 w0[NBK], w1[NBK];
+        if constexpr (v == 0) {
+#pragma unroll
+            for (int nb = 0; nb < NBK; ++nb) { w0[nb] = lds_read16(wb0 + nb * 2048 + rdo0); w1[nb] = lds_read16(wb0 + nb * 2048 + rdo1); }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x0), "+v"(x1), "+v"(y0), "+v"(y1)::"memory");
+        if constexpr (v == 0) {
+#pragma unroll
+            for (int nb = 0; nb < NBK; ++nb) {
+                asm volatile("" : "+v"(w0[nb]), "+v"(w1[nb]));          // used after the wait above, not before
+                wf[nb] = i32x8{(int)w0[nb].x, (int)w0[nb].y, (int)w0[nb].z, (int)w0[nb].w, (int)w1[nb].x, (int)w1[nb].y, (int)w1[nb].z, (int)w1[nb].w};
+            }
+        }
+        if constexpr (u + 2 < UNITS) request_a(u + 2);
+        if constexpr (v == 0 && j + 1 < PER) request_b(j + 1);
+        const i32x8 af0 = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        const i32x8 af1 = {(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+#pragma unroll
+        for (int nb = 0; nb < NBK; ++nb) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                constexpr int g0 = 2 * v;
+                const int g = g0 + h;
+                const f32x4v p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[nb], h ? af1 : af0, zero, 0, 0, 0, 0, 0, 0);
+                const float sc = sa[g][j] * sb[nb][j];
+                acc[g][nb].x = __builtin_fmaf(p.x, sc, acc[g][nb].x);
+                acc[g][nb].y = __builtin_fmaf(p.y, sc, acc[g][nb].y);
+                acc[g][nb].z = __builtin_fmaf(p.z, sc, acc[g][nb].z);
+                acc[g][nb].w = __builtin_fmaf(p.w, sc, acc[g][nb].w);
+            }
+        }
+    };
+    unrolled(step, std::make_integer_sequence<int, UNITS>{});
+
+    // partial sums through the (drained) rings, two row groups at a time: pair (g, nb) of the pass is added up by wave
+    // pair % 8 over the waves in their order
+    f32x4v *red = (f32x4v *)ring;                        // [wave][2 NBK][lane], 2 NBK KB per wave <= R + 8 KB
+    static_assert(2 * NBK * 1024 <= WAVE_LDS, "a wave's partial sums of a pass fit its own ring");
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        __syncthreads();                                 // every wave is done with its ring (or with the previous pass)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int nb = 0; nb < NBK; ++nb) red[(wave * (WAVE_LDS / 1024) + h * NBK + nb) * 64 + lane] = acc[2 * pass + h][nb];
+        __syncthreads();
+        for (int pair = wave; pair < 2 * NBK; pair += kThinWaves) {
+            const int h = pair / NBK, nb = pair % NBK;
+            f32x4v sum = red[(h * NBK + nb) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < kThinWaves; ++w) {
+                const f32x4v x = red[(w * (WAVE_LDS / 1024) + h * NBK + nb) * 64 + lane];
+                sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+            }
+            const int row = 16 * (2 * pass + h) + l16, col = 16 * nb + 4 * lq;
+            const int64_t n = n0 + col;
+            if (row >= M || col >= 8 * R || n >= N) continue;
+            if (out_dtype == LP_BF16) {
+                const u32x2 o = {pack_bf16(sum.x, sum.y), pack_bf16(sum.z, sum.w)};
+                *(u32x2 *)((uint16_t *)C + (int64_t)row * N + n) = o;
+            } else {
+                *(f32x4v *)((float *)C + (int64_t)row * N + n) = sum;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 namespace lowp {
@@ -454,6 +672,64 @@ bool thin_ok(int64_t M, int64_t N, int64_t K)
     if (M < 1 || M > 64 || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun) return false;
     const int64_t groups = N / 16;
     return groups >= 192 && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
+}
+
+// 17 .. 64 activation rows against more weight rows than one 16-row workgroup per CU: 8 R rows per workgroup, R from {4, 6, 8, 9,
+// 10} such that the rounds of 256 workgroups times R are fewest (18432 rows: R = 9, 256 workgroups).
+// Groups of 16 weight rows from which the many-rows kernel takes over from the 16-row cut at more than 16 activation rows
+// (one MI355X, M = 64, K = 7168, us per call, 16-row cut or 128 x 128 tiles -> 8 R rows: N = 6144 23.1 -> 16.9, 8192 24.2 ->
+// 17.8, 12288 36.3 -> 22.0, 18432 38.4 -> 29.3, 36864 73.3 -> 60.7; N = 4096 is one 16-row workgroup per CU either way).
+constexpr int64_t kRowsFromGroups = 256;
+
+bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
+{
+    static const bool off = getenv("LP_GEMM_THIN_ROWS") && atoi(getenv("LP_GEMM_THIN_ROWS")) == 0;       // tuning aid
+    static const int64_t min_groups = getenv("LP_GEMM_THIN_ROWS_FROM") ? atoi(getenv("LP_GEMM_THIN_ROWS_FROM")) : kRowsFromGroups;
+    return !off && M > 16 && M <= 64 && N % 16 == 0 && K % 128 == 0 && K / 128 <= kThinWaves * kThinRun && N / 16 > min_groups &&
+           N * K < 0xFFFFFFFFll;
+}
+
+template <int SDT, int PER, int R>
+void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
+                        int out_dtype, hipStream_t st)
+{
+    const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
+    hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K, C,
+                       out_dtype);
+}
+
+template <int SDT, int PER>
+void launch_thin_rows_per(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
+                          int out_dtype, int per, int r, hipStream_t st)
+{
+    if constexpr (PER > 1) {
+        if (per < PER) return launch_thin_rows_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, r, st);
+    }
+    switch (r) {
+    case 4: return launch_thin_rows_r<SDT, PER, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    case 6: return launch_thin_rows_r<SDT, PER, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    case 8: return launch_thin_rows_r<SDT, PER, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    case 9: return launch_thin_rows_r<SDT, PER, 9>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    default: return launch_thin_rows_r<SDT, PER, 10>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    }
+}
+
+int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
+                     void *C, int out_dtype, hipStream_t st)
+{
+    static const int forced = getenv("LP_GEMM_THIN_ROWS") ? atoi(getenv("LP_GEMM_THIN_ROWS")) : 0;     // tuning aid: 4, 6, 8, 9, 10
+    const int kblocks = (int)(K / 128);
+    const int per = (kblocks + kThinWaves - 1) / kThinWaves;
+    int best = 10;
+    int64_t best_cost = INT64_MAX;
+    for (int r : {4, 6, 8, 9, 10}) {
+        const int64_t wgs = (N + 8 * r - 1) / (8 * r), cost = ((wgs + 255) / 256) * r;
+        if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
+    }
+    if (forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) best = forced;
+    if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
+    else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
+    return check_launch("lp_gemm_fp8_block(thin, many rows)");
 }
 
 template <int SDT, int PER>

@@ -697,3 +697,22 @@ def test_gemm_four_wave_loop_equals_the_eight_wave_loop(G):
     assert r.returncode == 0, (r.stdout[-1500:], r.stderr[-1500:])
     theirs = [l.split()[1] for l in r.stdout.splitlines() if l.startswith("md5 ")]
     assert theirs == mine, (theirs, mine, r.stdout[-800:])
+
+
+@pytest.mark.parametrize("shape", [(64, 18432, 7168), (17, 18432, 1024), (33, 16384, 2048), (48, 12288, 896), (64, 8320, 512), (64, 6144, 7168), (20, 7168, 2048),
+                                   (40, 18560, 3584), (64, 36864, 1536)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
+def test_gemm_decode_rows_against_many_weight_rows(G, shape, pow2):
+    """17 .. 64 activation rows against more than 4096 weight rows: the kernel that gives a workgroup 8 R weight rows
+    (R = 4 .. 10, chosen from N), so rows per workgroup that are not a multiple of 16 (R = 9), a last workgroup with
+    rows missing (18560 = 257 x 72 + 56), runs of 1 .. 7 K blocks per wave including a last wave with fewer (896 = 7
+    blocks over 8 waves), blocks of 16 rows that straddle two weight-scale blocks."""
+    M, N, K = shape
+    xq, xs, wq, ws = quantized_problem(M, N, K, seed=M + N + K, pow2=pow2)
+    say("decode rows", shape, "e8m0" if pow2 else "f32")
+    c = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda())
+    wide = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), out_dtype=torch.float32)
+    assert torch.equal(c, wide.to(torch.bfloat16))
+    check(c, ref_gemm(xq, xs, wq, ws), f"decode rows {shape}")
+    assert torch.equal(c, G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda()))
