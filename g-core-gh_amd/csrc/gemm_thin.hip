@@ -441,7 +441,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// 17 to 64 activation rows against many weight rows (more than one group of 16 per CU): a workgroup owns 8 R weight
+// 9 to 64 activation rows against many weight rows (more than one group of 16 per CU): a workgroup owns 8 R weight
 // rows (R = 4 .. 10: N / (8 R) workgroups, e.g. 256 of 72 rows for N = 18432) over the whole of K, so the 64 activation
 // rows a workgroup pulls through its CU's copy path are shared by 4 R / 8 times the weight bytes of the 16-row cut.
 // Same scheme as gemm_thin_ring2 otherwise: the 8 waves take runs of PER K blocks, wave-private rings fed by LDS-direct
@@ -451,34 +451,35 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 // of 16 for the matrix instruction; with odd R the last block's upper 8 rows are never loaded and its upper 8 columns
 // never stored (a column of the result depends on its own weight row only).  8 R is not a multiple of 128, so a
 // block of 16 rows can straddle two weight-scale blocks: every lane takes the scale of its own four columns.
-template <int PER, int R>
+// U: activation units of 32 rows per K block (1 for at most 32 activation rows, 2 up to 64); two units are in flight.
+template <int PER, int R, int U>
 struct RowsPlan {
-    int a_end[PER * 2];          // requests issued up to and including activation unit u
+    int a_end[PER * U];          // requests issued up to and including activation unit u
     int b_end[PER];              // ... weight block j
-    int before[PER * 2];         // requests issued before the wait of step u
+    int before[PER * U];         // requests issued before the wait of step u
     constexpr RowsPlan() : a_end{}, b_end{}, before{}
     {
         int n = R;
         b_end[0] = n;
-        for (int u = 0; u < 2; ++u) { n += 4; a_end[u] = n; }
-        for (int u = 0; u < PER * 2; ++u) {
+        for (int u = 0; u < 2 && u < PER * U; ++u) { n += 4; a_end[u] = n; }
+        for (int u = 0; u < PER * U; ++u) {
             before[u] = n;
-            if (u + 2 < PER * 2) { n += 4; a_end[u + 2] = n; }
-            if (u % 2 == 0 && u / 2 + 1 < PER) { n += R; b_end[u / 2 + 1] = n; }
+            if (u + 2 < PER * U) { n += 4; a_end[u + 2] = n; }
+            if (u % U == 0 && u / U + 1 < PER) { n += R; b_end[u / U + 1] = n; }
         }
     }
 };
 
-template <int SDT, int PER, int R>
+template <int SDT, int PER, int R, int U = 2>
 __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                                   int M, int64_t N, int64_t K, void *__restrict__ C,
                                                                   int out_dtype)
 {
-    constexpr int MB = 4, NBK = (R + 1) / 2, UNITS = PER * 2;
+    constexpr int MB = 2 * U, NBK = (R + 1) / 2, UNITS = PER * U, A0 = UNITS < 2 ? UNITS : 2;
     constexpr int SV = (16 * MB * kThinWaves * kThinRun + 64 * kThinWaves - 1) / (64 * kThinWaves);      // table entries per lane
     constexpr int WAVE_LDS = R * 1024 + 2 * 4096;
-    constexpr RowsPlan<PER, R> plan{};
+    constexpr RowsPlan<PER, R, U> plan{};
     __shared__ __attribute__((aligned(1024))) uint8_t ring[kThinWaves * WAVE_LDS];       // per wave: R KB of weights, two activation units
     __shared__ float sSa[SV * 64 * kThinWaves];          // activation scales, [row][K block] as in memory
     const int t = threadIdx.x, lane = t & 63;
@@ -513,10 +514,10 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
         for (int i = 0; i < R; ++i)              // read once by the whole launch: streamed past the L2's resident lines
             __builtin_amdgcn_global_load_lds(GLB_PTR(Bq + boff[i] + (uint32_t)kb * 128u), LDS_PTR(wb + i * 1024), 16, 0, 2);
     };
-    auto request_a = [&](int u) {                        // unit u: rows 32 (u % 2) .. + 31 of block u / 2
-        const int j = u / 2, v = u % 2;
+    auto request_a = [&](int u) {                        // unit u: rows 32 (u % U) .. + 31 of block u / U, into slot u % 2
+        const int j = u / U, v = u % U;
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
-        uint8_t *dst = wa + v * 4096;
+        uint8_t *dst = wa + (u % 2) * 4096;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = 32 * v + 8 * i + ld_row;
@@ -525,8 +526,8 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
         }
     };
     request_b(0);
-    request_a(0);
-    request_a(1);
+#pragma unroll
+    for (int u = 0; u < A0; ++u) request_a(u);
 
     // weight scales of the lane's own four columns of every block of 16
     float sb[NBK][PER];
@@ -542,7 +543,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
         }
     }
     const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R + 8) : "memory");          // the table requests are the oldest
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R + 4 * A0) : "memory");          // the table requests are the oldest
 #pragma unroll
     for (int q = 0; q < SV; ++q) {
         asm volatile("" : "+v"(sv[q]));
@@ -583,12 +584,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
 #pragma unroll
         for (int nb = 0; nb < NBK; ++nb) acc[g][nb] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
     const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    i32x8 wf[NBK];                                       // weight fragments of the current block, kept over its two units
+    i32x8 wf[NBK];                                       // weight fragments of the current block, kept over its units
     auto step = [&](auto uc) {
-        constexpr int u = decltype(uc)::value, j = u / 2, v = u % 2;
+        constexpr int u = decltype(uc)::value, j = u / U, v = u % U;
         constexpr int need = (v == 0 && plan.b_end[j] > plan.a_end[u]) ? plan.b_end[j] : plan.a_end[u];
         wait_requests<plan.before[u] - need>();
-        const uint32_t ao = wa0 + v * 4096;
+        const uint32_t ao = wa0 + (u % 2) * 4096;
         u32x4 x0 = lds_read16(ao + rdo0), x1 = lds_read16(ao + rdo1);
         u32x4 y0 = lds_read16(ao + 2048 + rdo0), y1 = lds_read16(ao + 2048 + rdo1);
         u32x4 w0[NBK], w1[NBK];
@@ -630,7 +631,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
     f32x4v *red = (f32x4v *)ring;                        // [wave][2 NBK][lane], 2 NBK KB per wave <= R + 8 KB
     static_assert(2 * NBK * 1024 <= WAVE_LDS, "a wave's partial sums of a pass fit its own ring");
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < U; ++pass) {
         __syncthreads();                                 // every wave is done with its ring (or with the previous pass)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
@@ -674,7 +675,7 @@ bool thin_ok(int64_t M, int64_t N, int64_t K)
     return groups >= 192 && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
 }
 
-// 17 .. 64 activation rows against more weight rows than one 16-row workgroup per CU: 8 R rows per workgroup, R from {4, 6, 8, 9,
+// 9 .. 64 activation rows against more weight rows than one 16-row workgroup per CU: 8 R rows per workgroup, R from {4, 6, 8, 9,
 // 10} such that the rounds of 256 workgroups times R are fewest (18432 rows: R = 9, 256 workgroups).
 // Groups of 16 weight rows from which the many-rows kernel takes over from the 16-row cut at more than 16 activation rows
 // (one MI355X, M = 64, K = 7168, us per call, 16-row cut or 128 x 128 tiles -> 8 R rows: N = 6144 23.1 -> 16.9, 8192 24.2 ->
@@ -685,7 +686,10 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
 {
     static const bool off = getenv("LP_GEMM_THIN_ROWS") && atoi(getenv("LP_GEMM_THIN_ROWS")) == 0;       // tuning aid
     static const int64_t min_groups = getenv("LP_GEMM_THIN_ROWS_FROM") ? atoi(getenv("LP_GEMM_THIN_ROWS_FROM")) : kRowsFromGroups;
-    return !off && M > 16 && M <= 64 && N % 16 == 0 && K % 128 == 0 && K / 128 <= kThinWaves * kThinRun && N / 16 > min_groups &&
+    // from 9 activation rows: at 16 rows it is 8 % ahead of the 16-row ring kernel from N = 18432 (28.2 -> 25.9 us at K = 7168),
+    // at 8 rows level with it (25.1 / 25.5), at 1 row behind (23.6 / 25.4)
+    static const int64_t min_m = getenv("LP_GEMM_THIN_ROWS_MIN_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MIN_M")) : 9;
+    return !off && M >= min_m && M <= 64 && N % 16 == 0 && K % 128 == 0 && K / 128 <= kThinWaves * kThinRun && N / 16 > min_groups &&
            N * K < 0xFFFFFFFFll;
 }
 
@@ -694,8 +698,12 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
                         int out_dtype, hipStream_t st)
 {
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
-    hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K, C,
-                       out_dtype);
+    if (M <= 32)
+        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype);
+    else
+        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 2>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype);
 }
 
 template <int SDT, int PER>

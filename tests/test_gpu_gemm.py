@@ -699,12 +699,12 @@ def test_gemm_four_wave_loop_equals_the_eight_wave_loop(G):
     assert theirs == mine, (theirs, mine, r.stdout[-800:])
 
 
-@pytest.mark.parametrize("shape", [(64, 18432, 7168), (17, 18432, 1024), (33, 16384, 2048), (48, 12288, 896), (64, 8320, 512), (64, 6144, 7168), (20, 7168, 2048),
+@pytest.mark.parametrize("shape", [(64, 18432, 7168), (17, 18432, 1024), (16, 18432, 7168), (9, 8192, 1024), (33, 16384, 2048), (48, 12288, 896), (64, 8320, 512), (64, 6144, 7168), (20, 7168, 2048),
                                    (40, 18560, 3584), (64, 36864, 1536)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_gemm_decode_rows_against_many_weight_rows(G, shape, pow2):
-    """17 .. 64 activation rows against more than 4096 weight rows: the kernel that gives a workgroup 8 R weight rows
+    """9 .. 64 activation rows against more than 4096 weight rows: the kernel that gives a workgroup 8 R weight rows
     (R = 4 .. 10, chosen from N), so rows per workgroup that are not a multiple of 16 (R = 9), a last workgroup with
     rows missing (18560 = 257 x 72 + 56), runs of 1 .. 7 K blocks per wave including a last wave with fewer (896 = 7
     blocks over 8 waves), blocks of 16 rows that straddle two weight-scale blocks."""
