@@ -637,23 +637,26 @@ def main():
         fnw = lambda: chk(L.lp_gemm_fp8_rowscale(a_w.data_ptr(), sa_w.data_ptr(), b_w.data_ptr(), sb_w.data_ptr(), A.E8M0,  # noqa: E731
                                                  4096, 7168, Pw, dw.data_ptr(), A.BF16, stream()))
         msw, _ = time_launches([fnw], 10, 3)
-        # the whole layer's weight gradient in one (two) launches: 256 problems [4096, 7168] x P_e, config 4's rows per
-        # expert padded as the wrapper pads them; operands are random codes (the time does not depend on the values), 15 GB of bf16 out
-        from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad
-        padw = choose_colwise_pad(m_splits.tolist())                   # rows the wrapper pads every expert to (512 here)
-        nblkw = [(int(m) + padw - 1) // padw * (padw // 128) for m in m_splits.tolist()]
+        # the whole layer's weight gradient, one launch per kind of problem (K a multiple of 512; one K block; two K blocks):
+        # 256 problems [4096, 7168] x P_e, config 4's rows per expert padded as the wrapper pads them (experts of at most 256
+        # rows to 128 or 256, the others to multiples of 512); operands are random codes (the time does not depend on the
+        # values), 15 GB of bf16 out
+        from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad, padded_blocks
+        padw = choose_colwise_pad(m_splits.tolist())
+        nblkw = [padded_blocks(int(m), padw) for m in m_splits.tolist()]
         pbw = sum(nblkw)
-        pre, fast, rest = 0, [], []
+        pre, fast, one, two, rest = 0, [], [], [], []
         for e, nb in enumerate(nblkw):
             if nb:
-                (fast if nb % 4 == 0 else rest).append((e, nb, pre, 0))
+                (fast if nb % 4 == 0 else one if nb == 1 else two if nb == 2 else rest).append((e, nb, pre, 0))
             pre += nb
         aT = torch.randint(0, 120, (4096 * pbw * 128,), dtype=torch.uint8, device=dev)
         bT = torch.randint(0, 120, (7168 * pbw * 128,), dtype=torch.uint8, device=dev)
         saT = torch.full((4096 * pbw,), 120, dtype=torch.uint8, device=dev)
         sbT = torch.full((7168 * pbw,), 121, dtype=torch.uint8, device=dev)
         dW = torch.empty(E4, 4096, 7168, dtype=torch.bfloat16, device=dev)
-        tabs = [(torch.tensor(g, dtype=torch.int32, device=dev), len(g), max(x[1] for x in g), mult) for g, mult in ((fast, 4), (rest, 1)) if g]
+        tabs = [(torch.tensor(g, dtype=torch.int32, device=dev), len(g), max(x[1] for x in g), mult)
+                for g, mult in ((fast, 4), (one, 1), (two, 2), (rest, 1)) if g]
 
         def fng():
             for tab, n, mx, mult in tabs:
@@ -661,13 +664,17 @@ def main():
                                                    mult, 4096, 7168, dW.data_ptr(), A.BF16, stream()))
         msg, _ = time_launches([fng], 3, 1)
         flg = 2.0 * 4096 * 7168 * pbw * 128
+        n_launches_w = len(tabs)
         del aT, bT, saT, sbT, dW, tabs
         extras["grouped_linear_backward"] = {
             "dgrad_grouped_256_experts_65536x4096_to_7168": dgrad_res,
-            "wgrad_grouped_256_experts_4096x7168": {"ms": msg, "rows_padded_to": padw, "tflops_on_padded_rows": flg / msg / 1e9,
+            "wgrad_grouped_256_experts_4096x7168": {"ms": msg, "rows_padded_to": "128 up to 256 rows, 512 beyond" if padw == 0 else padw,
+                                                    "problems_by_kernel": {"k_multiple_of_512": len(fast), "one_k_block": len(one),
+                                                                           "two_k_blocks": len(two), "other": len(rest)},
+                                                    "tflops_on_padded_rows": flg / msg / 1e9,
                                                     "mfma_frac": flg / msg / 1e9 / FP8_PEAK_TFLOPS,
                                                     "output_GB": E4 * 4096 * 7168 * 2 / 1e9,
-                                                    "output_write_GB/s": E4 * 4096 * 7168 * 2 / msg / 1e6, "launches": len([g for g in (fast, rest) if g])},
+                                                    "output_write_GB/s": E4 * 4096 * 7168 * 2 / msg / 1e6, "launches": n_launches_w},
             "quant_colwise_t_65536x4096": {"ms": msq, "GB/s": byq / msq / 1e6, "hbm_frac": byq / msq / 1e6 / HBM_PEAK_GBS, "bytes": byq},
             "wgrad_gemm_rowscale_4096x7168xP1024": {"ms": msw, "tflops": 2.0 * 4096 * 7168 * Pw / msw / 1e9,
                                                     "mfma_frac": 2.0 * 4096 * 7168 * Pw / msw / 1e9 / FP8_PEAK_TFLOPS}}

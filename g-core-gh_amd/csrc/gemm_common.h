@@ -80,6 +80,9 @@ bool thin_ok(int64_t M, int64_t N, int64_t K);
 bool thin_rows_ok(int64_t M, int64_t N, int64_t K);
 int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                      void *C, int out_dtype, hipStream_t st);
+// per-row e8m0 scales, problems of one or two K blocks, no K loop (gemm_rowscale_small.hip); groups == nullptr: one problem
+int launch_rowscale_small(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int k_blocks,
+                          int64_t M, int64_t N, void *C, int out_dtype, hipStream_t st);
 int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                 void *C, int out_dtype, hipStream_t st);
 void skinny_plan(int64_t N, int64_t K, int &splits, int &per);

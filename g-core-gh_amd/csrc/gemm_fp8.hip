@@ -451,6 +451,10 @@ extern "C" int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *
     const int64_t grid = padded_grid(tiles_m, tiles_n);
     LP_REQUIRE(grid <= 0x7FFFFFFF, "lp_gemm_fp8_rowscale: problem too large");
     hipStream_t st = (hipStream_t)stream;
+    // one or two K blocks: the kernel without a K loop (the grouped entry uses it for such problems too: same bits)
+    if (scale_dtype == LP_E8M0 && (K == 128 || K == 256) && M % 128 == 0 && N % 128 == 0 && ((uintptr_t)As | (uintptr_t)Bs) % 2 == 0 &&
+        ((uintptr_t)Aq | (uintptr_t)Bq) % 16 == 0)
+        return gemm::launch_rowscale_small(Aq, As, Bq, Bs, nullptr, 1, (int)(K / 128), M, N, C, out_dtype, st);
     if (gemm::rowscale_asm_ok(As, Bs, scale_dtype, M, N, K)) return gemm::launch_rowscale_asm(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
     if (scale_dtype == LP_F32)
         hipLaunchKernelGGL((gemm_dense<LP_F32, true>), dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)Aq, As,
@@ -472,6 +476,10 @@ extern "C" int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, cons
     LP_REQUIRE(groups, "lp_gemm_fp8_rowscale_grouped: null pointer");
     LP_REQUIRE(M % 128 == 0, "lp_gemm_fp8_rowscale_grouped: M (%lld) must be a multiple of 128", (long long)M);
     hipStream_t st = (hipStream_t)stream;
+    // problems of exactly one or exactly two K blocks (short experts): no K loop, several workgroups per CU
+    if (scale_dtype == LP_E8M0 && (max_k_blocks == 1 || max_k_blocks == 2) && k_blocks_multiple == max_k_blocks && N % 128 == 0 &&
+        ((uintptr_t)As | (uintptr_t)Bs) % 2 == 0 && ((uintptr_t)Aq | (uintptr_t)Bq) % 16 == 0)
+        return gemm::launch_rowscale_small(Aq, As, Bq, Bs, groups, G, max_k_blocks, M, N, C, out_dtype, st);
     // every problem's K a multiple of 512 (promised by the caller: k_blocks_multiple), e8m0 scales: the hand-scheduled loop
     if (k_blocks_multiple % 4 == 0 && gemm::rowscale_asm_ok(As, Bs, scale_dtype, M, N, (int64_t)max_k_blocks * 128))
         return gemm::launch_rowscale_grouped_asm(Aq, As, Bq, Bs, groups, G, max_k_blocks, M, N, C, out_dtype, st);

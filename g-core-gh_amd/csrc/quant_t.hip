@@ -30,6 +30,14 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b)
     return r;
 }
 
+// 128-row blocks an expert of `rows` rows takes: rows rounded up to pad_rows, or with pad_rows = LP_PAD_MIXED to 128 up to
+// 256 rows and to 512 beyond (short experts then run the row-scaled GEMM's one- and two-block kernel, the others its loop)
+__device__ __forceinline__ int padded_blocks_of(int rows, int pad_rows)
+{
+    if (pad_rows == LP_PAD_MIXED) return rows <= 256 ? (rows + 127) >> 7 : ((rows + 511) >> 9) << 2;
+    return (rows + pad_rows - 1) / pad_rows * (pad_rows >> 7);
+}
+
 template <bool IS_BF16>
 __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ x, int64_t cols, const int32_t *__restrict__ m_offsets,
                                                        int E, int pad_rows, uint8_t *__restrict__ qT, void *__restrict__ sT, int scale_dtype,
@@ -47,7 +55,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     for (int e0 = 0; e0 < E; e0 += 64) {
         const int ee = e0 + lane;
         const int rb = ee < E ? m_offsets[ee] : 0, re = ee < E ? m_offsets[ee + 1] : 0;
-        const int cnt = (re - rb + pad_rows - 1) / pad_rows * (pad_rows >> 7);
+        const int cnt = padded_blocks_of(re - rb, pad_rows);
         int incl = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -70,7 +78,7 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
     if (hit_e < 0) return;
     pb = hit_pb;
     const int r_begin = hit_rb, r_end = hit_re;
-    const int nblk = (r_end - r_begin + pad_rows - 1) / pad_rows * (pad_rows >> 7);
+    const int nblk = padded_blocks_of(r_end - r_begin, pad_rows);
     const int lb = (int)(blk - pb);                      // block inside the expert
     const int64_t r0 = (int64_t)r_begin + (int64_t)lb * 128;
     const int valid = r_end - r0 < 128 ? (r_end - r0 > 0 ? (int)(r_end - r0) : 0) : 128;      // 0: a block of padding only
@@ -235,7 +243,8 @@ __global__ __launch_bounds__(256) void quant_colwise_t(const void *__restrict__ 
 extern "C" int lp_quant_fp8_colwise_t(const void *x, int x_dtype, int64_t rows, int64_t cols, const int32_t *m_offsets, int E,
                                       int64_t padded_blocks, int pad_rows, void *qT, void *sT, int scale_dtype, lp_stream_t stream)
 {
-    LP_REQUIRE(pad_rows == 128 || pad_rows == 256 || pad_rows == 512, "lp_quant_fp8_colwise_t: pad_rows must be 128, 256 or 512");
+    LP_REQUIRE(pad_rows == 128 || pad_rows == 256 || pad_rows == 512 || pad_rows == LP_PAD_MIXED,
+               "lp_quant_fp8_colwise_t: pad_rows must be 128, 256, 512 or LP_PAD_MIXED");
     LP_REQUIRE(x_dtype == LP_BF16 || x_dtype == LP_F32, "lp_quant_fp8_colwise_t: x_dtype must be LP_BF16 or LP_F32");
     LP_REQUIRE(scale_dtype == LP_F32 || scale_dtype == LP_E8M0, "lp_quant_fp8_colwise_t: scale_dtype must be LP_F32 or LP_E8M0");
     LP_REQUIRE(rows >= 0 && cols >= 0 && E >= 0 && padded_blocks >= 0, "lp_quant_fp8_colwise_t: bad shape");

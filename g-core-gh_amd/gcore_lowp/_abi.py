@@ -21,6 +21,7 @@ SCALE_POW2, SCALE_DIV, SCALE_MUL, SCALE_RCP, SCALE_RCP_POW2, SCALE_MUL_FLOOR = 0
 ZERO_NONE, ZERO_AMAX_TO_ONE, ZERO_SCALE_TO_ONE = 0, 1, 2
 # enum lp_fp4_zero
 FP4_POS_ZERO, FP4_NEG_ZERO = 0, 1
+PAD_MIXED = 0              # lp_quant_fp8_colwise_t: 128-row padding up to 256 rows, 512 beyond
 
 _i64, _p, _i32, _f32 = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 

@@ -134,30 +134,35 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs, rhs, out: torch.Tensor, m_ind
     grouped_gemm_fp8(xq, xs, wq, ws, offsets_from_m_indices(m_indices.to(xq.device), wq.shape[0]), out=out)
 
 
+def padded_blocks(rows: int, pad_rows: int) -> int:
+    """128-row blocks an expert of `rows` rows takes in the column-wise operands (lp_quant_fp8_colwise_t's rule)."""
+    rows = int(rows)
+    if pad_rows == A.PAD_MIXED:
+        return (rows + 127) // 128 if rows <= 256 else (rows + 511) // 512 * 4
+    return (rows + pad_rows - 1) // pad_rows * (pad_rows // 128)
+
+
 def choose_colwise_pad(m_splits) -> int:
-    """Rows every expert is padded to in the column-wise operands: 512 (the row-scaled GEMM then runs its
-    hand-scheduled kernel, which needs K in multiples of 512) unless that takes more than two and a half times the padded rows of 128.
-    A weight gradient is as much a write of E x N x K values as a GEMM, and on short K the hand-scheduled kernel is
-    ahead of the compiler-scheduled one by more than the extra rows cost: 256 experts of [4096, 7168] with 28 .. 7146
-    rows each, 1296 blocks at 512 against 643 at 128, 7.4 ms against 9.7 ms in one grouped launch: per padded block the hand-scheduled
-    kernel is about 2.6 times as fast."""
-    p128 = sum((int(m) + 127) // 128 for m in m_splits)
-    p512 = sum((int(m) + 511) // 512 * 4 for m in m_splits)
-    return 512 if p512 * 2 <= p128 * 5 else 128
+    """How the experts' rows are padded in the column-wise operands: A.PAD_MIXED -- experts of at most 256 rows to 128 or
+    256 (the row-scaled GEMM has a kernel without a K loop for problems of one and two K blocks: a weight gradient of a
+    short expert is a write of N x K values more than a GEMM), the others to multiples of 512 (its hand-scheduled loop
+    needs K in multiples of 512).  256 experts of [4096, 7168] with 0 .. 7163 rows: 6.7 ms with every expert padded to
+    512, 9.7 ms with every expert padded to 128 (the experts above 256 rows then run on the compiler-scheduled kernel)."""
+    return A.PAD_MIXED
 
 
 def quant_fp8_colwise_t(x: torch.Tensor, m_offsets: torch.Tensor, m_splits, pad_rows: int | None = None):
     """Column-wise quantisation of expert-grouped rows with transposed output (the operands of the weight-gradient
     GEMM): x [M, C] bf16/fp32 on the GPU -> (codes uint8 [C * P], e8m0 scales [C * P / 128], blocks per expert),
-    expert e's [C, P_e] / [C, P_e / 128] matrices stored one after the other, P_e = M_e rounded up to pad_rows.
-    pad_rows None: choose_colwise_pad(m_splits)."""
+    expert e's [C, P_e] / [C, P_e / 128] matrices stored one after the other, P_e = M_e rounded up to pad_rows (128, 256,
+    512, or A.PAD_MIXED: 128 up to 256 rows and 512 beyond).  pad_rows None: choose_colwise_pad(m_splits)."""
     assert x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32)
     rows, cols = x.shape
     assert all(int(m) >= 0 for m in m_splits) and sum(int(m) for m in m_splits) <= rows, "m_splits must fit the rows of x"
     m_offsets = _check_offsets(m_offsets, len(m_splits), x.device, "quant_fp8_colwise_t")
     if pad_rows is None:
         pad_rows = choose_colwise_pad(m_splits)
-    nblk = [(int(m) + pad_rows - 1) // pad_rows * (pad_rows // 128) for m in m_splits]
+    nblk = [padded_blocks(m, pad_rows) for m in m_splits]
     total = sum(nblk)
     q = torch.empty(cols * total * 128, dtype=torch.uint8, device=x.device)
     s = torch.empty(cols * total, dtype=ops.E8M0, device=x.device)
@@ -182,23 +187,24 @@ def gemm_fp8_rowscale(aq, a_s, bq, b_s, M, N, K, out: torch.Tensor) -> torch.Ten
 def gemm_fp8_rowscale_grouped(aq, a_s, bq, b_s, k_blocks, M, N, out: torch.Tensor) -> torch.Tensor:
     """out[e] [M, N] = the row-scaled product of problem e, whose operands ([M, K_e] / [N, K_e] codes and their e8m0
     scales, K_e = 128 * k_blocks[e]) lie one after the other in aq / a_s / bq / b_s.  The problems whose K is a multiple
-    of 512 go to the hand-scheduled loop in one launch, the others to the compiler-scheduled kernel in a second one;
-    problems with no K blocks are zero-filled.  (The reference issues one grouped GEMM call: fp8.py:325-341.)"""
+    of 512 go to the hand-scheduled loop in one launch, those of one and of two K blocks to the kernel without a K loop
+    (a launch each), the others to the compiler-scheduled kernel; problems with no K blocks are zero-filled.  (The
+    reference issues one grouped GEMM call: fp8.py:325-341.)"""
     E = len(k_blocks)
     assert out.is_contiguous() and tuple(out.shape) == (E, M, N) and out.dtype in (torch.bfloat16, torch.float32)
-    before, fast, rest, empty = 0, [], [], []
+    before, fast, one, two, rest, empty = 0, [], [], [], [], []
     for e, kb in enumerate(k_blocks):
         kb = int(kb)
         if kb == 0:
             empty.append(e)
         else:
-            (fast if kb % 4 == 0 else rest).append((e, kb, before, 0))
+            (fast if kb % 4 == 0 else one if kb == 1 else two if kb == 2 else rest).append((e, kb, before, 0))
         before += kb
     if empty:
         out[torch.tensor(empty, device=out.device)] = 0
     odt = A.BF16 if out.dtype == torch.bfloat16 else A.F32
     with torch.cuda.device(out.device):
-        for groups, multiple in ((fast, 4), (rest, 1)):
+        for groups, multiple in ((fast, 4), (one, 1), (two, 2), (rest, 1)):
             if not groups:
                 continue
             table = torch.tensor(groups, dtype=torch.int32).to(out.device)

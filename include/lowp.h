@@ -77,6 +77,11 @@ enum lp_fp4_zero {
     LP_FP4_NEG_ZERO = 1   /* -0.0: gpatch_v4/kernel/quantize/eager_quant_kernels.py:56-58 */
 };
 
+/* pad_rows of lp_quant_fp8_colwise_t: besides 128, 256 and 512 */
+enum lp_pad_rows {
+    LP_PAD_MIXED = 0      /* experts of at most 256 rows to multiples of 128, the others to multiples of 512 */
+};
+
 int lp_version(void);
 const char *lp_last_error(void);
 
@@ -298,7 +303,8 @@ int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const v
  * reads Aq + M * 128 * before (its [M, K_g] codes), As + M * before scales, Bq / Bs likewise with N, and writes
  * C + slot * M * N elements.  max_k_blocks bounds every entry's K blocks (argument checks); k_blocks_multiple is
  * the caller's promise that every entry's K block count is a multiple of it (4 selects the hand-scheduled loop
- * with e8m0 scales).  M must be a multiple of 128.  Entries with 0 blocks write nothing.  The table lives in
+ * with e8m0 scales; max_k_blocks = k_blocks_multiple = 1 or 2, i.e. every entry has exactly that many blocks, selects the
+ * kernel without a K loop for short experts, whose entries of any other size write nothing).  M must be a multiple of 128.  Entries with 0 blocks write nothing.  The table lives in
  * device memory, so the host cannot check it: an entry that breaks these promises (more K blocks than max_k_blocks,
  * a count that is not a multiple of 4 on the hand-scheduled kernel, a negative slot or offset) computes and writes
  * nothing -- its C_g keeps what it held.
@@ -311,7 +317,9 @@ int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, const void *Bq,
  * Column-wise quantiser with transposed output for expert-grouped rows.  x: device [rows, cols]
  * (LP_BF16 or LP_F32), rows of expert e = m_offsets[e] .. m_offsets[e+1]-1 (device int32 [E+1]),
  * cols % 128 == 0.  Per expert, P_e = ceil(M_e / pad_rows) * pad_rows (pad_rows 128, 256 or 512; with 512
- * lp_gemm_fp8_rowscale runs on its hand-scheduled kernel) and
+ * lp_gemm_fp8_rowscale runs on its hand-scheduled kernel), or with pad_rows = LP_PAD_MIXED: M_e rounded up to 128 for
+ * experts of at most 256 rows and to 512 for the others (lp_gemm_fp8_rowscale_grouped has a kernel for problems of one
+ * and two K blocks, which most experts of a routed batch are), and
  *   qT block e: [cols, P_e] e4m3fn at byte offset cols * (P_0 + .. + P_{e-1}), zero codes in the pad,
  *   sT block e: [cols, P_e / 128] scales at element offset cols * (P_0 + .. + P_{e-1}) / 128,
  * scale = 2^ceil(log2(amax / 448)) per (column, 128 rows of the expert), 1 for an all-zero block

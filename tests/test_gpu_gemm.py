@@ -379,9 +379,22 @@ def test_quant_colwise_t_matches_oracle(G):
             assert torch.equal(got_q[:, :nb * 128], wq.view(torch.uint8)) and not got_q[:, nb * 128:].any()
             assert torch.equal(got_s[:, :nb], ws.view(torch.uint8)) and bool((got_s[:, nb:] == 127).all())
         done += nblk5[e]
+    # mixed padding: experts of at most 256 rows to multiples of 128, the others to multiples of 512
+    import gcore_lowp._abi as _A
+    qm, sm_, nblkm = G.quant_fp8_colwise_t(x.to(torch.bfloat16).cuda(), offs.cuda(), m_splits, pad_rows=_A.PAD_MIXED)
+    assert nblkm == [4, 0, 1, 1, 1, 8]
+    done = 0
+    for e, (wq, ws) in enumerate(want):
+        pm, nb = nblkm[e] * 128, wq.shape[1] // 128
+        got_q = qm[384 * done * 128:384 * (done * 128 + pm)].view(384, pm).cpu()
+        got_s = sm_.view(torch.uint8)[384 * done:384 * (done + nblkm[e])].view(384, nblkm[e]).cpu()
+        if pm:
+            assert torch.equal(got_q[:, :nb * 128], wq.view(torch.uint8)) and not got_q[:, nb * 128:].any(), e
+            assert torch.equal(got_s[:, :nb], ws.view(torch.uint8)) and bool((got_s[:, nb:] == 127).all()), e
+        done += nblkm[e]
 
 
-@pytest.mark.parametrize("shape", [(128, 128, 128), (512, 384, 256), (300, 256, 1024), (4096, 7168, 384), (128, 128, 512),
+@pytest.mark.parametrize("shape", [(128, 128, 128), (512, 384, 256), (256, 384, 128), (4096, 7168, 256), (300, 256, 1024), (4096, 7168, 384), (128, 128, 512),
                                    (1000, 640, 2048), (4096, 7168, 1024), (77, 128, 1536)],
                          ids=lambda s: "M%d_N%d_K%d" % s)
 def test_gemm_rowscale(G, shape):
@@ -404,11 +417,12 @@ def test_gemm_rowscale(G, shape):
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
 def test_gemm_rowscale_grouped_equals_per_problem_launches(G, out_dtype):
-    """One grouped launch (two when some K are not multiples of 512) writes what one lp_gemm_fp8_rowscale launch per
-    problem writes, bit for bit: same kernels, same order of summation.  K blocks per problem cover multiples of 4,
-    other counts and an empty problem, which is zero-filled."""
+    """The grouped launches (one per kind of problem: K a multiple of 512, one K block, two K blocks, the rest) write what
+    one lp_gemm_fp8_rowscale launch per problem writes, bit for bit: same kernels, same order of summation.  K blocks per
+    problem cover multiples of 4, one and two blocks (the kernel without a K loop), other counts and an empty problem,
+    which is zero-filled."""
     M, N = 256, 384
-    k_blocks = [4, 1, 0, 8, 3, 12, 0, 5]
+    k_blocks = [4, 1, 0, 8, 3, 12, 0, 5, 2, 1, 2]
     say("gemm rowscale grouped", (M, N), k_blocks, out_dtype)
     total = sum(k_blocks)
     a = I.act_like(M, total * 128, 21)
@@ -446,6 +460,13 @@ def test_gemm_rowscale_grouped_equals_per_problem_launches(G, out_dtype):
     assert torch.equal(out2[0], out[0])                      # problem 0: 4 blocks from block 0
     assert bool((out2[1] == 7).all()) and bool((out2[2] == 7).all())           # 16 > max_k_blocks; 3 is not a multiple of 4
     assert torch.equal(out2[3], out[3])                      # problem 3: 8 blocks behind the 5 of problems 0 .. 2
+    # the same for the kernel of one-block problems: an entry of another size, or with a negative slot, writes nothing
+    table = torch.tensor([[0, 1, 4, 0], [1, 2, 25, 0], [-1, 1, 4, 0], [2, 1, 35, 0]], dtype=torch.int32, device="cuda")
+    out3 = torch.full((3, M, N), 7.0, dtype=out_dtype, device="cuda")
+    A.check(A.lib().lp_gemm_fp8_rowscale_grouped(aqf.data_ptr(), asf.data_ptr(), bqf.data_ptr(), bsf.data_ptr(), A.E8M0, table.data_ptr(), 4, 1, 1,
+                                                 M, N, out3.data_ptr(), A.BF16 if out_dtype == torch.bfloat16 else A.F32, A.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(out3[0], out[1]) and bool((out3[1] == 7).all()) and torch.equal(out3[2], out[9])
 
 
 @pytest.mark.parametrize("case", [([300, 0, 128, 1, 77, 513], 512, 512), ([2048, 16, 700], 1024, 2048), ([64, 64, 64, 64], 2048, 512),
