@@ -641,22 +641,20 @@ def main():
         # 256 problems [4096, 7168] x P_e, config 4's rows per expert padded as the wrapper pads them (experts of at most 256
         # rows to 128 or 256, the others to multiples of 512); operands are random codes (the time does not depend on the
         # values), 15 GB of bf16 out
-        from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad, padded_blocks
+        from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad, padded_blocks, rowscale_launches
         padw = choose_colwise_pad(m_splits.tolist())
         nblkw = [padded_blocks(int(m), padw) for m in m_splits.tolist()]
         pbw = sum(nblkw)
-        pre, fast, one, two, rest = 0, [], [], [], []
-        for e, nb in enumerate(nblkw):
-            if nb:
-                (fast if nb % 4 == 0 else one if nb == 1 else two if nb == 2 else rest).append((e, nb, pre, 0))
-            pre += nb
+        launches_w, _ = rowscale_launches(nblkw)
+        kinds_w = {"k_multiple_of_512": sum(1 for nb in nblkw if nb and nb % 4 == 0), "one_k_block": nblkw.count(1),
+                   "two_k_blocks": nblkw.count(2), "other": sum(1 for nb in nblkw if nb > 2 and nb % 4)}
         aT = torch.randint(0, 120, (4096 * pbw * 128,), dtype=torch.uint8, device=dev)
         bT = torch.randint(0, 120, (7168 * pbw * 128,), dtype=torch.uint8, device=dev)
         saT = torch.full((4096 * pbw,), 120, dtype=torch.uint8, device=dev)
         sbT = torch.full((7168 * pbw,), 121, dtype=torch.uint8, device=dev)
         dW = torch.empty(E4, 4096, 7168, dtype=torch.bfloat16, device=dev)
         tabs = [(torch.tensor(g, dtype=torch.int32, device=dev), len(g), max(x[1] for x in g), mult)
-                for g, mult in ((fast, 4), (one, 1), (two, 2), (rest, 1)) if g]
+                for g, mult in launches_w]
 
         def fng():
             for tab, n, mx, mult in tabs:
@@ -669,8 +667,7 @@ def main():
         extras["grouped_linear_backward"] = {
             "dgrad_grouped_256_experts_65536x4096_to_7168": dgrad_res,
             "wgrad_grouped_256_experts_4096x7168": {"ms": msg, "rows_padded_to": "128 up to 256 rows, 512 beyond" if padw == 0 else padw,
-                                                    "problems_by_kernel": {"k_multiple_of_512": len(fast), "one_k_block": len(one),
-                                                                           "two_k_blocks": len(two), "other": len(rest)},
+                                                    "problems_by_kernel": kinds_w,
                                                     "tflops_on_padded_rows": flg / msg / 1e9,
                                                     "mfma_frac": flg / msg / 1e9 / FP8_PEAK_TFLOPS,
                                                     "output_GB": E4 * 4096 * 7168 * 2 / 1e9,

@@ -184,6 +184,25 @@ def gemm_fp8_rowscale(aq, a_s, bq, b_s, M, N, K, out: torch.Tensor) -> torch.Ten
     return out
 
 
+def rowscale_launches(k_blocks):
+    """How the row-scaled problems of a grouped weight gradient are dealt to kernels: -> (launches, empty) with launches a
+    list of (table, multiple) -- table rows {problem, K blocks, K blocks of the problems before it, 0} as
+    lp_gemm_fp8_rowscale_grouped reads them, multiple = what every K block count of the table is a multiple of -- and
+    empty the problems without K blocks (their outputs are zeros).  Problems whose K is a multiple of 512 share the
+    hand-scheduled loop, those of one K block and those of two the kernel without a K loop, whatever is left the
+    compiler-scheduled kernel."""
+    before, fast, one, two, rest, empty = 0, [], [], [], [], []
+    for e, kb in enumerate(k_blocks):
+        kb = int(kb)
+        assert kb >= 0
+        if kb == 0:
+            empty.append(e)
+        else:
+            (fast if kb % 4 == 0 else one if kb == 1 else two if kb == 2 else rest).append((e, kb, before, 0))
+        before += kb
+    return [(g, m) for g, m in ((fast, 4), (one, 1), (two, 2), (rest, 1)) if g], empty
+
+
 def gemm_fp8_rowscale_grouped(aq, a_s, bq, b_s, k_blocks, M, N, out: torch.Tensor) -> torch.Tensor:
     """out[e] [M, N] = the row-scaled product of problem e, whose operands ([M, K_e] / [N, K_e] codes and their e8m0
     scales, K_e = 128 * k_blocks[e]) lie one after the other in aq / a_s / bq / b_s.  The problems whose K is a multiple
@@ -192,21 +211,12 @@ def gemm_fp8_rowscale_grouped(aq, a_s, bq, b_s, k_blocks, M, N, out: torch.Tenso
     reference issues one grouped GEMM call: fp8.py:325-341.)"""
     E = len(k_blocks)
     assert out.is_contiguous() and tuple(out.shape) == (E, M, N) and out.dtype in (torch.bfloat16, torch.float32)
-    before, fast, one, two, rest, empty = 0, [], [], [], [], []
-    for e, kb in enumerate(k_blocks):
-        kb = int(kb)
-        if kb == 0:
-            empty.append(e)
-        else:
-            (fast if kb % 4 == 0 else one if kb == 1 else two if kb == 2 else rest).append((e, kb, before, 0))
-        before += kb
+    launches, empty = rowscale_launches(k_blocks)
     if empty:
         out[torch.tensor(empty, device=out.device)] = 0
     odt = A.BF16 if out.dtype == torch.bfloat16 else A.F32
     with torch.cuda.device(out.device):
-        for groups, multiple in ((fast, 4), (one, 1), (two, 2), (rest, 1)):
-            if not groups:
-                continue
+        for groups, multiple in launches:
             table = torch.tensor(groups, dtype=torch.int32).to(out.device)
             A.check(A.lib().lp_gemm_fp8_rowscale_grouped(aq.data_ptr(), a_s.data_ptr(), bq.data_ptr(), b_s.data_ptr(), A.E8M0,
                                                          table.data_ptr(), len(groups), max(g[1] for g in groups), multiple,
@@ -228,11 +238,11 @@ class _GroupedGemmFp8(torch.autograd.Function):
                                   kernel turns the weight operand while it reads it out of LDS (a 128 x 128 block
                                   scaling is its own transpose, its table is read by column); no transposed copy;
       wgrad  dW_e = dY_e^T X_e    (layout NT over column-wise operands): dY and X quantised per (column, 128 rows of
-                                  the expert), transposed, all experts' row-scaled GEMMs in one launch (two when some experts'
-                                  padded row counts are not multiples of 512) straight into dW.
+                                  the expert), transposed, the experts' row-scaled GEMMs in one launch per kind of
+                                  expert (rowscale_launches: at most four) straight into dW.
     The reference pads every expert to a multiple of 16 rows for TE (fp8.py:29-58); here a ragged expert needs no
-    padding in the forward and dgrad (tiles are masked), and the column-wise operands are zero-padded to 128 rows,
-    which does not change any block's amax or sum."""
+    padding in the forward and dgrad (tiles are masked), and the column-wise operands are zero-padded to whole blocks
+    of 128 rows (choose_colwise_pad), which does not change any block's amax or sum."""
 
     @staticmethod
     def forward(ctx, inp, weight, wq, ws, m_splits, out_dtype):

@@ -161,3 +161,40 @@ def test_wide_tile_weight_copy_plan():
     assert sorted(moved) == list(range(36))
     rows_mid = sorted(r for g in mid for r in range(8 * g, 8 * g + 8))
     assert rows_mid == list(range(0, 64)) + list(range(144, 208))
+
+
+def test_weight_gradient_padding_and_launch_split():
+    """Host side of the grouped weight gradient: blocks of 128 rows per expert under each padding rule (the rule the
+    column-wise quantiser applies on the device), and the deal of the problems to kernels: every problem with K blocks in
+    exactly one table, each table's K block counts multiples of what the launch promises, the running offsets those of
+    the operands' layout, problems without rows listed apart."""
+    pytest.importorskip("torch")
+    from gcore_lowp import _abi as A
+    from gcore_lowp.grouped_gemm_fp8 import choose_colwise_pad, padded_blocks, rowscale_launches
+    rows = [0, 1, 128, 129, 256, 257, 512, 513, 1024, 1025, 7163]
+    assert [padded_blocks(r, 128) for r in rows] == [0, 1, 1, 2, 2, 3, 4, 5, 8, 9, 56]
+    assert [padded_blocks(r, 256) for r in rows] == [0, 2, 2, 2, 2, 4, 4, 6, 8, 10, 56]
+    assert [padded_blocks(r, 512) for r in rows] == [0, 4, 4, 4, 4, 4, 4, 8, 8, 12, 56]
+    assert [padded_blocks(r, A.PAD_MIXED) for r in rows] == [0, 1, 1, 2, 2, 4, 4, 8, 8, 12, 56]
+    assert choose_colwise_pad(rows) == A.PAD_MIXED
+    k_blocks = [4, 1, 0, 8, 3, 12, 0, 5, 2, 1, 2]
+    launches, empty = rowscale_launches(k_blocks)
+    assert empty == [2, 6]
+    seen = {}
+    for table, multiple in launches:
+        assert table and multiple in (1, 2, 4)
+        for e, kb, before, zero in table:
+            assert e not in seen and kb == k_blocks[e] and kb % multiple == 0 and zero == 0
+            assert before == sum(k_blocks[:e])
+            seen[e] = multiple
+        if multiple == 2:
+            assert all(kb == 2 for _, kb, _, _ in table)
+    assert sorted(seen) == [e for e, kb in enumerate(k_blocks) if kb]
+    assert {e for e, m in seen.items() if m == 4} == {0, 3, 5}
+    # the problems of one K block and the odd ones never share a table: the kernel without a K loop takes a table whose
+    # largest problem has one block
+    ones = [t for t, m in launches if m == 1 and all(kb == 1 for _, kb, _, _ in t)]
+    assert len(ones) == 1 and {e for e, _, _, _ in ones[0]} == {1, 9}
+    # a mixed padding never leaves a problem to the compiler-scheduled kernel
+    launches, _ = rowscale_launches([padded_blocks(r, A.PAD_MIXED) for r in range(0, 3000, 37)])
+    assert all(m in (2, 4) or all(kb == 1 for _, kb, _, _ in t) for t, m in launches)
