@@ -1,0 +1,99 @@
+"""Seeded sweeps around the dispatch boundaries of the GEMM entry points: row counts either side of the decode kernels'
+limits (8 / 9, 16 / 17, 64 / 65), weight-row counts either side of the tile-width choices (multiples of 224, 256 and
+288, a ragged last tile), K from one block to 7168, both scale types and both output types -- every shape against the
+fp32 dequantise-then-matmul reference to the path's tolerance.  The grouped sweeps draw the rows per expert from the
+values that change a tile class or a padding rule (0, 1, 128, 129, 256, 257, 512, 513) and from ranges."""
+import random
+
+import pytest
+import torch
+
+from oracle import torch_ref as T
+from tests import test_gpu_gemm as t
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gcore_lowp
+    return gcore_lowp
+
+
+ROWS = [1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 511, 512, 513, 777, 1024,
+        1500, 2048, 2560, 4096]
+WEIGHT_ROWS = [128, 256, 384, 512, 896, 1024, 2048, 2688, 3072, 3584, 4096, 4224, 4352, 5120, 6144, 6272, 7168, 8192, 8320, 9216,
+               12288, 16384, 18432, 18560, 20480]
+DEPTHS = [128, 256, 384, 512, 640, 896, 1024, 1536, 2048, 2560, 3584, 4096, 7168]
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_dense_gemm_shape_sweep(G, seed):
+    rng = random.Random(seed)
+    done = 0
+    while done < 36:
+        M, N, K = rng.choice(ROWS), rng.choice(WEIGHT_ROWS), rng.choice(DEPTHS)
+        if M * N * K > 2 ** 35:
+            continue
+        pow2, wide = rng.random() < 0.5, rng.random() < 0.3
+        t.say("dense sweep", seed, done, (M, N, K), "e8m0" if pow2 else "fp32", "f32 out" if wide else "bf16 out")
+        xq, xs, wq, ws = t.quantized_problem(M, N, K, seed=seed * 1000 + done, pow2=pow2)
+        out = G.gemm_fp8_block_scaling_impl(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(),
+                                            out_dtype=torch.float32 if wide else torch.bfloat16)
+        t.check(out, t.ref_gemm(xq, xs, wq, ws), f"dense sweep {(M, N, K)}")
+        done += 1
+
+
+def _splits(rng, E, hi):
+    return [rng.choice([0, 1, 127, 128, 129, 255, 256, 257, 511, 512, 513, rng.randint(1, hi), rng.randint(1, hi)]) for _ in range(E)]
+
+
+def test_grouped_gemm_shape_sweep(G):
+    rng = random.Random(21)
+    done = 0
+    while done < 24:
+        E = rng.choice([1, 2, 3, 5, 8, 16, 33])
+        N, K = rng.choice([128, 256, 384, 512, 768, 1024, 2048]), rng.choice([128, 256, 512, 640, 1024, 2048, 2560])
+        m_splits = _splits(rng, E, rng.choice([40, 400, 1200]))
+        M = sum(m_splits)
+        if M == 0 or M * N * K > 2 ** 32:
+            continue
+        t.say("grouped sweep", done, E, N, K, m_splits)
+        xq, xs, wq, ws = t._grouped_problem(E, N, K, m_splits, seed=2100 + done)
+        offs = torch.zeros(E + 1, dtype=torch.int32)
+        offs[1:] = torch.cumsum(torch.tensor(m_splits), 0)
+        out = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda())
+        t.check(out, T.grouped_gemm_fp8_ref(xq, xs, wq, ws, m_splits), f"grouped sweep {done}")
+        wide = G.grouped_gemm_fp8(xq.cuda(), xs.cuda(), wq.cuda(), ws.cuda(), offs.cuda(), out_dtype=torch.float32)
+        assert torch.equal(out, wide.to(torch.bfloat16))
+        done += 1
+
+
+def test_grouped_linear_backward_sweep(G):
+    """Forward, data gradient and weight gradient of every expert within 6 % (norm) of bf16 matmuls on that expert's rows:
+    an expert that reads another's rows, blocks or padding is off by the order of 100 %."""
+    rng = random.Random(31)
+    rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-30)).item()
+    for case in range(12):
+        E = rng.choice([1, 3, 4, 7, 12, 20])
+        h_in, h_out = rng.choice([(256, 512), (512, 256), (128, 384), (1024, 256)])
+        m_splits = _splits(rng, E, rng.choice([300, 900]))
+        if sum(m_splits) == 0:
+            continue
+        t.say("backward sweep", case, E, h_in, h_out, m_splits)
+        torch.manual_seed(3100 + case)
+        x = torch.randn(sum(m_splits), h_in, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+        w = torch.randn(E, h_out, h_in, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+        g = torch.randn(sum(m_splits), h_out, device="cuda", dtype=torch.bfloat16)
+        out = G.MyTeGroupedLinearFp8(E)(x, w, m_splits)
+        out.backward(g)
+        off = 0
+        for e, m in enumerate(m_splits):
+            xe, ge, we = x.detach()[off:off + m].float(), g[off:off + m].float(), w.detach()[e].float()
+            if m == 0:
+                assert not w.grad[e].any(), (case, e)
+            else:
+                assert rel(out[off:off + m], xe @ we.T) < 0.06, (case, e, m, "forward")
+                assert rel(x.grad[off:off + m], ge @ we) < 0.06, (case, e, m, "dgrad")
+                assert rel(w.grad[e], ge.T @ xe) < 0.06, (case, e, m, "wgrad")
+            off += m
