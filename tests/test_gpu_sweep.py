@@ -97,3 +97,59 @@ def test_grouped_linear_backward_sweep(G):
                 assert rel(x.grad[off:off + m], ge @ we) < 0.06, (case, e, m, "dgrad")
                 assert rel(w.grad[e], ge.T @ xe) < 0.06, (case, e, m, "wgrad")
             off += m
+
+
+def _bits_equal(a, b):
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    return a.dtype == b.dtype and a.shape == b.shape and torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+def test_quantise_dequantise_shape_sweep(G):
+    """The tile and the row-group quantisers and the dequantiser, bit for bit against the oracle, on shapes that end
+    inside a launch's unit of work: row counts that are not multiples of the 16 groups a pass takes, tile counts that
+    do not fill the XCDs evenly, one tile, one row."""
+    from tests import _inputs as I
+    rng = random.Random(41)
+    for case in range(30):
+        tiles = rng.random() < 0.5
+        if tiles:
+            rows, cols = 128 * rng.choice([1, 2, 3, 5, 7, 8, 9, 17, 31]), 128 * rng.choice([1, 2, 3, 5, 8, 11, 16, 29])
+            block = (128, 128)
+        else:
+            rows, cols = rng.choice([1, 2, 3, 15, 16, 17, 33, 63, 64, 65, 100, 257, 1000, 2049]), 128 * rng.choice([1, 2, 3, 7, 8, 25, 56])
+            block = (1, 128)
+        dt = torch.float32 if rng.random() < 0.3 else torch.bfloat16
+        x = (I.weight_like if tiles else I.act_like)(rows, cols, 4100 + case, dtype=dt)
+        t.say("quantise sweep", case, (rows, cols), block, dt)
+        rq, rs = T.quant_fp8_e4m3_scale_e8m0(x, block)
+        hq, hs = G.quant_fp8_e4m3_scale_e8m0(x.cuda(), block)
+        assert _bits_equal(hs, rs) and _bits_equal(hq, rq), ("pow2", case)
+        rq2, rs2 = T.quant_block_fp32_scale(x, block, amax_floor=1e-12)
+        hq2, hs2 = (G.quant_2d(x.cuda(), block) if tiles else G.quant_1d(x.cuda(), 128))
+        assert _bits_equal(hs2, rs2) and _bits_equal(hq2, rq2), ("divide", case)
+        want = T.dequant_fp4_e2m1_fp8_scale_e8m0_packed(rq, rs)
+        got = G.dequant_fp4_e2m1_fp8_scale_e8m0_packed(hq, hs)
+        assert _bits_equal(got, want), ("dequantise", case)
+
+
+def test_fp4_conversion_shape_sweep(G):
+    """FP4 -> bf16, FP4 -> FP8 re-based and FP4 -> FP8 fused (128 x 128, amax / 448) on expert shapes that end inside a
+    super tile of 128 x 256 and on single tiles, bit for bit against the oracle."""
+    from tests import _inputs as I
+    rng = random.Random(51)
+    for case in range(16):
+        rows, cols = 128 * rng.choice([1, 2, 3, 5, 8, 13]), 128 * rng.choice([1, 2, 3, 5, 7, 12])
+        lo = rng.choice([2, 60, 110, 117])
+        p, s = I.fp4_expert(rows, cols, 5100 + case, lo, lo + rng.choice([4, 10, 60]))
+        t.say("fp4 sweep", case, (rows, cols), lo)
+        w = T.cast_e2m1fn_to_bf16(p, s)
+        assert _bits_equal(G.cast_e2m1fn_to_bf16(p.cuda(), s.cuda()), w)
+        rq, rs = T.cast_e2m1fn_to_e4m3fn(p, s)
+        hq, hs = G.cast_e2m1fn_to_e4m3fn(p.cuda(), s.cuda())
+        assert _bits_equal(hs, rs) and _bits_equal(hq, rq)
+        rq, rs = T.quant_block_fp32_scale(w, (128, 128))
+        hq, hs = G.fp4_to_fp8_blockwise(p.cuda(), s.cuda())
+        assert _bits_equal(hs, rs)
+        a, b = hq.cpu().view(torch.uint8), rq.view(torch.uint8)
+        nan = (b & 0x7F) == 0x7F
+        assert torch.equal(a[~nan], b[~nan]) and bool(((a[nan] & 0x7F) == 0x7F).all())
