@@ -303,11 +303,13 @@ int lp_gemm_fp8_rowscale(const void *Aq, const void *As, const void *Bq, const v
  * reads Aq + M * 128 * before (its [M, K_g] codes), As + M * before scales, Bq / Bs likewise with N, and writes
  * C + slot * M * N elements.  max_k_blocks bounds every entry's K blocks (argument checks); k_blocks_multiple is
  * the caller's promise that every entry's K block count is a multiple of it (4 selects the hand-scheduled loop
- * with e8m0 scales; max_k_blocks = k_blocks_multiple = 1 or 2, i.e. every entry has exactly that many blocks, selects the
- * kernel without a K loop for short experts, whose entries of any other size write nothing).  M must be a multiple of 128.  Entries with 0 blocks write nothing.  The table lives in
- * device memory, so the host cannot check it: an entry that breaks these promises (more K blocks than max_k_blocks,
- * a count that is not a multiple of 4 on the hand-scheduled kernel, a negative slot or offset) computes and writes
- * nothing -- its C_g keeps what it held.
+ * with e8m0 scales; max_k_blocks = k_blocks_multiple = 1 or 2, i.e. every entry has exactly that many blocks,
+ * selects the kernel without a K loop for short experts, whose entries of any other size write nothing).  A caller
+ * with problems of several kinds makes one call per kind (gcore_lowp/grouped_gemm_fp8.py: rowscale_launches).
+ * M must be a multiple of 128.  Entries with 0 blocks write nothing.  The table lives in device memory, so the
+ * host cannot check it: an entry that breaks these promises (more K blocks than max_k_blocks, a count that is not
+ * a multiple of 4 on the hand-scheduled kernel, a negative slot or offset) computes and writes nothing -- its C_g
+ * keeps what it held.
  */
 int lp_gemm_fp8_rowscale_grouped(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype,
                                  const int32_t *groups, int G, int max_k_blocks, int k_blocks_multiple, int64_t M,
