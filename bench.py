@@ -261,6 +261,18 @@ def main():
                                                   "mfma_frac": 2.0 * n4 ** 3 / ms_nt / 1e9 / FP8_PEAK_TFLOPS,
                                                   "reference_ms_on_its_hardware": 0.575}
         del a_nt, b_nt, c_nt
+        # the same product on bf16 operands (the reference's benchmark quotes fp8 against bf16: 0.575 against 1.087 ms)
+        a_bf = torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).to(torch.bfloat16)
+        b_bf = [torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).to(torch.bfloat16) for _ in range(4)]
+        c_bf = torch.empty(n4, n4, dtype=torch.bfloat16, device=dev)
+        fns = [(lambda i=i: chk(L.lp_gemm_nt(a_bf.data_ptr(), b_bf[i].data_ptr(), A.BF16, n4, n4, n4, c_bf.data_ptr(), A.BF16, stream())))
+               for i in range(4)]
+        ms_bf, _ = time_launches(fns, 12, 4)
+        extras["gemm_impl_bf16_4096x4096x4096"] = {"ms": ms_bf, "tflops": 2.0 * n4 ** 3 / ms_bf / 1e9,
+                                                   "mfma_frac_of_bf16_peak": 2.0 * n4 ** 3 / ms_bf / 1e9 / 2500.0,
+                                                   "fp8_speed_up": ms_bf / ms_nt, "reference_ms_on_its_hardware": 1.087,
+                                                   "reference_fp8_speed_up": 1.89}
+        del a_bf, b_bf, c_bf
         torch.cuda.empty_cache()
         # what the matrix cores hold with the loop's arithmetic and nothing else: the fp8 16x16x128 instruction on registers
         # only, two waves per SIMD, with 0 / 4 / 8 fp32 FMAs after each (the fp32-scaled loops fold with four), on zeros and

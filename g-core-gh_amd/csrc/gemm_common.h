@@ -93,7 +93,7 @@ int launch_skinny(const void *Aq, const void *As, const void *Bq, const void *Bs
 int launch_rowscale_grouped_asm(const void *Aq, const void *As, const void *Bq, const void *Bs, const int32_t *groups, int G, int max_k_blocks, int64_t M,
                                 int64_t N, void *C, int out_dtype, hipStream_t st);
 int launch_nt_unit_scales(const void *A, const void *B, const void *ones, int64_t M, int64_t N, int64_t K, void *C, int out_dtype,
-                          hipStream_t st);
+                          hipStream_t st, bool bf16 = false);
 bool nt_unit_scales_ok(const void *ones, int64_t M, int64_t N, int64_t K);
 bool launch_wide(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                  void *C, int64_t ldc, int out_dtype, hipStream_t st, int *rc);

@@ -338,7 +338,8 @@ struct AsmTile {
 // check_asm_operands.py verifies both on the generated assembly at build time.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false, int WN = 2, bool NN = false>
+template <int TM, int TN, int KSUB, bool HWS = false, bool DUAL = false, int NST = 2, bool BROW = false, bool STAGED = false, int WN = 2, bool NN = false,
+          bool BF16 = false>
 __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restrict__ Aq, const float *__restrict__ As,
                                          const uint8_t *__restrict__ Bq, const float *__restrict__ Bs, int64_t m0, int64_t M,
                                          int64_t n0, int64_t N, int64_t K, void *__restrict__ C, int64_t ldc, int out_dtype)
@@ -564,12 +565,23 @@ __device__ __forceinline__ void tile_asm(uint8_t *smem, const uint8_t *__restric
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
     } else if constexpr (HWS && NBW == 8) {
         f32x16v acc0, acc1, acc2, acc3, acc4, acc5, acc6, acc7;
-        asm volatile(
+        if constexpr (BF16) {
+            // bf16 operands (K counts bytes: two per value): the same loop with two bf16 matrix instructions in place of
+            // each fp8 one; the scale operands are read and not used
+            asm volatile(
+#include "gemm_big_bf16_loop.inc"
+                : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+                  "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
+                : LP_ASM_INPUTS
+                : LP_ASM_CLOBBERS);
+        } else {
+            asm volatile(
 #include "gemm_big_hw_loop.inc"
-            : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
-              "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
-            : LP_ASM_INPUTS
-            : LP_ASM_CLOBBERS);
+                : "=&{v[128:143]}"(acc0), "=&{v[144:159]}"(acc1), "=&{v[160:175]}"(acc2), "=&{v[176:191]}"(acc3),
+                  "=&{v[192:207]}"(acc4), "=&{v[208:223]}"(acc5), "=&{v[224:239]}"(acc6), "=&{v[240:255]}"(acc7)
+                : LP_ASM_INPUTS
+                : LP_ASM_CLOBBERS);
+        }
         accs[0] = acc0; accs[1] = acc1; accs[2] = acc2; accs[3] = acc3;
         accs[4] = acc4; accs[5] = acc5; accs[6] = acc6; accs[7] = acc7;
     } else if constexpr (BROW) {
@@ -895,6 +907,17 @@ __global__ __launch_bounds__(TM * 2) void gemm_asm(const uint8_t *__restrict__ A
     int64_t tm, tn;
     if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
     tile_asm<TM, TN, KSUB, HWS, false, NST, false, true>(smem, Aq, As, Bq, Bs, tm * TM, M, tn * TN, N, K, C, ldc, out_dtype);
+}
+
+// The unscaled bf16 NT GEMM on the 256 x 256 loop (tile_asm with BF16): row_bytes = 2 K, every scale byte 2^0.
+__global__ __launch_bounds__(512) void gemm_asm_bf16(const uint8_t *__restrict__ A, const float *__restrict__ ones,
+                                                     const uint8_t *__restrict__ B, int64_t M, int64_t N, int64_t row_bytes,
+                                                     int64_t tiles_m, int64_t tiles_n, void *__restrict__ C, int64_t ldc, int out_dtype)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[AsmTile<256, 256, 1>::LDS_BYTES];
+    int64_t tm, tn;
+    if (!gemm::tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+    tile_asm<256, 256, 1, true, false, 2, false, true, 2, false, true>(smem, A, ones, B, ones, tm * 256, M, tn * 256, N, row_bytes, C, ldc, out_dtype);
 }
 
 // 256 x 288 tiles: N = 18432 is 64 of them, so a 2048-row problem is 512 tiles, exactly two rounds on 256 CUs.
@@ -1318,13 +1341,20 @@ int launch_big(const void *Aq, const void *As, const void *Bq, const void *Bs, i
 }
 
 // Unscaled fp8 NT GEMM on the hardware-scaled 256 x 256 loop with every scale byte 0x7F (2^0): `ones` holds at least
-// max(M, N / 128) * K / 128 such bytes.  out_dtype may be LP_E4M3 here (see tile_asm's last store loop).
+// max(M, N / 128) * K / 128 such bytes.  out_dtype may be LP_E4M3 here (see tile_asm's last store loop).  bf16: the operands
+// are bf16 and K is the number of bytes of an operand row (two per value).
 int launch_nt_unit_scales(const void *A, const void *B, const void *ones, int64_t M, int64_t N, int64_t K, void *C, int out_dtype,
-                          hipStream_t st)
+                          hipStream_t st, bool bf16)
 {
     const int64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + 255) / 256;
     const int64_t grid = gemm::padded_grid(tiles_m, tiles_n);
     if (grid > 0x7FFFFFFF) return fail(LP_ERR_UNSUPPORTED, "lp_gemm_nt: problem too large");
+    if (bf16) {
+        // K = bytes per operand row here
+        hipLaunchKernelGGL(gemm_asm_bf16, dim3((unsigned)grid), dim3(THREADS), 0, st, (const uint8_t *)A, (const float *)ones,
+                           (const uint8_t *)B, M, N, K, tiles_m, tiles_n, C, N, out_dtype);
+        return check_launch("lp_gemm_nt(asm, bf16)");
+    }
     if (quad_ok(M, N)) {
         hipLaunchKernelGGL(gemm_asm_quad, dim3((unsigned)grid), dim3(256), 0, st, (const uint8_t *)A, (const uint8_t *)ones,
                            (const uint8_t *)B, (const uint8_t *)ones, M, N, K, tiles_m, tiles_n, C, N, out_dtype);

@@ -244,6 +244,12 @@ extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M,
         const void *ones = unit_scale_array(st);
         if (ones && gemm::nt_unit_scales_ok(ones, M, N, K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, K, C, out_dtype, st);
     }
+    // bf16 operands on the same loop (two bf16 matrix instructions per fp8 one): K counted in bytes
+    if (!plain && in_dtype == LP_BF16 && (2 * K) % 512 == 0 && N % 16 == 0 && N >= 128 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
+        M * (2 * K / 128) <= kUnitScaleBytes && ((N + 127) / 128) * (2 * K / 128) <= kUnitScaleBytes) {
+        const void *ones = unit_scale_array(st);
+        if (ones && gemm::nt_unit_scales_ok(ones, M, N, 2 * K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, 2 * K, C, out_dtype, st, true);
+    }
     // 256 x 256 tiles once they fill the machine about twice, 128 x 128 otherwise
     // (bf16: from one round of tiles on -- 4096^3, 256 tiles: 127.5 us against 141.5 on 128 x 128 tiles)
     const bool big = M >= 192 && ((M + 255) / 256) * ((N + 255) / 256) >= (in_dtype == LP_BF16 ? 200 : 400);

@@ -35,13 +35,21 @@ import os
 MB = 4                                     # 16-row blocks per wave (64 activation rows)
 
 
-def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False, pingpong=False, nn=False):
+def configure(tm, tn, waves_m, waves_n, ksub, hw=False, nstage=2, brow=False, early=False, wide=False, idle=False, pingpong=False, nn=False,
+              bf16=False):
     """Tile tm x tn, waves_m x waves_n waves of 64 x (tn / waves_n); a stage holds ksub K blocks of 128; nstage
     stages in LDS (2: the copies of the next stage overlap this one; 4 with ksub 1: three K steps are in flight,
     for problems of about one tile per CU whose time is the chain of K steps)."""
     global A_BYTES, B_BYTES, SCL_LDS, SCL_HALF, NB, WAVES, KSUB, SPLIT, HW, NSTAGE, BROW, EARLY, WIDE, lines
     global ACC, P, AF, SC, SC2, SAN, WFB, RA0, RA1, RB0, RB1, SRD0, SRD, WS1, WS2, WSCUR, HALFSPLIT, ROT, WITH_IDLE, IDLE, PINGPONG, GRP, SPREAD, NN, BF, RBN
-    global WIDE_GROUP, WIDE_PART
+    global WIDE_GROUP, WIDE_PART, BF16
+    # bf16: the operands are bf16 values (a K step of 128 bytes is 64 of them) and every matrix instruction of the
+    # hardware-scaled loop becomes two v_mfma_f32_16x16x32_bf16 on the halves of the same fragment registers, accumulating
+    # in place: a lane's first four registers hold values 16 lq .. 16 lq + 7 of its row and the other four 16 lq + 8 .. + 15,
+    # for both operands alike, so the two instructions together sum over all 64 values.  Nothing else changes (copies,
+    # fragment reads, waits, hand-backs; the scale operands are simply not used): the unscaled bf16 NT GEMM.
+    BF16 = bf16
+    assert not bf16 or (hw and not brow and not nn and not wide)
     # idle: a second copy of the loop for waves none of whose activation rows exist (s93 = 1): an expert's short tile
     # of at most 64 rows leaves the second wave row of the 128 x 256 tile without work
     WITH_IDLE, IDLE = idle, False
@@ -431,6 +439,10 @@ def mfma(nb, mb, c=0):
         # scales applied by the matrix core: byte c of the weight-scale register (uniform) and of the lane's
         # activation-scale register; accumulation in place
         acc = vr(ACC + 16 * nb + 4 * mb, 4)
+        if BF16:
+            for half in (0, 4):
+                emit(f"v_mfma_f32_16x16x32_bf16 {acc}, {vr(WFB[par(c, nb)] + half, 4)}, {vr(AF + 8 * mb + half, 4)}, {acc}")
+            return
         wscale = f"v{WSN + nb}" if BROW else WSCUR
         emit(f"v_mfma_scale_f32_16x16x128_f8f6f4 {acc}, {vr(WFB[par(c, nb)], 8)}, {vr(AF + 8 * mb, 8)}, {acc}, {wscale}, v{SAN + mb} "
              f"op_sel:[{c & 1},{c & 1},0] op_sel_hi:[{c >> 1},{c >> 1},0]")
@@ -804,7 +816,8 @@ def main():
                       ("gemm_mid4_loop.inc", (128, 128, 2, 2, 1, False, 4)), ("gemm_mid4_hw_loop.inc", (128, 128, 2, 2, 1, True, 4)),
                       ("gemm_mid_hwrow_loop.inc", (128, 128, 2, 2, 1, True, 2, True, True)),
                       ("gemm_big_hw_nn_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True, PP, True)),
-                      ("gemm_flat_hw_nn_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True, False, True))):
+                      ("gemm_flat_hw_nn_loop.inc", (128, 256, 2, 4, 1, True, 3, False, True, False, True, False, True)),
+                      ("gemm_big_bf16_loop.inc", (256, 256, 4, 2, 1, True, 2, False, True, False, True, PP, False, True))):
         configure(*cfg)
         generate()
         write(here, name)
