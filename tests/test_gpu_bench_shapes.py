@@ -86,6 +86,32 @@ def test_prefill_gemm_at_benchmark_shape(G, pow2, shape):
     assert torch.equal(out, G.gemm_fp8_block_scaling_impl(xq, xs, wq, ws))
 
 
+@pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
+def test_gemm_at_the_reference_benchmarks_largest_shape(G, pow2):
+    """8096 x 129280 x 4096 (tests/test_gfused/test_my_gemm_fp8.py:280: a vocabulary projection; 8096 rows end inside a
+    256-row tile, 2.1 GB of bf16 output): checked slab by slab of 16160 weight rows against fp32 dequantise-then-matmul."""
+    M, N, K = 8096, 129280, 4096
+    x, w = _randn(M, K, 1.0, 21), _randn(N, K, 0.02, 22)
+    if pow2:
+        xq, xs = G.quant_fp8_e4m3_scale_e8m0(x, (1, 128))
+        wq, ws = G.quant_fp8_e4m3_scale_e8m0(w, (128, 128))
+    else:
+        xq, xs = G.quant_1d(x)
+        wq, ws = G.quant_2d(w)
+    del x, w
+    say("largest reference benchmark shape", (M, N, K), "e8m0" if pow2 else "f32")
+    out = G.gemm_fp8_block_scaling_impl(xq, xs, wq, ws)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N)
+    a = _dequant_a(xq, xs)
+    slab = 16160                                           # 126.25 x 128 rows: slab borders inside scale blocks and tiles
+    for n0 in range(0, N, slab):
+        n1 = min(n0 + slab, N)
+        lo, hi = n0 // 128 * 128, (n1 + 127) // 128 * 128
+        wd = _dequant_w(wq[lo:hi], ws[lo // 128:hi // 128])[n0 - lo:n1 - lo]
+        _bars(out[:, n0:n1], a @ wd.T, f"slab {n0}")
+        del wd
+
+
 @pytest.mark.parametrize("proj,N,K", [("gate_up", 4096, 7168), ("down", 7168, 2048)])
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_grouped_gemm_at_benchmark_shape(G, proj, N, K, pow2):
