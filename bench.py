@@ -281,6 +281,36 @@ def main():
                                                                 "reference_ms_on_its_hardware": ref_ms}
             del xb, wb, xq_, xs_, wq_, ws_, cq_
         torch.cuda.empty_cache()
+        # the GEMM alone on pre-quantised operands at the reference's three shapes (test_my_gemm_fp8.py:411-424: its tile
+        # compiler / TransformerEngine; tests/test_libs/test_deepgemm.py:230-249: DeepGEMM), workspace as the Python wrapper passes it
+        ref_only = {(4096, n4, n4): {"tile_compiler": 0.625, "transformer_engine": 0.571, "deepgemm": 0.536},
+                    (128, n4, n4): {"tile_compiler": 0.044, "transformer_engine": 0.217, "deepgemm": 0.023},
+                    (8096, 129280, 4096): {"tile_compiler": 38.334, "transformer_engine": 30.667, "deepgemm": 31.097}}
+        for (m_q, n_q, k_q), refs in ref_only.items():
+            n_sets_q = 1 if n_q > 100000 else 4
+            xb = randn(m_q, k_q)
+            xq_, xs_ = torch.empty(m_q, k_q, dtype=torch.uint8, device=dev), torch.empty(m_q, k_q // 128, dtype=torch.float32, device=dev)
+            quant_into(xb, 1, 128, xq_, xs_)
+            wqs_, wss_ = [], []
+            for _ in range(n_sets_q):
+                wb = randn(n_q, k_q, std=0.02)
+                wq_, ws_ = torch.empty(n_q, k_q, dtype=torch.uint8, device=dev), torch.empty(n_q // 128, k_q // 128, dtype=torch.float32, device=dev)
+                quant_into(wb, 128, 128, wq_, ws_)
+                wqs_.append(wq_)
+                wss_.append(ws_)
+                del wb
+            cq_ = torch.empty(m_q, n_q, dtype=torch.bfloat16, device=dev)
+            nws_q = L.lp_gemm_workspace_bytes(m_q, n_q, k_q)
+            wsp_q = torch.empty(max(nws_q, 16), dtype=torch.uint8, device=dev)
+            fns = [(lambda i=i: chk(L.lp_gemm_fp8_block(xq_.data_ptr(), xs_.data_ptr(), wqs_[i].data_ptr(), wss_[i].data_ptr(), A.F32, m_q, n_q, k_q,
+                                                        cq_.data_ptr(), A.BF16, wsp_q.data_ptr(), nws_q, stream()))) for i in range(n_sets_q)]
+            ms_o, _ = time_launches(fns, 4 if n_q > 100000 else 16, 4)
+            extras[f"gemm_only_{m_q}x{n_q}x{k_q}_fp32_scales"] = {"ms": ms_o, "tflops": 2.0 * m_q * n_q * k_q / ms_o / 1e9,
+                                                                  "mfma_frac": 2.0 * m_q * n_q * k_q / ms_o / 1e9 / FP8_PEAK_TFLOPS,
+                                                                  "weight_GB/s": n_q * k_q / ms_o / 1e6,
+                                                                  "reference_ms_on_its_hardware": refs}
+            del xb, xq_, xs_, wqs_, wss_, cq_, wsp_q
+        torch.cuda.empty_cache()
         # the same product on bf16 operands (the reference's benchmark quotes fp8 against bf16: 0.575 against 1.087 ms)
         a_bf = torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).to(torch.bfloat16)
         b_bf = [torch.randint(-3, 4, (n4, n4), generator=gen, device=dev).to(torch.bfloat16) for _ in range(4)]
