@@ -441,7 +441,8 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// 9 to 64 activation rows against many weight rows (more than one group of 16 per CU): a workgroup owns 8 R weight
+// 9 to 64 activation rows against many weight rows (more than one group of 16 per CU), and 65 to 128 rows against at
+// most 8192 weight rows (where 128 x 128 tiles would leave most CUs without one; R = 4, U = 4): a workgroup owns 8 R weight
 // rows (R = 4 .. 10: N / (8 R) workgroups, e.g. 256 of 72 rows for N = 18432) over the whole of K, so the 64 activation
 // rows a workgroup pulls through its CU's copy path are shared by 4 R / 8 times the weight bytes of the 16-row cut.
 // Same scheme as gemm_thin_ring2 otherwise: the 8 waves take runs of PER K blocks, wave-private rings fed by LDS-direct
@@ -451,7 +452,10 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 // of 16 for the matrix instruction; with odd R the last block's upper 8 rows are never loaded and its upper 8 columns
 // never stored (a column of the result depends on its own weight row only).  8 R is not a multiple of 128, so a
 // block of 16 rows can straddle two weight-scale blocks: every lane takes the scale of its own four columns.
-// U: activation units of 32 rows per K block (1 for at most 32 activation rows, 2 up to 64); two units are in flight.
+// U: activation units of 32 rows per K block (1 for at most 32 activation rows, 2 up to 64, 4 up to 128); two units are
+// in flight.  One MI355X, us per call with fp32 scales, split-K pair or tiles -> U = 4: 128 x 4096 x 4096 20.6 -> 16.1,
+// 96 x 7168 x 2048 13.5 -> 9.1, 128 x 8192 x 4096 23.3 -> 17.3, 128 x 4096 x 7168 22.0 -> 21.7; beyond 8192 weight rows
+// the tiles are ahead (128 x 12288 x 4096: 23.5 against 31.7).
 template <int PER, int R, int U>
 struct RowsPlan {
     int a_end[PER * U];          // requests issued up to and including activation unit u
@@ -689,8 +693,12 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     // from 9 activation rows: at 16 rows it is 8 % ahead of the 16-row ring kernel from N = 18432 (28.2 -> 25.9 us at K = 7168),
     // at 8 rows level with it (25.1 / 25.5), at 1 row behind (23.6 / 25.4)
     static const int64_t min_m = getenv("LP_GEMM_THIN_ROWS_MIN_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MIN_M")) : 9;
-    return !off && M >= min_m && M <= 64 && N % 16 == 0 && K % 128 == 0 && K / 128 <= kThinWaves * kThinRun && N / 16 > min_groups &&
-           N * K < 0xFFFFFFFFll;
+    // 65 .. 128 rows (four activation units per K block): where the tiled kernels would leave most CUs without a tile
+    static const int64_t max_m = getenv("LP_GEMM_THIN_ROWS_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MAX_M")) : 128;
+    static const int64_t wide_max_n = getenv("LP_GEMM_THIN_ROWS_WIDE_N") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_N")) : 8192;
+    if (off || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun || N * K >= 0xFFFFFFFFll) return false;
+    if (M > 64) return M <= max_m && M <= 128 && N / 16 >= 192 && N <= wide_max_n;
+    return M >= min_m && N / 16 > min_groups;
 }
 
 template <int SDT, int PER, int R>
@@ -698,6 +706,16 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
                         int out_dtype, hipStream_t st)
 {
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
+    if constexpr (R == 4) {
+        // 65 .. 128 activation rows: four units of 32 per K block (R = 4 only: with more weight rows the accumulators of eight
+        // row blocks no longer fit the registers, and a spill's reload would go through the request counter this kernel
+        // counts by hand)
+        if (M > 64) {
+            hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                               C, out_dtype);
+            return;
+        }
+    }
     if (M <= 32)
         hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                            C, out_dtype);
@@ -731,10 +749,11 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
     int best = 10;
     int64_t best_cost = INT64_MAX;
     for (int r : {4, 6, 8, 9, 10}) {
+        if (M > 64 && r > 4) break;
         const int64_t wgs = (N + 8 * r - 1) / (8 * r), cost = ((wgs + 255) / 256) * r;
         if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
     }
-    if (forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) best = forced;
+    if ((forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M <= 64 || forced == 4)) best = forced;
     if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
     else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
     return check_launch("lp_gemm_fp8_block(thin, many rows)");

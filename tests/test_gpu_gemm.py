@@ -79,6 +79,10 @@ DENSE_SHAPES = [
     (16, 4096, 7168), (1, 4096, 7168), (5, 3072, 2048), (16, 7168, 2560), (13, 18432, 128), (16, 3200, 6528),
     # 17 to 64 rows: the same cut with separate rings for weights and activations (2, 3, 4 row groups)
     (17, 4096, 7168), (32, 3072, 1024), (40, 3200, 6528), (48, 4096, 896), (50, 3072, 4096), (64, 18432, 2048),
+    # 65 to 128 rows against at most 8192 weight rows: the many-rows decode kernel with four activation units per K block
+    # (ragged last unit, one K block, a last workgroup past the end of N, 8192 / 8320 either side of its limit)
+    (65, 4096, 7168), (128, 4096, 4096), (100, 3072, 1024), (96, 7168, 2048), (127, 6144, 128), (128, 8192, 896), (128, 8320, 512),
+    (97, 3200, 640),
 ]
 
 
@@ -95,7 +99,8 @@ def test_gemm_dense(G, shape, pow2):
 
 @pytest.mark.parametrize("shape", [(2048, 2048, 7168), (300, 2048, 1024), (129, 1280, 2560), (1000, 4096, 512), (513, 18432, 1024),
                                    (2048, 18432, 512), (777, 4224, 1536), (257, 19200, 512), (64, 24576, 1536), (16, 4096, 2048),
-                                   (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024), (2048, 9472, 1024)],
+                                   (2048, 18432, 1024), (1900, 18432, 2048), (3000, 12800, 1024), (2048, 9472, 1024),
+                                   (128, 4096, 4096), (70, 7168, 2048)],
                          ids=lambda s: "M%d_N%d_K%d" % s)
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_gemm_bf16_output_is_the_rounded_fp32_output(G, shape, pow2):
