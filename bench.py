@@ -649,6 +649,20 @@ def main():
                                                     offs_d.data_ptr(), E4, Mt, N4, K4, c4.data_ptr(), A.BF16, stream()))
             ms48, _ = time_launches([fn8], 5, 2)
             res4[name + "_e8m0_scales"] = {"ms": ms48, "tflops": fl / ms48 / 1e9, "mfma_frac": fl / ms48 / 1e9 / FP8_PEAK_TFLOPS}
+            # a decode-sized batch through the same weights: 64 tokens x top-8 = 512 rows over the 256 experts (same Zipf
+            # recipe), where the launch is a stream of the weights of the experts that got a row
+            m_dec = zipf_m_splits(E4, 64, topk, seed=99)
+            offs_dec = torch.zeros(E4 + 1, dtype=torch.int32)
+            offs_dec[1:] = torch.cumsum(m_dec, 0)
+            offs_dec_d = offs_dec.to(dev)
+            rows_dec = int(offs_dec[-1])
+            fn_dec = lambda: chk(L.lp_gemm_fp8_grouped(x4q.data_ptr(), x4s.data_ptr(), w4q.data_ptr(), w4s.data_ptr(), A.F32,  # noqa: E731
+                                                       offs_dec_d.data_ptr(), E4, rows_dec, N4, K4, c4.data_ptr(), A.BF16, stream()))
+            ms_dec, _ = time_launches([fn_dec], 5, 2)
+            hit = int((m_dec > 0).sum())
+            res4[name + "_decode_sized_512_rows"] = {"ms": ms_dec, "experts_with_rows": hit, "max_rows": int(m_dec.max()),
+                                                     "weight_GB/s": hit * N4 * K4 / ms_dec / 1e6,
+                                                     "hbm_frac": hit * N4 * K4 / ms_dec / 1e6 / HBM_PEAK_GBS}
             if name == "gate_up":
                 # the data gradient of the same layer, dX_e = dY_e W_e on the stored [N4, K4] weights (layout NN,
                 # gpatch_v4/models/deepseek_v4/fp8.py:301-313): the kernel that turns the weight operand on its way out of

@@ -1571,13 +1571,17 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
 {
     static const char *force = getenv("LP_GEMM_GROUPED_MODE");          // tuning aid: 0 = 128 tiles, 1 = 256 + 128 in two launches, 2 = one mixed launch
     const int mode = force ? atoi(force) : -1;
-    // One launch with both tile heights when the experts are not all tiny (with fewer than 128 rows per expert on
-    // average hardly any 256-row tile exists and the 128 x 128 kernel, two workgroups per CU, streams weights as well)
+    // One launch with both tile heights when the experts are not all tiny and few (see many_flat_tiles below)
     // and K is not short: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden
     // behind a second workgroup (config 4, down projection, K = 2048: 1.76 ms against 1.87 for the 128 x 128 kernel
     // with fp32 scales in the same process, 1.46 against 1.57 with e8m0).
     // An expert has at most one small tile, and M_e / 256 big ones plus one when more than 128 rows are left over.
-    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && M_total >= (int64_t)E * 128 && K >= 2048)) {
+    // Experts of few rows all round (decode-sized batches: fewer than 128 rows per expert on average) take the mixed launch
+    // as well once their flat 128 x 256 tiles are at least two per CU: three LDS stages of streamed weights against the
+    // two of the 128 x 128 kernel (256 experts of 1 .. 127 rows, gate_up shape: 1.10 - 1.30 ms against 1.26 - 1.49; 128
+    // experts: 0.56 - 0.66 against 0.62 - 0.78; with 8 experts the 128 x 128 tiles are twice as many and win, 45 against 72 us).
+    const bool many_flat_tiles = (int64_t)E * (N / 256) >= 512;
+    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && (M_total >= (int64_t)E * 128 || many_flat_tiles) && K >= 2048)) {
         // an expert with r rows has r / 256 tiles plus one when rows are left over, big or small: M_total / 256 + E row
         // tiles at most over both classes, each class rounded up to whole groups of 8 x 32 workgroups
         int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;

@@ -161,6 +161,8 @@ GROUPED = [
     (5, 128, 384, [0, 0, 0, 0, 0]),
     (3, 384, 512, [300, 0, 77]),
     (300, 128, 128, [i % 7 for i in range(300)]),
+    # decode-sized batch: many experts of a few rows each and enough flat tiles for the launch with two tile heights
+    (64, 2048, 2048, [i % 5 for i in range(64)]),
     # many rows per expert: 256-row tiles on the hand-scheduled kernel (ragged experts, empty experts)
     (8, 512, 512, [700, 0, 300, 1, 255, 256, 257, 600]),
     (16, 768, 1024, [513, 0, 0, 90, 1024, 17, 256, 300, 2, 511, 128, 129, 64, 1, 700, 333]),
