@@ -1571,17 +1571,19 @@ int launch_big_grouped(const void *Aq, const void *As, const void *Bq, const voi
 {
     static const char *force = getenv("LP_GEMM_GROUPED_MODE");          // tuning aid: 0 = 128 tiles, 1 = 256 + 128 in two launches, 2 = one mixed launch
     const int mode = force ? atoi(force) : -1;
-    // One launch with both tile heights when the experts are not all tiny and few (see many_flat_tiles below)
-    // and K is not short: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden
-    // behind a second workgroup (config 4, down projection, K = 2048: 1.76 ms against 1.87 for the 128 x 128 kernel
-    // with fp32 scales in the same process, 1.46 against 1.57 with e8m0).
+    // One launch with both tile heights when the experts are not all tiny and few (see many_flat_tiles below), whatever
+    // the K: its workgroups own a CU alone, so what a tile spends before and after its K loop is not hidden behind a
+    // second workgroup, and still it is ahead of the 128 x 128 kernel down to K = 512 (config 4's rows per expert, N =
+    // 4096, fp32 scales: K = 512 0.29 against 0.36 ms, 1024 0.48 / 0.54, 1536 0.63 / 0.71, 2048 (down) 1.29 / 1.40).
     // An expert has at most one small tile, and M_e / 256 big ones plus one when more than 128 rows are left over.
-    // Experts of few rows all round (decode-sized batches: fewer than 128 rows per expert on average) take the mixed launch
-    // as well once their flat 128 x 256 tiles are at least two per CU: three LDS stages of streamed weights against the
-    // two of the 128 x 128 kernel (256 experts of 1 .. 127 rows, gate_up shape: 1.10 - 1.30 ms against 1.26 - 1.49; 128
-    // experts: 0.56 - 0.66 against 0.62 - 0.78; with 8 experts the 128 x 128 tiles are twice as many and win, 45 against 72 us).
-    const bool many_flat_tiles = (int64_t)E * (N / 256) >= 512;
-    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && (M_total >= (int64_t)E * 128 || many_flat_tiles) && K >= 2048)) {
+    // The launch needs work for every CU: at least one 256-row tile's worth per CU, counting an expert as half a tile on
+    // top of its rows (the host sees the row total, not the split).  Below that the 128 x 128 kernel, whose workgroups
+    // start at once and share CUs in pairs, is up to twice as fast (8 experts of 256 rows, N = 2048, K = 512: 8.3 against
+    // 17.8 us; 16 experts, N = 4096, K = 1536: 37.4 against 32.9 the other way).  Decode-sized batches pass the same test
+    // with their flat tiles alone: 256 experts of 1 .. 127 rows, gate_up shape, 1.10 - 1.30 ms against 1.26 - 1.49 on the
+    // 128 x 128 kernel (three LDS stages of streamed weights against two); 8 such experts stay there, 45 against 72 us.
+    const bool enough_tiles = (M_total / 256 + E / 2) * (N / 256) >= 256;
+    if (mode == 2 || (mode < 0 && E <= kMixedMaxExperts && enough_tiles)) {
         // an expert with r rows has r / 256 tiles plus one when rows are left over, big or small: M_total / 256 + E row
         // tiles at most over both classes, each class rounded up to whole groups of 8 x 32 workgroups
         int64_t grid = padded_grid(M_total / 256 + E, N / 256) + 2 * 8 * CHUNK;
