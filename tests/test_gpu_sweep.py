@@ -153,3 +153,34 @@ def test_fp4_conversion_shape_sweep(G):
         a, b = hq.cpu().view(torch.uint8), rq.view(torch.uint8)
         nan = (b & 0x7F) == 0x7F
         assert torch.equal(a[~nan], b[~nan]) and bool(((a[nan] & 0x7F) == 0x7F).all())
+
+
+def test_fp4_quantiser_and_qat_shape_sweep(G, corc):
+    """The FP4 quantiser (1 x 32 blocks), the fake-quantiser and the fused FP4 -> FP8 QAT conversion on shapes with row
+    counts and widths that end inside a launch's unit of work: the quantiser against both oracles through its own test's
+    comparison, the other two bit for bit against the eager restatement."""
+    from gcore_lowp import eager_quant_kernels as Q
+    from gcore_lowp.fused_quant_kernels import fp4_qat_then_to_fp8
+    from gcore_lowp.qat import fp4_simulate_qat
+    from tests import test_gpu_fp4_quant as q4
+    Q._corc = corc
+    rng = random.Random(61)
+    for case in range(14):
+        rows, cols = rng.choice([1, 2, 3, 31, 33, 100, 255, 257, 1000, 2049]), 32 * rng.choice([1, 2, 3, 5, 8, 33, 100, 224])
+        t.say("fp4 quantiser sweep", case, (rows, cols))
+        g = torch.Generator().manual_seed(6100 + case)
+        w = torch.randn(rows, cols, generator=g) * torch.logspace(-3, 2, cols // 32).repeat_interleave(32)
+        w[0, :32] = 0
+        q4.check(Q, w.to(torch.bfloat16 if case % 2 else torch.float32))
+        x = w.bfloat16()
+        assert torch.equal(fp4_simulate_qat(x.cuda()).cpu().view(torch.int16), T.fp4_simulate(x).view(torch.int16)), case
+    for case in range(6):
+        m, n = 128 * rng.choice([1, 2, 3, 5, 9]), 128 * rng.choice([1, 2, 3, 7, 12])
+        t.say("fp4 qat -> fp8 sweep", case, (m, n))
+        g = torch.Generator().manual_seed(6200 + case)
+        w = torch.randn(m, n, generator=g)
+        w[:, 32:64] *= 2.0 ** -4
+        w[:16, :32] = 0
+        q, s = fp4_qat_then_to_fp8(w.cuda())
+        wq, ws = T.fp4_qat_then_to_fp8(w)
+        assert _bits_equal(s, ws) and _bits_equal(q, wq), case
