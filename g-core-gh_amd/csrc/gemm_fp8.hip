@@ -559,10 +559,13 @@ extern "C" int lp_gemm_fp8_block(const void *Aq, const void *As, const void *Bq,
     static const bool force_small = getenv("LP_GEMM_FORCE_SMALL") != nullptr;
     static const char *force_tn = getenv("LP_GEMM_TN");
     const int esz = out_dtype == LP_BF16 ? 2 : 4, ssz = scale_dtype == LP_F32 ? 4 : 1;
-    // From 800 tiles of 128 x 128 on, and already above the 512 that fit the chip at once when the 256-row tiles
-    // still fit one round (576 tiles at K = 7168: 126 us as 128-tiles in two rounds, ~105 us as 144 big tiles).
+    // 256-row tiles from 800 tiles of 128 x 128 on, and already above the 512 that fit the chip at once when the 256-row
+    // tiles fill most of one round: more than 192 of them.  With fewer, the 128 x 128 tiles are ahead although they need a
+    // second, short round (K = 7168, fp32 / e8m0 scales, us as 256-row tiles -> 128 x 128: 2304 x 4096, 144 big tiles, 96.6
+    // -> 87.1 / 83.5 -> 74.7; 2560 x 4096, 160: 92.8 -> 87.4 / 80.2 -> 73.7; 2816 x 4096, 176: 91.1 -> 88.7 / 79.3 -> 75.0; the
+    // other way at 1664 x 7168, 196: 86.4 <- 88.9, and 2048 x 7168, 224: 92.2 <- 107.5).
     const int64_t small_tiles = tiles_m * tiles_n, big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-    if (!force_small && M >= 192 && (small_tiles >= 800 || (small_tiles > 512 && big_tiles <= 256))) {
+    if (!force_small && M >= 192 && (small_tiles >= 800 || (small_tiles > 512 && big_tiles > 192 && big_tiles <= 256))) {
         if (force_tn) return gemm::launch_big(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, atoi(force_tn), st);
         if (gemm::launch_wide(Aq, As, Bq, Bs, scale_dtype, M, N, K, C, N, out_dtype, st, &rc)) return rc;
         const int64_t bm = (M + 255) / 256, bn = (N + 255) / 256, tiles = bm * bn;
