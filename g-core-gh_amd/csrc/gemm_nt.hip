@@ -239,13 +239,18 @@ extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M,
     // compiler-scheduled kernel below.  LP_GEMM_NT_PLAIN=1 keeps that one.
     static const bool plain = getenv("LP_GEMM_NT_PLAIN") != nullptr;
     // (N >= 128: the loop indexes weight scales by 128-row block and needs at least one whole block)
-    if (!plain && in_dtype == LP_E4M3 && K % 512 == 0 && N % 16 == 0 && N >= 128 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
+    // From the point on where the 128 x 128 tiles of the kernel below no longer fit the chip at once (two workgroups per
+    // CU: 512): 2048 x 4096 x 4096, 512 tiles, 36.9 us there against 47.5 on the loop; 2304 x 4096 x 4096, 576 tiles, 58.8
+    // against 45.9 (bf16: 99.0 against 80.3).  LP_GEMM_NT_ASM_FROM = n (tuning aid): from n tiles of 128 x 128 instead.
+    static const int64_t asm_from = getenv("LP_GEMM_NT_ASM_FROM") ? atoi(getenv("LP_GEMM_NT_ASM_FROM")) : 513;
+    const int64_t small_tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    if (!plain && in_dtype == LP_E4M3 && K % 512 == 0 && N % 16 == 0 && N >= 128 && small_tiles >= asm_from &&
         M * (K / 128) <= kUnitScaleBytes && ((N + 127) / 128) * (K / 128) <= kUnitScaleBytes) {
         const void *ones = unit_scale_array(st);
         if (ones && gemm::nt_unit_scales_ok(ones, M, N, K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, K, C, out_dtype, st);
     }
     // bf16 operands on the same loop (two bf16 matrix instructions per fp8 one): K counted in bytes
-    if (!plain && in_dtype == LP_BF16 && (2 * K) % 512 == 0 && N % 16 == 0 && N >= 128 && ((M + 255) / 256) * ((N + 255) / 256) >= 200 &&
+    if (!plain && in_dtype == LP_BF16 && (2 * K) % 512 == 0 && N % 16 == 0 && N >= 128 && small_tiles >= asm_from &&
         M * (2 * K / 128) <= kUnitScaleBytes && ((N + 127) / 128) * (2 * K / 128) <= kUnitScaleBytes) {
         const void *ones = unit_scale_array(st);
         if (ones && gemm::nt_unit_scales_ok(ones, M, N, 2 * K)) return gemm::launch_nt_unit_scales(A, B, ones, M, N, 2 * K, C, out_dtype, st, true);
