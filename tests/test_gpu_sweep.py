@@ -184,3 +184,29 @@ def test_fp4_quantiser_and_qat_shape_sweep(G, corc):
         q, s = fp4_qat_then_to_fp8(w.cuda())
         wq, ws = T.fp4_qat_then_to_fp8(w)
         assert _bits_equal(s, ws) and _bits_equal(q, wq), case
+
+
+def test_unscaled_nt_gemm_shape_sweep(G):
+    """gemm_impl either side of the point where it changes kernels (512 tiles of 128 x 128), with ragged last row and
+    column tiles, K in and out of whole groups of 512 bytes, fp8 and bf16 operands, every output type."""
+    rng = random.Random(61)
+    shapes = [(2048, 4096), (2049, 4096), (2304, 4096), (2300, 4112), (1153, 8192), (4096, 2064), (640, 16400), (8200, 1040),
+              (3000, 3000 // 16 * 16), (5000, 1776), (16384, 528), (1024, 8208)]
+    for case, (M, N) in enumerate(shapes):
+        K = rng.choice([256, 512, 768, 1024, 1536])
+        kind = "fp8" if case % 2 == 0 else "bf16"
+        t.say("nt sweep", case, (M, N, K), kind)
+        g = torch.Generator().manual_seed(6100 + case)
+        dt = torch.float8_e4m3fn if kind == "fp8" else torch.bfloat16
+        a, b = torch.randn(M, K, generator=g).to(dt).cuda(), torch.randn(N, K, generator=g).to(dt).cuda()
+        ref = a.float() @ b.float().T
+        for out_dtype in ([torch.float8_e4m3fn, torch.bfloat16] if kind == "fp8" else [torch.bfloat16, torch.float32]):
+            c = G.gemm_impl(a, b, 128, 128, 64, dtype=dt, out_dtype=out_dtype)
+            assert c.dtype == out_dtype and tuple(c.shape) == (M, N)
+            if out_dtype == torch.float8_e4m3fn:
+                want = ref.clamp(-448, 448).to(out_dtype)
+                ci, wi = c.view(torch.uint8).int(), want.view(torch.uint8).int()
+                assert ((ci - wi).abs() <= 1).float().mean() > 0.9999, (M, N, K)
+            else:
+                err = ((c.float() - ref).abs().max() / ref.abs().max()).item()
+                assert err < (1e-2 if out_dtype == torch.bfloat16 else 1e-5), (M, N, K, err)
