@@ -442,8 +442,8 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 
 // ---------------------------------------------------------------------------------------------------------
 // 9 to 64 activation rows against many weight rows (more than one group of 16 per CU), and 65 to 128 rows against at
-// most 8192 weight rows (where 128 x 128 tiles would leave most CUs without one; R = 4, U = 4): a workgroup owns 8 R weight
-// rows (R = 4 .. 10: N / (8 R) workgroups, e.g. 256 of 72 rows for N = 18432) over the whole of K, so the 64 activation
+// most 8192 weight rows (where 128 x 128 tiles would leave most CUs without one; R = 2 or 4, U = 4): a workgroup owns 8 R weight
+// rows (R = 2 .. 10: N / (8 R) workgroups, e.g. 256 of 72 rows for N = 18432) over the whole of K, so the 64 activation
 // rows a workgroup pulls through its CU's copy path are shared by 4 R / 8 times the weight bytes of the 16-row cut.
 // Same scheme as gemm_thin_ring2 otherwise: the 8 waves take runs of PER K blocks, wave-private rings fed by LDS-direct
 // loads (a request = 8 rows x 128 bytes), hand-counted waits, no barrier inside the loop, partial sums added through LDS
@@ -670,17 +670,21 @@ namespace gemm {
 
 bool thin_ok(int64_t M, int64_t N, int64_t K)
 {
-    // one run of K blocks per wave, and enough workgroups to cover the chip (fewer are better served by the
-    // K-split kernels).  Above 16 rows a workgroup holds 128 KB of LDS and its activations (M / 16 times the
+    // one run of K blocks per wave.  Above 16 rows a workgroup holds 128 KB of LDS and its activations (M / 16 times the
     // bytes of its weights) come through the same request path, so beyond about two workgroups per CU the
     // K-split kernel, which shares the activations between 128 weight rows, is ahead (measured at N = 18432).
+    // No lower limit on the weight rows: with fewer workgroups than CUs this one launch is still ahead of the K-split
+    // pair's two (one MI355X, us per call, pair -> this kernel: 32 x 2048 x 1024 8.8 -> 4.0, 64 x 2048 x 7168 16.0 -> 11.8,
+    // 8 x 512 x 4096 10.1 -> 5.3, 16 x 128 x 7168 11.2 -> 5.3, 64 x 128 x 7168 12.4 -> 11.0).  LP_GEMM_THIN_FROM = n
+    // (tuning aid): only from n groups of 16 weight rows.
     if (M < 1 || M > 64 || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun) return false;
     const int64_t groups = N / 16;
-    return groups >= 192 && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
+    static const int64_t min_groups = getenv("LP_GEMM_THIN_FROM") ? atoi(getenv("LP_GEMM_THIN_FROM")) : 1;
+    return groups >= min_groups && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
 }
 
 // 9 .. 64 activation rows against more weight rows than one 16-row workgroup per CU: 8 R rows per workgroup, R from {4, 6, 8, 9,
-// 10} such that the rounds of 256 workgroups times R are fewest (18432 rows: R = 9, 256 workgroups).
+// 10} (65 .. 128 activation rows: from {2, 4}) such that the rounds of 256 workgroups times R are fewest (18432 rows: R = 9, 256 workgroups).
 // Groups of 16 weight rows from which the many-rows kernel takes over from the 16-row cut at more than 16 activation rows
 // (one MI355X, M = 64, K = 7168, us per call, 16-row cut or 128 x 128 tiles -> 8 R rows: N = 6144 23.1 -> 16.9, 8192 24.2 ->
 // 17.8, 12288 36.3 -> 22.0, 18432 38.4 -> 29.3, 36864 73.3 -> 60.7; N = 4096 is one 16-row workgroup per CU either way).
@@ -693,11 +697,16 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     // from 9 activation rows: at 16 rows it is 8 % ahead of the 16-row ring kernel from N = 18432 (28.2 -> 25.9 us at K = 7168),
     // at 8 rows level with it (25.1 / 25.5), at 1 row behind (23.6 / 25.4)
     static const int64_t min_m = getenv("LP_GEMM_THIN_ROWS_MIN_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MIN_M")) : 9;
-    // 65 .. 128 rows (four activation units per K block): where the tiled kernels would leave most CUs without a tile
+    // 65 .. 128 rows (four activation units per K block): where the tiled kernels would leave most CUs without a tile.  Up to
+    // 4096 weight rows a workgroup takes 16 of them (R = 2: 256 workgroups at N = 4096; 128 x 4096 x 4096 16.6 -> 15.3 us,
+    // 96 x 3072 x 2048 8.3 -> 7.5), and there is no lower limit on the weight rows either (tiles or K-split pair -> this
+    // kernel: 128 x 2048 x 7168 21.5 -> 14.2, 128 x 2048 x 2048 12.9 -> 7.9, 128 x 512 x 1024 8.9 -> 6.0, 128 x 128 x 7168
+    // 13.7 -> 13.1).  LP_GEMM_THIN_ROWS_WIDE_FROM = n (tuning aid): only from n groups of 16 weight rows.
     static const int64_t max_m = getenv("LP_GEMM_THIN_ROWS_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MAX_M")) : 128;
     static const int64_t wide_max_n = getenv("LP_GEMM_THIN_ROWS_WIDE_N") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_N")) : 8192;
     if (off || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun || N * K >= 0xFFFFFFFFll) return false;
-    if (M > 64) return M <= max_m && M <= 128 && N / 16 >= 192 && N <= wide_max_n;
+    static const int64_t wide_min_groups = getenv("LP_GEMM_THIN_ROWS_WIDE_FROM") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_FROM")) : 1;
+    if (M > 64) return M <= max_m && M <= 128 && N / 16 >= wide_min_groups && N <= wide_max_n;
     return M >= min_m && N / 16 > min_groups;
 }
 
@@ -706,6 +715,12 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
                         int out_dtype, hipStream_t st)
 {
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
+    if constexpr (R == 2) {
+        // 16 weight rows per workgroup exist for 65 .. 128 activation rows only (up to 64 the ring kernels serve that cut)
+        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype);
+        return;
+    }
     if constexpr (R == 4) {
         // 65 .. 128 activation rows: four units of 32 per K block (R = 4 only: with more weight rows the accumulators of eight
         // row blocks no longer fit the registers, and a spill's reload would go through the request counter this kernel
@@ -732,6 +747,7 @@ void launch_thin_rows_per(const void *Aq, const void *As, const void *Bq, const 
         if (per < PER) return launch_thin_rows_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, r, st);
     }
     switch (r) {
+    case 2: return launch_thin_rows_r<SDT, PER, 2>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
     case 4: return launch_thin_rows_r<SDT, PER, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
     case 6: return launch_thin_rows_r<SDT, PER, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
     case 8: return launch_thin_rows_r<SDT, PER, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
@@ -743,17 +759,17 @@ void launch_thin_rows_per(const void *Aq, const void *As, const void *Bq, const 
 int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                      void *C, int out_dtype, hipStream_t st)
 {
-    static const int forced = getenv("LP_GEMM_THIN_ROWS") ? atoi(getenv("LP_GEMM_THIN_ROWS")) : 0;     // tuning aid: 4, 6, 8, 9, 10
+    static const int forced = getenv("LP_GEMM_THIN_ROWS") ? atoi(getenv("LP_GEMM_THIN_ROWS")) : 0;     // tuning aid: 2, 4, 6, 8, 9, 10
     const int kblocks = (int)(K / 128);
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
     int best = 10;
     int64_t best_cost = INT64_MAX;
-    for (int r : {4, 6, 8, 9, 10}) {
-        if (M > 64 && r > 4) break;
+    for (int r : {2, 4, 6, 8, 9, 10}) {
+        if (M > 64 ? r > 4 : r < 4) continue;
         const int64_t wgs = (N + 8 * r - 1) / (8 * r), cost = ((wgs + 255) / 256) * r;
         if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
     }
-    if ((forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M <= 64 || forced == 4)) best = forced;
+    if ((forced == 2 || forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M > 64 ? forced <= 4 : forced >= 4)) best = forced;
     if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
     else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
     return check_launch("lp_gemm_fp8_block(thin, many rows)");

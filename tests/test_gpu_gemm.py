@@ -83,6 +83,10 @@ DENSE_SHAPES = [
     # (ragged last unit, one K block, a last workgroup past the end of N, 8192 / 8320 either side of its limit)
     (65, 4096, 7168), (128, 4096, 4096), (100, 3072, 1024), (96, 7168, 2048), (127, 6144, 128), (128, 8192, 896), (128, 8320, 512),
     (97, 3200, 640),
+    # the same cuts with fewer workgroups than CUs (few weight rows): 16 rows per workgroup up to 64 activation rows and, from 65,
+    # on the many-rows kernel (its narrowest cut); one group of 16 rows, a ragged last K-block run, one K block
+    (64, 512, 7168), (33, 128, 1024), (8, 256, 4096), (1, 128, 128), (20, 1024, 6528), (128, 512, 7168), (65, 2048, 2048), (100, 128, 1024),
+    (128, 1024, 128), (90, 384, 6528),
 ]
 
 
