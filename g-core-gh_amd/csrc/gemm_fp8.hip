@@ -298,12 +298,14 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ w
     }
 }
 
-// how many K ranges to use: aim at >= 2 workgroups per CU (256 CUs).  Only for few tiles: from about 96 tiles on
-// the hand-scheduled 128 x 128 kernel (which splits K inside the workgroup) is ahead of this kernel pair
-// (measured at K = 7168: 64 tiles 26 us against 37, 96 tiles 44 against 37, 192 tiles 63 against 37).
+// how many K ranges to use: aim at >= 2 workgroups per CU (256 CUs).  Only for at most 32 tiles: with more, the
+// hand-scheduled 128 x 128 kernel (which splits K inside the workgroup) is ahead of this kernel pair (one MI355X, us per
+// call, pair against that kernel, fp32 / e8m0 scales: 16 tiles, 512 x 512 x 7168, 21.4 / 22.1 against 27.6 / 24.2; 32 tiles,
+// 1024 x 512 x 7168, 22.4 / 23.5 against 29.5 / 26.0; 64 tiles, 2048 x 512 x 4096, 26.0 / 27.8 against 20.2 / 17.2; 72 tiles,
+// 384 x 3072 x 4096, 30.7 / 32.5 against 20.4 / 17.7; 80 tiles, 640 x 2048 x 7168, 42.5 / 46.1 against 30.6 / 26.4).
 int choose_splits(int64_t tiles, int64_t kblocks)
 {
-    if (tiles > 80 || kblocks < 32) return 1;                 // short K: the second launch costs more than the split gains
+    if (tiles > 32 || kblocks < 32) return 1;                 // short K: the second launch costs more than the split gains
     int64_t s = (512 + tiles - 1) / tiles;
     if (s > kblocks / 4) s = kblocks / 4;     // keep >= 4 K steps per range
     if (s > 16) s = 16;

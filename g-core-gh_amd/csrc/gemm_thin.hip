@@ -452,8 +452,8 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 // of 16 for the matrix instruction; with odd R the last block's upper 8 rows are never loaded and its upper 8 columns
 // never stored (a column of the result depends on its own weight row only).  8 R is not a multiple of 128, so a
 // block of 16 rows can straddle two weight-scale blocks: every lane takes the scale of its own four columns.
-// U: activation units of 32 rows per K block (1 for at most 32 activation rows, 2 up to 64, 4 up to 128); two units are
-// in flight.  One MI355X, us per call with fp32 scales, split-K pair or tiles -> U = 4: 128 x 4096 x 4096 20.6 -> 16.1,
+// U: activation units of 32 rows per K block (1 for at most 32 activation rows, 2 up to 64, 4 up to 128 and for slices of
+// 128 rows of more, one slice per blockIdx.y); two units are in flight.  One MI355X, us per call with fp32 scales, split-K pair or tiles -> U = 4: 128 x 4096 x 4096 20.6 -> 16.1,
 // 96 x 7168 x 2048 13.5 -> 9.1, 128 x 8192 x 4096 23.3 -> 17.3, 128 x 4096 x 7168 22.0 -> 21.7; beyond 8192 weight rows
 // the tiles are ahead (128 x 12288 x 4096: 23.5 against 31.7).
 template <int PER, int R, int U>
@@ -492,6 +492,14 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
     const int kblocks = (int)(K / 128);
     const int64_t n0 = (int64_t)blockIdx.x * (8 * R);
     const int kb0 = wave * PER;
+    if constexpr (U == 4) {
+        // more than 128 activation rows: blockIdx.y picks a slice of 128 (the last one may be shorter)
+        const int64_t r0 = (int64_t)blockIdx.y * 128;
+        Aq += r0 * K;
+        As = (const char *)As + r0 * kblocks * (SDT == LP_F32 ? 4 : 1);
+        C = (char *)C + r0 * N * (out_dtype == LP_BF16 ? 2 : 4);
+        M = M - (int)r0 < 128 ? M - (int)r0 : 128;
+    }
 
     uint32_t sv[SV];
 #pragma unroll
@@ -706,7 +714,17 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     static const int64_t wide_max_n = getenv("LP_GEMM_THIN_ROWS_WIDE_N") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_N")) : 8192;
     if (off || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun || N * K >= 0xFFFFFFFFll) return false;
     static const int64_t wide_min_groups = getenv("LP_GEMM_THIN_ROWS_WIDE_FROM") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_FROM")) : 1;
-    if (M > 64) return M <= max_m && M <= 128 && N / 16 >= wide_min_groups && N <= wide_max_n;
+    if (M > 128) {
+        // slices of 128 rows (blockIdx.y) in one launch, where all workgroups run at once and the tiled kernels would give most
+        // CUs no tile, so that a tile's chain of K steps is the whole time (0.7 us per step of 128): one MI355X, us per call,
+        // tiles or K-split pair -> slices: 512 x 2048 x 4096 26.8 -> 16.3, 256 x 4096 x 4096 23.9 -> 17.5, 1024 x 1024 x 7168
+        // 28.6 -> 22.7, 512 x 2048 x 1024 10.2 -> 7.5, 256 x 2048 x 2048 13.6 -> 8.5.  Not with two rounds of workgroups (512 x
+        // 3072 x 4096: 22.0 -> 29.6), not at K = 512 (level), not with few weight rows and a long K (256 x 256 x 7168: 14.4 ->
+        // 16.7).  LP_GEMM_THIN_ROWS_SLICES_MAX_M = n (tuning aid): up to n rows, 128 switches the slices off.
+        static const int64_t slices_max_m = getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M")) : 1024;
+        return M <= slices_max_m && max_m >= 128 && K >= 1024 && ((M + 127) / 128) * ((N + 31) / 32) <= 256 && (K <= 4096 || N >= 1024);
+    }
+    if (M > 64) return M <= max_m && N / 16 >= wide_min_groups && N <= wide_max_n;
     return M >= min_m && N / 16 > min_groups;
 }
 
@@ -716,8 +734,8 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
 {
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
     if constexpr (R == 2) {
-        // 16 weight rows per workgroup exist for 65 .. 128 activation rows only (up to 64 the ring kernels serve that cut)
-        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+        // 16 weight rows per workgroup exist from 65 activation rows on only (up to 64 the ring kernels serve that cut)
+        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                            C, out_dtype);
         return;
     }
@@ -726,7 +744,7 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
         // row blocks no longer fit the registers, and a spill's reload would go through the request counter this kernel
         // counts by hand)
         if (M > 64) {
-            hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+            hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                                C, out_dtype);
             return;
         }
@@ -764,9 +782,11 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
     int best = 10;
     int64_t best_cost = INT64_MAX;
+    const int64_t slices = M > 64 ? (M + 127) / 128 : 1;
     for (int r : {2, 4, 6, 8, 9, 10}) {
         if (M > 64 ? r > 4 : r < 4) continue;
-        const int64_t wgs = (N + 8 * r - 1) / (8 * r), cost = ((wgs + 255) / 256) * r;
+        // a workgroup's time goes with the bytes it pulls: 8 r weight rows and, from 65 rows on, 128 activation rows
+        const int64_t wgs = slices * ((N + 8 * r - 1) / (8 * r)), cost = ((wgs + 255) / 256) * (M > 64 ? 16 + r : r);
         if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
     }
     if ((forced == 2 || forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M > 64 ? forced <= 4 : forced >= 4)) best = forced;

@@ -87,6 +87,10 @@ DENSE_SHAPES = [
     # on the many-rows kernel (its narrowest cut); one group of 16 rows, a ragged last K-block run, one K block
     (64, 512, 7168), (33, 128, 1024), (8, 256, 4096), (1, 128, 128), (20, 1024, 6528), (128, 512, 7168), (65, 2048, 2048), (100, 128, 1024),
     (128, 1024, 128), (90, 384, 6528),
+    # more than 128 rows in slices of 128 on that kernel (all workgroups in one round): a ragged last slice, a last slice of
+    # one row, the largest row count, 16- and 32-row workgroups; and shapes just outside the rule (two rounds, K = 512)
+    (129, 256, 1024), (256, 2048, 4096), (300, 1024, 7168), (512, 2048, 4096), (384, 2560, 2048), (1000, 128, 1024), (1024, 1024, 1152),
+    (513, 2048, 1024), (256, 4096, 512),
 ]
 
 
