@@ -398,6 +398,9 @@ extern "C" int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
 
 static int64_t split_bytes(int64_t M, int64_t N, int64_t K)
 {
+    // shapes the single-launch decode kernels take never reach the K split
+    static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;
+    if (!no_thin && (gemm::thin_ok(M, N, K) || gemm::thin_rows_ok(M, N, K))) return 0;
     static const bool skinny = getenv("LP_GEMM_SKINNY") != nullptr && getenv("LP_GEMM_NO_SKINNY") == nullptr;
     if (M <= 64 && skinny) {
         int sp, per;
@@ -672,9 +675,10 @@ extern "C" int lp_gemm_fp8_block_static(const void *Aq, const void *As, const vo
     if (rc) return rc > 0 ? LP_OK : rc;
     // Only the K-split pair uses scratch (fp32 partial tiles, every one of them written before the reduction reads
     // it, so the buffer's previous contents never matter and nothing is cleared).
-    // (decode shapes are served by the single-launch kernels before the K split is considered: no scratch, never refused)
-    static const bool no_thin = getenv("LP_GEMM_NO_THIN") != nullptr;
-    const int64_t need = !no_thin && (gemm::thin_ok(M, N, K) || gemm::thin_rows_ok(M, N, K)) ? 0 : split_bytes(M, N, K);
+    // (decode shapes are served by the single-launch kernels before the K split is considered: no scratch, never refused).
+    // The pair is taken for at most 32 tiles of 128 x 128 in at most 16 K ranges: 32 MiB, the buffer's size, so the
+    // size test below guards against a dispatcher that changes rather than against any shape of today's.
+    const int64_t need = split_bytes(M, N, K);
     LP_REQUIRE(need <= kStaticScratchBytes,
                "lp_gemm_fp8_block_static: M=%lld N=%lld K=%lld needs %lld bytes of K-split scratch, the built-in buffer holds %lld; "
                "call lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes()",

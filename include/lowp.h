@@ -236,8 +236,9 @@ int64_t lp_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * lp_gemm_static_scratch_bytes() = 32 MiB that is part of the library's device image (every GPU the process uses
  * holds one copy until the process ends).  Same kernels, same summation order and therefore the same bits as
  * lp_gemm_fp8_block with a workspace of lp_gemm_workspace_bytes(M, N, K).  The call allocates and frees nothing.
- * Shapes whose K split needs more than the buffer are rejected with LP_ERR_INVALID and a message naming both
- * sizes (shapes that need no scratch always pass).  All calls on one GPU share that GPU's buffer: calls that can
+ * A shape whose K split needed more than the buffer would be rejected with LP_ERR_INVALID and a message naming both
+ * sizes; the K split is taken for at most 32 tiles of 128 x 128 in at most 16 K ranges, which is 32 MiB, so no shape
+ * is turned away today (shapes that need no scratch always pass).  All calls on one GPU share that GPU's buffer: calls that can
  * overlap on one GPU (different streams, or threads) race on it -- serialise them or use lp_gemm_fp8_block.
  * Nothing has to be cleared between calls: every partial tile is written before it is read.
  * No counterpart in the reference (its GEMM is a JIT kernel without scratch, gfused/mygemm_fp8.py:44-97).
