@@ -720,9 +720,15 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
         // tiles or K-split pair -> slices: 512 x 2048 x 4096 26.8 -> 16.3, 256 x 4096 x 4096 23.9 -> 17.5, 1024 x 1024 x 7168
         // 28.6 -> 22.7, 512 x 2048 x 1024 10.2 -> 7.5, 256 x 2048 x 2048 13.6 -> 8.5.  Not with two rounds of workgroups (512 x
         // 3072 x 4096: 22.0 -> 29.6), not at K = 512 (level), not with few weight rows and a long K (256 x 256 x 7168: 14.4 ->
-        // 16.7).  LP_GEMM_THIN_ROWS_SLICES_MAX_M = n (tuning aid): up to n rows, 128 switches the slices off.
-        static const int64_t slices_max_m = getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M")) : 1024;
-        return M <= slices_max_m && max_m >= 128 && K >= 1024 && ((M + 127) / 128) * ((N + 31) / 32) <= 256 && (K <= 4096 || N >= 1024);
+        // 16.7).  The longer K, the fewer rows: up to 8192 at K <= 2048 (2048 x 512 x 2048: 13.3 -> 10.7, 4096 x 128 x 1024: 10.7 ->
+        // 7.5), up to 2048 at K <= 4096 and from 256 weight rows (1280 x 512 x 4096: 20.1 -> 17.5, but 4096 x 256 x 4096: 20.6 ->
+        // 28.2 and 1280 x 128 x 4096: 13.9 -> 15.7), up to 1024 beyond.
+        // LP_GEMM_THIN_ROWS_SLICES_MAX_M = n (tuning aid): up to n rows at most, 128 switches the slices off.
+        static const int64_t slices_max_m = getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_SLICES_MAX_M")) : 8192;
+        const int64_t rows_at_k = K <= 2048 ? 8192 : K <= 4096 ? 2048 : 1024;
+        const int64_t weight_rows_at_k = K <= 2048 ? 128 : K <= 4096 ? 256 : 1024;
+        return M <= slices_max_m && M <= rows_at_k && N >= weight_rows_at_k && max_m >= 128 && K >= 1024 &&
+               ((M + 127) / 128) * ((N + 31) / 32) <= 256;
     }
     if (M > 64) return M <= max_m && N / 16 >= wide_min_groups && N <= wide_max_n;
     return M >= min_m && N / 16 > min_groups;

@@ -90,7 +90,7 @@ DENSE_SHAPES = [
     # more than 128 rows in slices of 128 on that kernel (all workgroups in one round): a ragged last slice, a last slice of
     # one row, the largest row count, 16- and 32-row workgroups; and shapes just outside the rule (two rounds, K = 512)
     (129, 256, 1024), (256, 2048, 4096), (300, 1024, 7168), (512, 2048, 4096), (384, 2560, 2048), (1000, 128, 1024), (1024, 1024, 1152),
-    (513, 2048, 1024), (256, 4096, 512),
+    (513, 2048, 1024), (256, 4096, 512), (8192, 128, 1024), (5000, 128, 2048), (2048, 512, 4096), (1300, 768, 3072), (2049, 256, 4096),
 ]
 
 
