@@ -280,15 +280,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     store_tile(acc, ta.m0, M, ta.n0, N, ws + (int64_t)split * M * N, LP_F32);
 }
 
+// The ranges are added in their order.  All loads are issued before the first addition (a range past the last is read
+// from the last and not added): a thread's time is one trip to memory instead of one per range, which is what a
+// reduction of a few MB costs.
 __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ ws, int splits, int64_t mn,
                                                      void *__restrict__ C, int out_dtype)
 {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= mn) return;
     f32x4 s = *(const f32x4 *)(ws + i);
-    for (int k = 1; k < splits; ++k) {
-        f32x4 v = *(const f32x4 *)(ws + (int64_t)k * mn + i);
-        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    for (int k0 = 1; k0 < splits; k0 += 8) {
+        f32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = k0 + j < splits ? k0 + j : splits - 1;
+            v[j] = *(const f32x4 *)(ws + (int64_t)k * mn + i);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool on = k0 + j < splits;
+            s.x += on ? v[j].x : 0.0f; s.y += on ? v[j].y : 0.0f; s.z += on ? v[j].z : 0.0f; s.w += on ? v[j].w : 0.0f;
+        }
     }
     if (out_dtype == LP_BF16) {
         u32x2 o = {pack_bf16(s.x, s.y), pack_bf16(s.z, s.w)};
@@ -302,7 +314,12 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float *__restrict__ w
 // hand-scheduled 128 x 128 kernel (which splits K inside the workgroup) is ahead of this kernel pair (one MI355X, us per
 // call, pair against that kernel, fp32 / e8m0 scales: 16 tiles, 512 x 512 x 7168, 21.4 / 22.1 against 27.6 / 24.2; 32 tiles,
 // 1024 x 512 x 7168, 22.4 / 23.5 against 29.5 / 26.0; 64 tiles, 2048 x 512 x 4096, 26.0 / 27.8 against 20.2 / 17.2; 72 tiles,
-// 384 x 3072 x 4096, 30.7 / 32.5 against 20.4 / 17.7; 80 tiles, 640 x 2048 x 7168, 42.5 / 46.1 against 30.6 / 26.4).
+// 384 x 3072 x 4096, 30.7 / 32.5 against 20.4 / 17.7; 80 tiles, 640 x 2048 x 7168, 42.5 / 46.1 against 30.6 / 26.4; the pair's
+// figures are from before its reduction issued all its loads at once, which took 1 - 2 us off: 4 tiles 14.4 -> 12.5).
+// K ranges on the hand-scheduled 128 x 128 loop instead of this compiler-scheduled kernel were built and measured: level
+// (4 tiles 12.2 against 12.5, 16 tiles 18.9 against 20.2, 32 tiles 22.7 against 22.4, 2000 x 128 x 7168 19.0 against 18.5) and,
+// with more tiles, behind the single launch like this pair -- one workgroup per CU already keeps half of the CU's matrix
+// rate, so two ranges that land on one CU take as long as the unsplit tile.
 int choose_splits(int64_t tiles, int64_t kblocks)
 {
     if (tiles > 32 || kblocks < 32) return 1;                 // short K: the second launch costs more than the split gains
