@@ -234,7 +234,21 @@ extern "C" int lp_gemm_nt(const void *A, const void *B, int in_dtype, int64_t M,
     LP_REQUIRE((uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 && (uintptr_t)C % 16 == 0,
                "lp_gemm_nt: operands must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    // fp8 operands, K in whole groups of 512, enough 256 x 256 tiles to fill the chip: the block-scaled GEMM's hand-scheduled
+    // fp8 operands with bf16 or fp32 results, K and N in whole scale blocks: the block-scaled GEMM itself with every scale
+    // 2^0 (e8m0 scales are applied inside the matrix instruction at no cost), i.e. its whole choice of kernels by shape --
+    // the decode kernels, the hand-scheduled 128 x 128 and 256-row loops -- instead of the compiler-scheduled kernel below.
+    // Same bits on every shape compared; one MI355X, us per call, that kernel -> this route: 64 x 4096 x 7168 43.1 -> 12.4,
+    // 128 x 4096 x 2048 17.7 -> 9.5, 512 x 1024 x 4096 28.8 -> 15.4, 2048 x 4096 x 1024 15.8 -> 11.7, 1024 x 4096 x 4096 30.5 ->
+    // 18.8, 2048 x 4096 x 4096 36.3 -> 30.3, 2048 x 18432 x 1024 49.9 -> 42.4; level from 4096^3 on, where both end in the
+    // same loop.  LP_GEMM_NT_PLAIN=1 or LP_GEMM_NT_BLOCK=0 (tuning aids) keep it off.
+    static const bool plain_early = getenv("LP_GEMM_NT_PLAIN") != nullptr;
+    static const bool via_block = !(getenv("LP_GEMM_NT_BLOCK") && atoi(getenv("LP_GEMM_NT_BLOCK")) == 0);
+    if (!plain_early && via_block && in_dtype == LP_E4M3 && out_dtype != LP_E4M3 && K % 128 == 0 && N % 128 == 0 &&
+        M * (K / 128) <= kUnitScaleBytes && (N / 128) * (K / 128) <= kUnitScaleBytes) {
+        const void *ones = unit_scale_array(st);
+        if (ones) return lp_gemm_fp8_block(A, ones, B, ones, LP_E8M0, M, N, K, C, out_dtype, nullptr, 0, stream);
+    }
+    // e4m3 results (and whatever the route above leaves): K in whole groups of 512, enough tiles: the block-scaled GEMM's hand-scheduled
     // loop with every scale 2^0 (e8m0 scales are applied inside the matrix instruction at no cost), instead of the
     // compiler-scheduled kernel below.  LP_GEMM_NT_PLAIN=1 keeps that one.
     static const bool plain = getenv("LP_GEMM_NT_PLAIN") != nullptr;
