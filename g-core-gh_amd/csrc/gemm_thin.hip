@@ -638,19 +638,22 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
     };
     unrolled(step, std::make_integer_sequence<int, UNITS>{});
 
-    // partial sums through the (drained) rings, two row groups at a time: pair (g, nb) of the pass is added up by wave
-    // pair % 8 over the waves in their order
-    f32x4v *red = (f32x4v *)ring;                        // [wave][2 NBK][lane], 2 NBK KB per wave <= R + 8 KB
-    static_assert(2 * NBK * 1024 <= WAVE_LDS, "a wave's partial sums of a pass fit its own ring");
+    // partial sums through the (drained) rings, as many row groups at a time as fit a wave's own ring (all of them in one pass
+    // where they do: every pass costs two barriers at which the waves wait for the slowest): pair (g, nb) of the pass is
+    // added up by wave pair % 8 over the waves in their order
+    f32x4v *red = (f32x4v *)ring;                        // [wave][GP NBK][lane], GP NBK KB per wave <= its ring
+    constexpr int FIT = WAVE_LDS / 1024 / NBK;           // row groups whose partial sums fit
+    constexpr int GP = FIT >= MB ? MB : (FIT >= 4 && MB % 4 == 0 ? 4 : 2);
+    static_assert(GP * NBK * 1024 <= WAVE_LDS && MB % GP == 0, "a wave's partial sums of a pass fit its own ring");
 #pragma unroll
-    for (int pass = 0; pass < U; ++pass) {
+    for (int pass = 0; pass < MB / GP; ++pass) {
         __syncthreads();                                 // every wave is done with its ring (or with the previous pass)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int h = 0; h < GP; ++h)
 #pragma unroll
-            for (int nb = 0; nb < NBK; ++nb) red[(wave * (WAVE_LDS / 1024) + h * NBK + nb) * 64 + lane] = acc[2 * pass + h][nb];
+            for (int nb = 0; nb < NBK; ++nb) red[(wave * (WAVE_LDS / 1024) + h * NBK + nb) * 64 + lane] = acc[GP * pass + h][nb];
         __syncthreads();
-        for (int pair = wave; pair < 2 * NBK; pair += kThinWaves) {
+        for (int pair = wave; pair < GP * NBK; pair += kThinWaves) {
             const int h = pair / NBK, nb = pair % NBK;
             f32x4v sum = red[(h * NBK + nb) * 64 + lane];
 #pragma unroll
@@ -658,7 +661,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
                 const f32x4v x = red[(w * (WAVE_LDS / 1024) + h * NBK + nb) * 64 + lane];
                 sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
             }
-            const int row = 16 * (2 * pass + h) + l16, col = 16 * nb + 4 * lq;
+            const int row = 16 * (GP * pass + h) + l16, col = 16 * nb + 4 * lq;
             const int64_t n = n0 + col;
             if (row >= M || col >= 8 * R || n >= N) continue;
             if (out_dtype == LP_BF16) {
