@@ -131,6 +131,34 @@ __device__ __forceinline__ void wait_requests()          // at most N of the wav
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// K longer than the 8 x kThinRun blocks a workgroup's waves take in one run: the workgroup walks K in `rounds` rounds of
+// round_blocks K blocks -- scale table, requests and the unrolled run of every wave once per round, the accumulators kept
+// across them -- so nothing is added up outside the kernel and no scratch is needed; a round's start-up (the rings drain
+// and fill again) is paid rounds - 1 times more.  The operands and scale tables move on by a round's blocks, their row
+// pitches stay those of the whole K.  Sets kblocks to the K blocks of this round.
+#define LP_THIN_ROUND(SDT)                                                                                         \
+    const int rb = LONGK && rounds > 1 ? round_blocks : row_blocks;                                                \
+    if (LONGK && rd) {                                                                                                      \
+        Aq += (int64_t)rb * 128;                                                                                   \
+        Bq += (int64_t)rb * 128;                                                                                   \
+        As = (const char *)As + (int64_t)rb * ((SDT) == LP_F32 ? 4 : 1);                                           \
+        Bs = (const char *)Bs + (int64_t)rb * ((SDT) == LP_F32 ? 4 : 1);                                           \
+        __syncthreads(); /* every wave has its scales of the last round in registers before the table is rewritten */ \
+    }                                                                                                              \
+    const int kblocks = !LONGK ? row_blocks : (row_blocks - rd * rb < rb ? row_blocks - rd * rb : rb);
+
+// entry i of a workgroup's activation-scale table [M, kblocks] (its K blocks of every row, rows row_blocks entries apart
+// in memory)
+template <bool LONGK>
+__device__ __forceinline__ int table_index(int i, int M, int kblocks, int row_blocks)
+{
+    const int last = M * kblocks - 1;
+    const int c = i < last ? i : last;
+    if (!LONGK || kblocks == row_blocks) return c;       // (one pass over the whole K: the table is the one in memory)
+    const int row = c / kblocks;
+    return row * row_blocks + (c - row * kblocks);
+}
+
 template <class F, int... J>
 __device__ __forceinline__ void unrolled(F &&f, std::integer_sequence<int, J...>)
 {
@@ -138,11 +166,11 @@ __device__ __forceinline__ void unrolled(F &&f, std::integer_sequence<int, J...>
 }
 
 // SLOTS K blocks of (16 weight rows + 16 activation rows) x 128 bytes per wave: 4 KB a slot.
-template <int SDT, int PER, int SLOTS>
+template <int SDT, int PER, int SLOTS, bool LONGK = false>
 __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                                   int M, int64_t N, int64_t K, void *__restrict__ C,
-                                                                  int out_dtype)
+                                                                  int out_dtype, int rounds, int round_blocks)
 {
     constexpr int S0 = SLOTS < PER ? SLOTS : PER;        // blocks requested before the first one is used
     __shared__ __attribute__((aligned(1024))) uint8_t ring[kThinWaves * SLOTS * 4096];
@@ -151,10 +179,13 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l16 = lane & 15, lq = lane >> 4;
-    const int kblocks = (int)(K / 128);
+    const int row_blocks = (int)(K / 128);
     const int64_t n0 = (int64_t)blockIdx.x * 16;
     const int kb0 = wave * PER;
     const int m = l16 < M ? l16 : M - 1;
+    f32x4v acc;                                          // zeroed where the first round's run begins
+    auto round = [&](const int rd) {
+    LP_THIN_ROUND(SDT)
 
     // The activation-scale table [16, kblocks] goes through LDS (consecutive lanes on consecutive addresses
     // instead of 16-row gathers by every wave).  Its two requests per lane and everything that touches LDS before
@@ -163,9 +194,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
     uint32_t sv[2];
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
-        const int i = t + 64 * kThinWaves * q;
-        const int last = M * kblocks - 1;
-        const int idx = i < last ? i : last;
+        const int idx = table_index<LONGK>(t + 64 * kThinWaves * q, M, kblocks, row_blocks);
         if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
         else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
     }
@@ -192,7 +221,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
-        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * kblocks + kb);
+        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * row_blocks + kb);
     }
     const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
     asm volatile("s_waitcnt vmcnt(%2)" : "+v"(sv[0]), "+v"(sv[1]) : "n"(4 * S0) : "memory");          // the two oldest requests
@@ -218,7 +247,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
     // operand reads: lane (row lane % 16, part lane / 16) takes chunks 2 part and 2 part + 1 of its row
     const uint32_t ring0 = (uint32_t)(uintptr_t)LDS_PTR(wring);
     const uint32_t rd0 = ring0 + l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rd1 = ring0 + l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
-    f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (!LONGK || rd == 0) acc = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
     const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
     auto step = [&](auto jc) {
         constexpr int j = decltype(jc)::value;
@@ -239,6 +268,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring(const uint8_t 
         acc.w = __builtin_fmaf(p.w, sa[j], acc.w);
     };
     unrolled(step, std::make_integer_sequence<int, PER>{});
+    };
+    if constexpr (LONGK) {
+        for (int rd = 0; rd < rounds; ++rd) round(rd);
+    } else {
+        round(0);
+    }
 
     red[wave][lane] = acc;
     __syncthreads();
@@ -284,11 +319,11 @@ struct RingPlan {
     }
 };
 
-template <int SDT, int PER, int MB, int BS = 4, int AD = 2>
+template <int SDT, int PER, int MB, int BS = 4, int AD = 2, bool LONGK = false>
 __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                                    const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                                    int M, int64_t N, int64_t K, void *__restrict__ C,
-                                                                   int out_dtype)
+                                                                   int out_dtype, int rounds, int round_blocks)
 {
     constexpr int U = (MB + 1) / 2, UNITS = PER * U;
     constexpr int B0 = BS < PER ? BS : PER, A0 = AD < UNITS ? AD : UNITS;
@@ -300,17 +335,18 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l16 = lane & 15, lq = lane >> 4;
-    const int kblocks = (int)(K / 128);
+    const int row_blocks = (int)(K / 128);
     const int64_t n0 = (int64_t)blockIdx.x * 16;
     const int kb0 = wave * PER;
+    f32x4v acc[MB];                                      // zeroed where the first round's run begins
+    auto round = [&](const int rd) {
+    LP_THIN_ROUND(SDT)
 
     // scale table through LDS, requests and LDS accesses as asm with hand-placed waits (see gemm_thin_ring)
     uint32_t sv[SV];
 #pragma unroll
     for (int q = 0; q < SV; ++q) {
-        const int i = t + 64 * kThinWaves * q;
-        const int last = M * kblocks - 1;
-        const int idx = i < last ? i : last;
+        const int idx = table_index<LONGK>(t + 64 * kThinWaves * q, M, kblocks, row_blocks);
         if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
         else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
     }
@@ -346,7 +382,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
-        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * kblocks + kb);
+        sb[j] = gemm::scale_at<SDT>(Bs, (n0 >> 7) * row_blocks + kb);
     }
     const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * B0 + 4 * A0) : "memory");          // the table requests are the oldest
@@ -378,9 +414,10 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
 
     const uint32_t rdo0 = l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rdo1 = l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
     const uint32_t wb0 = (uint32_t)(uintptr_t)LDS_PTR(wb), wa0 = (uint32_t)(uintptr_t)LDS_PTR(wa);
-    f32x4v acc[MB];
+    if (!LONGK || rd == 0) {
 #pragma unroll
-    for (int g = 0; g < MB; ++g) acc[g] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int g = 0; g < MB; ++g) acc[g] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
     u32x4 w0, w1;                                        // weight fragment of the current block, kept over its units
     auto step = [&](auto uc) {
@@ -416,6 +453,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_ring2(const uint8_t
         }
     };
     unrolled(step, std::make_integer_sequence<int, UNITS>{});
+    };
+    if constexpr (LONGK) {
+        for (int rd = 0; rd < rounds; ++rd) round(rd);
+    } else {
+        round(0);
+    }
 
     // partial sums into the wave's own (drained) activation ring, then row group g is added up by wave g
     f32x4v *red = (f32x4v *)aring;                       // [wave][4 AD][lane]: the first 4 KB of each wave's own ring
@@ -474,11 +517,11 @@ struct RowsPlan {
     }
 };
 
-template <int SDT, int PER, int R, int U = 2>
+template <int SDT, int PER, int R, int U = 2, bool LONGK = false>
 __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t *__restrict__ Aq, const void *__restrict__ As,
                                                                   const uint8_t *__restrict__ Bq, const void *__restrict__ Bs,
                                                                   int M, int64_t N, int64_t K, void *__restrict__ C,
-                                                                  int out_dtype)
+                                                                  int out_dtype, int rounds, int round_blocks)
 {
     constexpr int MB = 2 * U, NBK = (R + 1) / 2, UNITS = PER * U, A0 = UNITS < 2 ? UNITS : 2;
     constexpr int SV = (16 * MB * kThinWaves * kThinRun + 64 * kThinWaves - 1) / (64 * kThinWaves);      // table entries per lane
@@ -489,24 +532,25 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int l16 = lane & 15, lq = lane >> 4;
-    const int kblocks = (int)(K / 128);
+    const int row_blocks = (int)(K / 128);
     const int64_t n0 = (int64_t)blockIdx.x * (8 * R);
     const int kb0 = wave * PER;
     if constexpr (U == 4) {
         // more than 128 activation rows: blockIdx.y picks a slice of 128 (the last one may be shorter)
         const int64_t r0 = (int64_t)blockIdx.y * 128;
         Aq += r0 * K;
-        As = (const char *)As + r0 * kblocks * (SDT == LP_F32 ? 4 : 1);
+        As = (const char *)As + r0 * row_blocks * (SDT == LP_F32 ? 4 : 1);
         C = (char *)C + r0 * N * (out_dtype == LP_BF16 ? 2 : 4);
         M = M - (int)r0 < 128 ? M - (int)r0 : 128;
     }
+    f32x4v acc[MB][NBK];                                 // zeroed where the first round's run begins
+    auto round = [&](const int rd) {
+    LP_THIN_ROUND(SDT)
 
     uint32_t sv[SV];
 #pragma unroll
     for (int q = 0; q < SV; ++q) {
-        const int i = t + 64 * kThinWaves * q;
-        const int last = M * kblocks - 1;
-        const int idx = i < last ? i : last;
+        const int idx = table_index<LONGK>(t + 64 * kThinWaves * q, M, kblocks, row_blocks);
         if (SDT == LP_F32) asm volatile("global_load_dword %0, %1, off" : "=v"(sv[q]) : "v"((const float *)As + idx));
         else asm volatile("global_load_ubyte %0, %1, off" : "=v"(sv[q]) : "v"((const uint8_t *)As + idx));
     }
@@ -551,7 +595,7 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
             const int kb = kb0 + j < kblocks ? kb0 + j : kblocks - 1;
-            sb[nb][j] = gemm::scale_at<SDT>(Bs, blk * kblocks + kb);
+            sb[nb][j] = gemm::scale_at<SDT>(Bs, blk * row_blocks + kb);
         }
     }
     const uint32_t ssa0 = (uint32_t)(uintptr_t)LDS_PTR(sSa);
@@ -590,11 +634,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
 
     const uint32_t rdo0 = l16 * 128 + (((2 * lq) ^ (l16 & 7)) << 4), rdo1 = l16 * 128 + (((2 * lq + 1) ^ (l16 & 7)) << 4);
     const uint32_t wb0 = (uint32_t)(uintptr_t)LDS_PTR(wb), wa0 = (uint32_t)(uintptr_t)LDS_PTR(wa);
-    f32x4v acc[MB][NBK];
+    if (!LONGK || rd == 0) {
 #pragma unroll
-    for (int g = 0; g < MB; ++g)
+        for (int g = 0; g < MB; ++g)
 #pragma unroll
-        for (int nb = 0; nb < NBK; ++nb) acc[g][nb] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int nb = 0; nb < NBK; ++nb) acc[g][nb] = f32x4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     const f32x4v zero = {0.0f, 0.0f, 0.0f, 0.0f};
     i32x8 wf[NBK];                                       // weight fragments of the current block, kept over its units
     auto step = [&](auto uc) {
@@ -637,6 +682,12 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
         }
     };
     unrolled(step, std::make_integer_sequence<int, UNITS>{});
+    };
+    if constexpr (LONGK) {
+        for (int rd = 0; rd < rounds; ++rd) round(rd);
+    } else {
+        round(0);
+    }
 
     // partial sums through the (drained) rings, as many row groups at a time as fit a wave's own ring (all of them in one pass
     // where they do: every pass costs two barriers at which the waves wait for the slowest): pair (g, nb) of the pass is
@@ -679,6 +730,34 @@ __global__ __launch_bounds__(64 * kThinWaves) void gemm_thin_rows(const uint8_t 
 namespace lowp {
 namespace gemm {
 
+// K longer than one run of the workgroup's waves (8 x kThinRun blocks = 7168): rounds of equal length inside the workgroup,
+// at most kThinMaxRounds of them (K <= 57344).  Returns the number of rounds and the K blocks of one.
+constexpr int kThinMaxRounds = 8;
+static int thin_rounds(int64_t K, int *round_blocks)
+{
+    const int64_t kblocks = K / 128, whole = kThinWaves * kThinRun;
+    const int rounds = (int)((kblocks + whole - 1) / whole);
+    *round_blocks = rounds <= 1 ? 0 : (int)((kblocks + rounds - 1) / rounds);
+    return rounds < 1 ? 1 : rounds;
+}
+
+// Which shapes of a long K the decode kernels take (one MI355X, us per call, tiled kernels or K-split pair -> rounds): up to
+// 16 rows all (1 x 7168 x 18432 64.1 -> 23.8, 8 x 7168 x 8192 32.5 -> 13.4, 16 x 4096 x 16384 18.7 -> 18.3); up to 64 rows from
+// 5120 to 8192 weight rows (64 x 7168 x 18432 70.4 -> 44.6, 64 x 5120 x 14336 55.8 -> 31.8, 64 x 6144 x 8192 34.9 -> 22.2, 64 x
+// 8192 x 8192 35.7 -> 24.0; but 64 x 4096 x 8192 18.0 -> 17.8, 32 x 2048 x 16384 15.6 -> 17.8, 48 x 18432 x 8192 37.3 -> 49.9);
+// up to 128 rows from 7168 weight rows (128 x 7168 x 18432 81.4 -> 70.5, 128 x 8192 x 8192 40.9 -> 35.4; but 128 x 4096 x 14336
+// 28.2 -> 39.7, 100 x 3072 x 9216 20.7 -> 26.1).  LP_GEMM_THIN_LONG_K = 0 / 1 (tuning aid): none / all of them.
+static bool long_k_ok(int64_t M, int64_t N, int64_t K)
+{
+    static const char *env = getenv("LP_GEMM_THIN_LONG_K");
+    if (K / 128 <= kThinWaves * kThinRun) return true;
+    if (K / 128 > kThinMaxRounds * kThinWaves * kThinRun || M > 128) return false;
+    if (env) return atoi(env) != 0;
+    if (M <= 16) return true;
+    if (M <= 64) return N >= 5120 && N <= 8192;
+    return N >= 7168;
+}
+
 bool thin_ok(int64_t M, int64_t N, int64_t K)
 {
     // one run of K blocks per wave.  Above 16 rows a workgroup holds 128 KB of LDS and its activations (M / 16 times the
@@ -688,7 +767,7 @@ bool thin_ok(int64_t M, int64_t N, int64_t K)
     // pair's two (one MI355X, us per call, pair -> this kernel: 32 x 2048 x 1024 8.8 -> 4.0, 64 x 2048 x 7168 16.0 -> 11.8,
     // 8 x 512 x 4096 10.1 -> 5.3, 16 x 128 x 7168 11.2 -> 5.3, 64 x 128 x 7168 12.4 -> 11.0).  LP_GEMM_THIN_FROM = n
     // (tuning aid): only from n groups of 16 weight rows.
-    if (M < 1 || M > 64 || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun) return false;
+    if (M < 1 || M > 64 || N % 16 != 0 || K % 128 != 0 || !long_k_ok(M, N, K)) return false;
     const int64_t groups = N / 16;
     static const int64_t min_groups = getenv("LP_GEMM_THIN_FROM") ? atoi(getenv("LP_GEMM_THIN_FROM")) : 1;
     return groups >= min_groups && groups <= (M <= 16 ? 0x7FFFFFFF : 512);
@@ -715,7 +794,7 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     // 13.7 -> 13.1).  LP_GEMM_THIN_ROWS_WIDE_FROM = n (tuning aid): only from n groups of 16 weight rows.
     static const int64_t max_m = getenv("LP_GEMM_THIN_ROWS_MAX_M") ? atoi(getenv("LP_GEMM_THIN_ROWS_MAX_M")) : 128;
     static const int64_t wide_max_n = getenv("LP_GEMM_THIN_ROWS_WIDE_N") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_N")) : 8192;
-    if (off || N % 16 != 0 || K % 128 != 0 || K / 128 > kThinWaves * kThinRun || N * K >= 0xFFFFFFFFll) return false;
+    if (off || N % 16 != 0 || K % 128 != 0 || !long_k_ok(M, N, K) || N * K >= 0xFFFFFFFFll) return false;
     static const int64_t wide_min_groups = getenv("LP_GEMM_THIN_ROWS_WIDE_FROM") ? atoi(getenv("LP_GEMM_THIN_ROWS_WIDE_FROM")) : 1;
     if (M > 128) {
         // slices of 128 rows (blockIdx.y) in one launch, where all workgroups run at once and the tiled kernels would give most
@@ -737,15 +816,24 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     return M >= min_m && N / 16 > min_groups;
 }
 
+// the variant that walks a long K in rounds exists from four K blocks per wave on (two rounds cover at least 57 blocks)
+#define LP_LAUNCH_LONGK(LONG_KERNEL, KERNEL, ...)                                                        \
+    do {                                                                                                 \
+        if constexpr (PER >= 4) {                                                                        \
+            if (rounds > 1) { hipLaunchKernelGGL(LONG_KERNEL, __VA_ARGS__); break; }                     \
+        }                                                                                                \
+        hipLaunchKernelGGL(KERNEL, __VA_ARGS__);                                                         \
+    } while (0)
+
 template <int SDT, int PER, int R>
 void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-                        int out_dtype, hipStream_t st)
+                        int out_dtype, int rounds, int round_blocks, hipStream_t st)
 {
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
     if constexpr (R == 2) {
         // 16 weight rows per workgroup exist from 65 activation rows on only (up to 64 the ring kernels serve that cut)
-        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
-                           C, out_dtype);
+        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype, rounds, round_blocks);
         return;
     }
     if constexpr (R == 4) {
@@ -753,33 +841,33 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
         // row blocks no longer fit the registers, and a spill's reload would go through the request counter this kernel
         // counts by hand)
         if (M > 64) {
-            hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
-                               C, out_dtype);
+            LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                               C, out_dtype, rounds, round_blocks);
             return;
         }
     }
     if (M <= 32)
-        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
-                           C, out_dtype);
+        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 1, true>), (gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype, rounds, round_blocks);
     else
-        hipLaunchKernelGGL((gemm_thin_rows<SDT, PER, R, 2>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
-                           C, out_dtype);
+        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 2, true>), (gemm_thin_rows<SDT, PER, R, 2>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+                           C, out_dtype, rounds, round_blocks);
 }
 
 template <int SDT, int PER>
 void launch_thin_rows_per(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-                          int out_dtype, int per, int r, hipStream_t st)
+                          int out_dtype, int per, int r, int rounds, int round_blocks, hipStream_t st)
 {
     if constexpr (PER > 1) {
-        if (per < PER) return launch_thin_rows_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, r, st);
+        if (per < PER) return launch_thin_rows_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, r, rounds, round_blocks, st);
     }
     switch (r) {
-    case 2: return launch_thin_rows_r<SDT, PER, 2>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
-    case 4: return launch_thin_rows_r<SDT, PER, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
-    case 6: return launch_thin_rows_r<SDT, PER, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
-    case 8: return launch_thin_rows_r<SDT, PER, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
-    case 9: return launch_thin_rows_r<SDT, PER, 9>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
-    default: return launch_thin_rows_r<SDT, PER, 10>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, st);
+    case 2: return launch_thin_rows_r<SDT, PER, 2>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
+    case 4: return launch_thin_rows_r<SDT, PER, 4>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
+    case 6: return launch_thin_rows_r<SDT, PER, 6>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
+    case 8: return launch_thin_rows_r<SDT, PER, 8>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
+    case 9: return launch_thin_rows_r<SDT, PER, 9>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
+    default: return launch_thin_rows_r<SDT, PER, 10>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, rounds, round_blocks, st);
     }
 }
 
@@ -787,7 +875,9 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
                      void *C, int out_dtype, hipStream_t st)
 {
     static const int forced = getenv("LP_GEMM_THIN_ROWS") ? atoi(getenv("LP_GEMM_THIN_ROWS")) : 0;     // tuning aid: 2, 4, 6, 8, 9, 10
-    const int kblocks = (int)(K / 128);
+    int round_blocks = 0;
+    const int rounds = thin_rounds(K, &round_blocks);
+    const int kblocks = rounds > 1 ? round_blocks : (int)(K / 128);
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
     int best = 10;
     int64_t best_cost = INT64_MAX;
@@ -799,43 +889,45 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
         if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
     }
     if ((forced == 2 || forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M > 64 ? forced <= 4 : forced >= 4)) best = forced;
-    if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
-    else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, st);
+    if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, rounds, round_blocks, st);
+    else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, rounds, round_blocks, st);
     return check_launch("lp_gemm_fp8_block(thin, many rows)");
 }
 
 template <int SDT, int PER>
 void launch_thin_per(const void *Aq, const void *As, const void *Bq, const void *Bs, int64_t M, int64_t N, int64_t K, void *C,
-                     int out_dtype, int per, int kind, hipStream_t st)
+                     int out_dtype, int per, int kind, int rounds, int round_blocks, hipStream_t st)
 {
     if constexpr (PER > 1) {
-        if (per < PER) return launch_thin_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
+        if (per < PER) return launch_thin_per<SDT, PER - 1>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, rounds, round_blocks, st);
     }
     const dim3 grid((unsigned)(N / 16)), block(64 * kThinWaves);
     const uint8_t *a = (const uint8_t *)Aq, *b = (const uint8_t *)Bq;
     // 49 to 64 rows: weight ring three blocks deep and activation ring three units (158 KB of LDS; with four and two,
     // 142 KB, M = 64, N = 4096, K = 7168 takes 12.9 instead of 12.75 us)
-    if (M > 48) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 4, 3, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
-    else if (M > 32) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
-    else if (M > 16) hipLaunchKernelGGL((gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    if (M > 48) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 4, 3, 3, true>), (gemm_thin_ring2<SDT, PER, 4, 3, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else if (M > 32) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 3, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else if (M > 16) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 2, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
     else if (kind == 0) hipLaunchKernelGGL((gemm_thin<SDT, PER>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
-    else if (kind == 4) hipLaunchKernelGGL((gemm_thin_ring<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
-    else hipLaunchKernelGGL((gemm_thin_ring<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
+    else if (kind == 4) LP_LAUNCH_LONGK((gemm_thin_ring<SDT, PER, 4, true>), (gemm_thin_ring<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else LP_LAUNCH_LONGK((gemm_thin_ring<SDT, PER, 2, true>), (gemm_thin_ring<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
 }
 
 int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
                 void *C, int out_dtype, hipStream_t st)
 {
-    const int kblocks = (int)(K / 128);
+    int round_blocks = 0;
+    const int rounds = thin_rounds(K, &round_blocks);
+    const int kblocks = rounds > 1 ? round_blocks : (int)(K / 128);
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
     // ring depth 2 (64 KB of LDS: two workgroups share a CU and one's tail overlaps the other's start) measured
     // as fast as depth 4 with one workgroup per CU at N = 4096 and faster beyond
     static const char *env = getenv("LP_GEMM_THIN_DIRECT");                      // tuning aids
     static const char *slots_env = getenv("LP_GEMM_THIN_SLOTS");
-    int kind = env ? 0 : 2;
+    int kind = env && rounds == 1 ? 0 : 2;              // (the kernel without rings takes no long K)
     if (!env && slots_env) kind = atoi(slots_env) == 4 ? 4 : 2;
-    if (scale_dtype == LP_F32) launch_thin_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
-    else launch_thin_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, st);
+    if (scale_dtype == LP_F32) launch_thin_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, rounds, round_blocks, st);
+    else launch_thin_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, kind, rounds, round_blocks, st);
     return check_launch("lp_gemm_fp8_block(thin)");
 }
 
