@@ -9,6 +9,7 @@ has already loaded.
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -49,15 +50,43 @@ def _compile(src: str, force: bool) -> str:
     spath = os.path.join(CSRC, src)
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(spath), _headers_mtime()):
         return obj
-    cmd = [HIPCC] + COMMON + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", spath, "-o", obj]
+    audited = src in SPILL_AUDIT
+    cmd = [HIPCC] + COMMON + (["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"] if audited else [])
+    cmd += (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", spath, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the packed-fp32 feature: harmless
-    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if audited:
+        spilled = _kernels_with_scratch(r.stderr, SPILL_AUDIT[src])
+        if spilled:
+            os.remove(obj)
+            raise RuntimeError(f"{src}: kernels that count their memory requests by hand must not spill registers "
+                               f"(a spill's reload goes through the same counter and costs them most of their rate): "
+                               + ", ".join(f"{n} ({b} bytes per lane)" for n, b in spilled))
     if err.strip():
         sys.stderr.write(err + "\n")
     return obj
+
+
+# Sources whose kernels are checked for register spills at build time (the compiler's own resource remarks), with the
+# mangled-name pattern of the kernels that must have none.  gemm_thin.hip: the single-run decode kernels (their last
+# template argument, LONGK, false: "Lb0E"); the variants that walk a long K in rounds are allowed theirs.
+SPILL_AUDIT = {"gemm_thin.hip": re.compile(r"gemm_thin(_ring2?|_rows)?I.*Lb0EEEv|gemm_thinILi")}
+
+
+def _kernels_with_scratch(remarks: str, pattern):
+    out, name = [], None
+    for line in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            continue
+        m = re.search(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and int(m.group(1)) > 0 and pattern.search(name):
+            out.append((name, int(m.group(1))))
+    return out
 
 
 def _generate():
