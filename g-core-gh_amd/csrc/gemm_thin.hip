@@ -742,7 +742,8 @@ static int thin_rounds(int64_t K, int *round_blocks)
 }
 
 // Which shapes of a long K the decode kernels take (one MI355X, us per call, tiled kernels or K-split pair -> rounds): up to
-// 16 rows all (1 x 7168 x 18432 64.1 -> 23.8, 8 x 7168 x 8192 32.5 -> 13.4, 16 x 4096 x 16384 18.7 -> 18.3); up to 64 rows from
+// 16 rows all from 4096 weight rows and, with fewer, up to two rounds (1 x 7168 x 18432 64.1 -> 23.8, 8 x 7168 x 8192 32.5 -> 13.4,
+// 12 x 12288 x 8192 35.5 -> 20.0, 16 x 18432 x 8192 37.8 -> 29.7, 16 x 4096 x 16384 18.7 -> 18.3, 2 x 512 x 8192 9.1 -> 8.0); up to 64 rows from
 // 5120 to 8192 weight rows (64 x 7168 x 18432 70.4 -> 44.6, 64 x 5120 x 14336 55.8 -> 31.8, 64 x 6144 x 8192 34.9 -> 22.2, 64 x
 // 8192 x 8192 35.7 -> 24.0; but 64 x 4096 x 8192 18.0 -> 17.8, 32 x 2048 x 16384 15.6 -> 17.8, 48 x 18432 x 8192 37.3 -> 49.9);
 // up to 128 rows from 7168 weight rows (128 x 7168 x 18432 81.4 -> 70.5, 128 x 8192 x 8192 40.9 -> 35.4; but 128 x 4096 x 14336
@@ -753,7 +754,7 @@ static bool long_k_ok(int64_t M, int64_t N, int64_t K)
     if (K / 128 <= kThinWaves * kThinRun) return true;
     if (K / 128 > kThinMaxRounds * kThinWaves * kThinRun || M > 128) return false;
     if (env) return atoi(env) != 0;
-    if (M <= 16) return true;
+    if (M <= 16) return N >= 4096 || K / 128 <= 2 * kThinWaves * kThinRun;        // (16 x 1024 x 20480, three rounds on 64 workgroups: 15.1 -> 17.6)
     if (M <= 64) return N >= 5120 && N <= 8192;
     return N >= 7168;
 }

@@ -93,7 +93,7 @@ DENSE_SHAPES = [
     (513, 2048, 1024), (256, 4096, 512), (8192, 128, 1024), (5000, 128, 2048), (2048, 512, 4096), (1300, 768, 3072), (2049, 256, 4096),
     # K beyond 7168 on the decode kernels: the workgroup walks K in rounds (two rounds of 29 blocks with a ragged last run, eight
     # rounds, every kernel of the family), and shapes the rule leaves to the tiled kernels
-    (1, 4096, 14336), (16, 7168, 8192), (64, 5120, 7296), (40, 6144, 9216), (128, 7168, 8192), (8, 256, 57344), (13, 18432, 8192),
+    (1, 4096, 14336), (16, 7168, 8192), (64, 5120, 7296), (40, 6144, 9216), (128, 7168, 8192), (8, 4096, 57344), (8, 256, 14336), (13, 18432, 8192),
     (64, 8192, 14336), (33, 7168, 18432), (48, 4096, 8192), (100, 3072, 9216),
 ]
 
