@@ -17,6 +17,15 @@ __all__ = ["grouped_gemm_fp8", "grouped_gemm_fp8_nn", "m_grouped_gemm_fp8_fp8_bf
            "quant_fp8_colwise_t", "gemm_fp8_rowscale"]
 
 
+
+def _quant_pow2(value: torch.Tensor, block_size):
+    """quant_fp8_e4m3_scale_e8m0's codes and scales without its NaN assertion, which reads a counter back from the device
+    and so stalls the stream once per call: inside the grouped linear (three quantisations per step and layer) a NaN
+    simply propagates into the product, as it does in the reference, whose layer quantises inside TransformerEngine
+    (fp8.py:180-343) without such a check."""
+    q, s, _ = ops.quant_fp8_block(value, block_size, scale_mode=A.SCALE_POW2, scale_dtype=ops.E8M0, count_nan=False)
+    return q, s
+
 def _scale_arg(s, dev):
     s = s.to(dev)
     if s.dtype == ops.E8M0:
@@ -248,8 +257,7 @@ class _GroupedGemmFp8(torch.autograd.Function):
     def forward(ctx, inp, weight, wq, ws, m_splits, out_dtype):
         E, n_out, k_in = wq.shape
         x = inp.reshape(-1, k_in)
-        from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
-        xq, xs = quant_fp8_e4m3_scale_e8m0(x, block_size=(1, 128))
+        xq, xs = _quant_pow2(x, (1, 128))
         offs = _offsets(m_splits, x.device)
         out = grouped_gemm_fp8(xq, xs, wq, ws, offs, out_dtype=out_dtype, total_rows=sum(m_splits))
         ctx.need_wgrad = weight is not None and weight.requires_grad
@@ -265,13 +273,12 @@ class _GroupedGemmFp8(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
         E, n_out, k_in = ctx.dims
         wq, ws, offs = ctx.saved_tensors[:3]
         dy = grad_output.contiguous().view(-1, n_out)
         dgrad = wgrad = None
         if ctx.need_dgrad:
-            dyq, dys = quant_fp8_e4m3_scale_e8m0(dy, block_size=(1, 128))
+            dyq, dys = _quant_pow2(dy, (1, 128))
             dgrad = grouped_gemm_fp8_nn(dyq, dys, wq.view(ops.E4M3), ws.view(ops.E8M0), offs, out_dtype=ctx.out_dtype,
                                         total_rows=sum(ctx.m_splits)).view(ctx.inp_shape)
         if ctx.need_wgrad:
@@ -307,10 +314,9 @@ class MyTeGroupedLinearFp8(torch.nn.Module):
         n_out, k_in = shape[1], shape[2]
         assert inp.size(-1) == k_in, (inp.size(-1), k_in)
         assert sum(m_splits) == inp.numel() // k_in, (sum(m_splits), inp.numel() // k_in)
-        from .eager_quant_kernels import quant_fp8_e4m3_scale_e8m0
         if wq is None:
             # Float8BlockScaling recipe: power-of-two scales for activations and weights
-            wq, ws = quant_fp8_e4m3_scale_e8m0(weight.detach(), block_size=(128, 128))
+            wq, ws = _quant_pow2(weight.detach(), (128, 128))
         if wq.dtype == torch.uint8:
             wq = wq.view(ops.E4M3)
         if ws.dtype != ops.E8M0:
