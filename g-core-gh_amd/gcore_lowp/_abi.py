@@ -90,7 +90,14 @@ def require_gpu() -> torch.device:
     return torch.device("cuda", torch.cuda.current_device())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr() -> int:
+    """The current stream of the current device as the handle the C ABI takes.  Through torch's raw accessor where it
+    exists: building a Stream object per call cost 4 us of the 15 an eager decode GEMM call takes."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
