@@ -746,17 +746,17 @@ static int thin_rounds(int64_t K, int *round_blocks)
 // 12 x 12288 x 8192 35.5 -> 20.0, 16 x 18432 x 8192 37.8 -> 29.7, 16 x 4096 x 16384 18.7 -> 18.3, 2 x 512 x 8192 9.1 -> 8.0); up to 64 rows from
 // 5120 to 8192 weight rows (64 x 7168 x 18432 70.4 -> 44.6, 64 x 5120 x 14336 55.8 -> 31.8, 64 x 6144 x 8192 34.9 -> 22.2, 64 x
 // 8192 x 8192 35.7 -> 24.0; but 64 x 4096 x 8192 18.0 -> 17.8, 32 x 2048 x 16384 15.6 -> 17.8, 48 x 18432 x 8192 37.3 -> 49.9);
-// up to 128 rows from 7168 weight rows (128 x 7168 x 18432 81.4 -> 70.5, 128 x 8192 x 8192 40.9 -> 35.4; but 128 x 4096 x 14336
-// 28.2 -> 39.7, 100 x 3072 x 9216 20.7 -> 26.1).  LP_GEMM_THIN_LONG_K = 0 / 1 (tuning aid): none / all of them.
+// not above 64 rows (128 x 4096 x 14336 28.2 -> 39.7, 100 x 3072 x 9216 20.7 -> 26.1; the gains at 7168 weight rows and more
+// came from a variant that spilled).  LP_GEMM_THIN_LONG_K = 0 / 1 (tuning aid): none / all of them up to 64 rows.
 static bool long_k_ok(int64_t M, int64_t N, int64_t K)
 {
     static const char *env = getenv("LP_GEMM_THIN_LONG_K");
     if (K / 128 <= kThinWaves * kThinRun) return true;
-    if (K / 128 > kThinMaxRounds * kThinWaves * kThinRun || M > 128) return false;
+    if (K / 128 > kThinMaxRounds * kThinWaves * kThinRun || M > 64) return false;
     if (env) return atoi(env) != 0;
     if (M <= 16) return N >= 4096 || K / 128 <= 2 * kThinWaves * kThinRun;        // (16 x 1024 x 20480, three rounds on 64 workgroups: 15.1 -> 17.6)
     if (M <= 64) return N >= 5120 && N <= 8192;
-    return N >= 7168;
+    return false;          // (65 .. 128 rows: 128 x 7168 x 18432 81.4 -> 70.5 us with a variant that spills registers; not kept, see LP_LAUNCH_LONGK)
 }
 
 bool thin_ok(int64_t M, int64_t N, int64_t K)
@@ -817,10 +817,13 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     return M >= min_m && N / 16 > min_groups;
 }
 
-// the variant that walks a long K in rounds exists from four K blocks per wave on (two rounds cover at least 57 blocks)
-#define LP_LAUNCH_LONGK(LONG_KERNEL, KERNEL, ...)                                                        \
+// The variant that walks a long K in rounds exists from four K blocks per wave on (two rounds cover at least 57 blocks)
+// and only where it needs no scratch (OK): loads and stores share one request counter and complete out of order with
+// respect to each other, so a spill's store inside the run could satisfy a hand-counted wait before the request that
+// wait is for has landed.  The host never asks for a long K where the variant is missing (long_k_ok, the choice of R).
+#define LP_LAUNCH_LONGK(OK, LONG_KERNEL, KERNEL, ...)                                                    \
     do {                                                                                                 \
-        if constexpr (PER >= 4) {                                                                        \
+        if constexpr (PER >= 4 && (OK)) {                                                                \
             if (rounds > 1) { hipLaunchKernelGGL(LONG_KERNEL, __VA_ARGS__); break; }                     \
         }                                                                                                \
         hipLaunchKernelGGL(KERNEL, __VA_ARGS__);                                                         \
@@ -833,7 +836,7 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
     const dim3 grid((unsigned)((N + 8 * R - 1) / (8 * R))), block(64 * kThinWaves);
     if constexpr (R == 2) {
         // 16 weight rows per workgroup exist from 65 activation rows on only (up to 64 the ring kernels serve that cut)
-        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+        LP_LAUNCH_LONGK(false, (gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                            C, out_dtype, rounds, round_blocks);
         return;
     }
@@ -842,16 +845,16 @@ void launch_thin_rows_r(const void *Aq, const void *As, const void *Bq, const vo
         // row blocks no longer fit the registers, and a spill's reload would go through the request counter this kernel
         // counts by hand)
         if (M > 64) {
-            LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+            LP_LAUNCH_LONGK(false, (gemm_thin_rows<SDT, PER, R, 4, true>), (gemm_thin_rows<SDT, PER, R, 4>), dim3(grid.x, (unsigned)((M + 127) / 128)), block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                                C, out_dtype, rounds, round_blocks);
             return;
         }
     }
     if (M <= 32)
-        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 1, true>), (gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+        LP_LAUNCH_LONGK(true, (gemm_thin_rows<SDT, PER, R, 1, true>), (gemm_thin_rows<SDT, PER, R, 1>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                            C, out_dtype, rounds, round_blocks);
     else
-        LP_LAUNCH_LONGK((gemm_thin_rows<SDT, PER, R, 2, true>), (gemm_thin_rows<SDT, PER, R, 2>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
+        LP_LAUNCH_LONGK(R <= 6, (gemm_thin_rows<SDT, PER, R, 2, true>), (gemm_thin_rows<SDT, PER, R, 2>), grid, block, 0, st, (const uint8_t *)Aq, As, (const uint8_t *)Bq, Bs, (int)M, N, K,
                            C, out_dtype, rounds, round_blocks);
 }
 
@@ -885,11 +888,15 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
     const int64_t slices = M > 64 ? (M + 127) / 128 : 1;
     for (int r : {2, 4, 6, 8, 9, 10}) {
         if (M > 64 ? r > 4 : r < 4) continue;
+        if (rounds > 1 && M > 32 && r > 6) continue;        // (no long-K variant with two activation units and more rows)
         // a workgroup's time goes with the bytes it pulls: 8 r weight rows and, from 65 rows on, 128 activation rows
         const int64_t wgs = slices * ((N + 8 * r - 1) / (8 * r)), cost = ((wgs + 255) / 256) * (M > 64 ? 16 + r : r);
         if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
     }
     if ((forced == 2 || forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M > 64 ? forced <= 4 : forced >= 4)) best = forced;
+    if (rounds > 1 && (M > 64 || (M > 32 && best > 6)))
+        return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: no decode kernel for K = %lld with %lld rows and %d weight rows per workgroup",
+                    (long long)K, (long long)M, 8 * best);
     if (scale_dtype == LP_F32) launch_thin_rows_per<LP_F32, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, rounds, round_blocks, st);
     else launch_thin_rows_per<LP_E8M0, kThinRun>(Aq, As, Bq, Bs, M, N, K, C, out_dtype, per, best, rounds, round_blocks, st);
     return check_launch("lp_gemm_fp8_block(thin, many rows)");
@@ -906,12 +913,12 @@ void launch_thin_per(const void *Aq, const void *As, const void *Bq, const void 
     const uint8_t *a = (const uint8_t *)Aq, *b = (const uint8_t *)Bq;
     // 49 to 64 rows: weight ring three blocks deep and activation ring three units (158 KB of LDS; with four and two,
     // 142 KB, M = 64, N = 4096, K = 7168 takes 12.9 instead of 12.75 us)
-    if (M > 48) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 4, 3, 3, true>), (gemm_thin_ring2<SDT, PER, 4, 3, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
-    else if (M > 32) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 3, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
-    else if (M > 16) LP_LAUNCH_LONGK((gemm_thin_ring2<SDT, PER, 2, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    if (M > 48) LP_LAUNCH_LONGK(true, (gemm_thin_ring2<SDT, PER, 4, 3, 3, true>), (gemm_thin_ring2<SDT, PER, 4, 3, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else if (M > 32) LP_LAUNCH_LONGK(true, (gemm_thin_ring2<SDT, PER, 3, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 3>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else if (M > 16) LP_LAUNCH_LONGK(true, (gemm_thin_ring2<SDT, PER, 2, 4, 2, true>), (gemm_thin_ring2<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
     else if (kind == 0) hipLaunchKernelGGL((gemm_thin<SDT, PER>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype);
-    else if (kind == 4) LP_LAUNCH_LONGK((gemm_thin_ring<SDT, PER, 4, true>), (gemm_thin_ring<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
-    else LP_LAUNCH_LONGK((gemm_thin_ring<SDT, PER, 2, true>), (gemm_thin_ring<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else if (kind == 4) LP_LAUNCH_LONGK(true, (gemm_thin_ring<SDT, PER, 4, true>), (gemm_thin_ring<SDT, PER, 4>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
+    else LP_LAUNCH_LONGK(true, (gemm_thin_ring<SDT, PER, 2, true>), (gemm_thin_ring<SDT, PER, 2>), grid, block, 0, st, a, As, b, Bs, (int)M, N, K, C, out_dtype, rounds, round_blocks);
 }
 
 int launch_thin(const void *Aq, const void *As, const void *Bq, const void *Bs, int scale_dtype, int64_t M, int64_t N, int64_t K,
