@@ -58,3 +58,22 @@ def test_accumulation_registers_outside_asm_are_reported():
                       "\tv_accvgpr_write_b32 a17, v3 ; 4-byte Folded Spill", "\t.amdhsa_accum_offset 256", "_Z5otherv:",
                       "\tv_accvgpr_read_b32 v0, a3"])
     assert C.accumulation_registers_outside_asm(text, "gemm_asm_quad") == ["_Z13gemm_asm_quadv: v_accvgpr_write_b32 a17, v3"]
+
+
+def test_build_refuses_decode_kernels_that_spill():
+    """The decode kernels count their memory requests by hand; a spilled register's store and reload go through the same
+    counter.  build.py reads the compiler's resource remarks for gemm_thin.hip and refuses to link when one of those
+    kernels uses scratch: here the reader of those remarks, on a made-up excerpt."""
+    spec = importlib.util.spec_from_file_location("lowp_build", os.path.join(os.path.dirname(CSRC), "build.py"))
+    B = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(B)
+    line = "gemm_thin.hip:525:1: remark: {} [-Rpass-analysis=kernel-resource-usage]"
+    def kernel(name, scratch):
+        return [line.format(f"Function Name: {name}"), line.format("    VGPRs: 128"),
+                line.format(f"    ScratchSize [bytes/lane]: {scratch}"), line.format("    VGPRs Spill: 0")]
+    remarks = "\n".join(kernel("_ZN12_GLOBAL__N_114gemm_thin_rowsILi0ELi7ELi9ELi2ELb0EEEvPKh", 0)
+                        + kernel("_ZN12_GLOBAL__N_115gemm_thin_ring2ILi2ELi7ELi4ELi3ELi3ELb1EEEvPKh", 24)
+                        + kernel("_ZN12_GLOBAL__N_19some_otherEvPKh", 64))
+    pattern = B.SPILL_AUDIT["gemm_thin.hip"]
+    assert B._kernels_with_scratch(remarks, pattern) == [("_ZN12_GLOBAL__N_115gemm_thin_ring2ILi2ELi7ELi4ELi3ELi3ELb1EEEvPKh", 24)]
+    assert B._kernels_with_scratch(remarks.replace(": 24", ": 0"), pattern) == []
