@@ -447,16 +447,19 @@ def main():
     if want("c3"):
         # -------------------------------------------------------------- config 3: skinny GEMM, and the same 64 tokens
         # against config 2's 18432 weight rows (a 132 MB weight stream, long enough to amortise launch and first bytes)
-        K3 = 7168
-        a3 = randn(64, K3)
-        a3q = torch.empty(64, K3, dtype=torch.uint8, device=dev)
-        a3s = torch.empty(64, K3 // 128, dtype=torch.float32, device=dev)
-        quant_into(a3, 1, 128, a3q, a3s)
+        # (and the transposed projection, K = 18432 against 7168 weight rows, which the decode kernels walk in three rounds
+        # of K, with 64 tokens and with one)
         ms_empty, _ = time_launches([lambda: PA.check(LP.lp_probe_stream(None, 0, None, 0, 256, stream()))], 48, 12)
         sink = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
-        for tag, probe_tag, M3, N3, sets in (("c3_skinny_gemm", "c3_floor_probe", 64, 4096, 12),
-                                             ("decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", 64, 18432, 4)):
-            w3q, w3s = [], []                           # sets x N3 x 7168 bytes of weights > 256 MB
+        for tag, probe_tag, M3, N3, K3, sets in (("c3_skinny_gemm", "c3_floor_probe", 64, 4096, 7168, 12),
+                                                 ("decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", 64, 18432, 7168, 4),
+                                                 ("decode_gemm_64x7168x18432", "decode_64x7168x18432_floor_probe", 64, 7168, 18432, 4),
+                                                 ("decode_gemm_1x7168x18432", "decode_1x7168x18432_floor_probe", 1, 7168, 18432, 4)):
+            a3 = randn(M3, K3)
+            a3q = torch.empty(M3, K3, dtype=torch.uint8, device=dev)
+            a3s = torch.empty(M3, K3 // 128, dtype=torch.float32, device=dev)
+            quant_into(a3, 1, 128, a3q, a3s)
+            w3q, w3s = [], []                           # sets x N3 x K3 bytes of weights > 256 MB
             for _ in range(sets):
                 w = randn(N3, K3, std=0.02)
                 q = torch.empty(N3, K3, dtype=torch.uint8, device=dev)
@@ -487,7 +490,7 @@ def main():
             probes["bare_read_best_GB/s"] = wbytes / best / 1e3
             probes["gemm_over_bare_read"] = ms3 * 1e3 / best
             extras[probe_tag] = probes
-            del w3q, w3s, c3, ws
+            del w3q, w3s, c3, ws, a3, a3q, a3s
             torch.cuda.empty_cache()
         del sink
 
