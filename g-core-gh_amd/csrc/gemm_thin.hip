@@ -744,10 +744,29 @@ static int thin_rounds(int64_t K, int *round_blocks)
 // Which shapes of a long K the decode kernels take (one MI355X, us per call, tiled kernels or K-split pair -> rounds): up to
 // 16 rows all from 4096 weight rows and, with fewer, up to two rounds (1 x 7168 x 18432 64.1 -> 23.8, 8 x 7168 x 8192 32.5 -> 13.4,
 // 12 x 12288 x 8192 35.5 -> 20.0, 16 x 18432 x 8192 37.8 -> 29.7, 16 x 4096 x 16384 18.7 -> 18.3, 2 x 512 x 8192 9.1 -> 8.0); up to 64 rows from
-// 5120 to 8192 weight rows (64 x 7168 x 18432 70.4 -> 44.6, 64 x 5120 x 14336 55.8 -> 31.8, 64 x 6144 x 8192 34.9 -> 22.2, 64 x
-// 8192 x 8192 35.7 -> 24.0; but 64 x 4096 x 8192 18.0 -> 17.8, 32 x 2048 x 16384 15.6 -> 17.8, 48 x 18432 x 8192 37.3 -> 49.9);
+// 5120 weight rows (64 x 7168 x 18432 70.4 -> 44.6, 64 x 5120 x 14336 55.8 -> 31.8, 64 x 6144 x 8192 34.9 -> 22.2, 64 x 8192 x 8192
+// 35.7 -> 24.0, 32 x 12288 x 14336 56.0 -> 35.2, 24 x 36864 x 8192 78.9 -> 57.1, 64 x 12288 x 8192 37.0 -> 28.7; but 64 x 4096 x
+// 8192 18.0 -> 17.8, 32 x 2048 x 16384 15.6 -> 17.8, and above 32 rows 48 x 18432 x 8192 36.3 -> 47.9, see below);
 // not above 64 rows (128 x 4096 x 14336 28.2 -> 39.7, 100 x 3072 x 9216 20.7 -> 26.1; the gains at 7168 weight rows and more
 // came from a variant that spilled).  LP_GEMM_THIN_LONG_K = 0 / 1 (tuning aid): none / all of them up to 64 rows.
+// Weight rows per workgroup of the many-rows kernel, / 8: the R for which rounds of 256 workgroups x bytes a workgroup pulls
+// are fewest (the larger R when they tie); *wgs_out = its workgroups.
+static int choose_rows_r(int64_t M, int64_t N, bool long_k, int64_t *wgs_out)
+{
+    int best = 10;
+    int64_t best_cost = INT64_MAX, best_wgs = 0;
+    const int64_t slices = M > 64 ? (M + 127) / 128 : 1;
+    for (int r : {2, 4, 6, 8, 9, 10}) {
+        if (M > 64 ? r > 4 : r < 4) continue;
+        if (long_k && M > 32 && r > 6) continue;        // (no long-K variant with two activation units and more rows)
+        // a workgroup's time goes with the bytes it pulls: 8 r weight rows and, from 65 rows on, 128 activation rows
+        const int64_t wgs = slices * ((N + 8 * r - 1) / (8 * r)), cost = ((wgs + 255) / 256) * (M > 64 ? 16 + r : r);
+        if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; best_wgs = wgs; }
+    }
+    if (wgs_out) *wgs_out = best_wgs;
+    return best;
+}
+
 static bool long_k_ok(int64_t M, int64_t N, int64_t K)
 {
     static const char *env = getenv("LP_GEMM_THIN_LONG_K");
@@ -755,7 +774,13 @@ static bool long_k_ok(int64_t M, int64_t N, int64_t K)
     if (K / 128 > kThinMaxRounds * kThinWaves * kThinRun || M > 64) return false;
     if (env) return atoi(env) != 0;
     if (M <= 16) return N >= 4096 || K / 128 <= 2 * kThinWaves * kThinRun;        // (16 x 1024 x 20480, three rounds on 64 workgroups: 15.1 -> 17.6)
-    if (M <= 64) return N >= 5120 && N <= 8192;
+    if (N < 5120) return false;
+    if (M <= 32) return true;
+    // 33 .. 64 rows take at most 48 weight rows per workgroup here: not where that leaves the last round of workgroups badly
+    // filled (N = 18432: 384 workgroups; 48 x 18432 x 8192 36.3 -> 47.9 us, where 12288 rows, 256 workgroups, go 36.2 -> 27.0)
+    int64_t wgs = 0;
+    (void)choose_rows_r(M, N, true, &wgs);
+    if (M <= 64) return wgs <= 256 || wgs * 100 >= ((wgs + 255) / 256) * 256 * 85;
     return false;          // (65 .. 128 rows: 128 x 7168 x 18432 81.4 -> 70.5 us with a variant that spills registers; not kept, see LP_LAUNCH_LONGK)
 }
 
@@ -883,16 +908,7 @@ int launch_thin_rows(const void *Aq, const void *As, const void *Bq, const void 
     const int rounds = thin_rounds(K, &round_blocks);
     const int kblocks = rounds > 1 ? round_blocks : (int)(K / 128);
     const int per = (kblocks + kThinWaves - 1) / kThinWaves;
-    int best = 10;
-    int64_t best_cost = INT64_MAX;
-    const int64_t slices = M > 64 ? (M + 127) / 128 : 1;
-    for (int r : {2, 4, 6, 8, 9, 10}) {
-        if (M > 64 ? r > 4 : r < 4) continue;
-        if (rounds > 1 && M > 32 && r > 6) continue;        // (no long-K variant with two activation units and more rows)
-        // a workgroup's time goes with the bytes it pulls: 8 r weight rows and, from 65 rows on, 128 activation rows
-        const int64_t wgs = slices * ((N + 8 * r - 1) / (8 * r)), cost = ((wgs + 255) / 256) * (M > 64 ? 16 + r : r);
-        if (cost < best_cost || (cost == best_cost && r > best)) { best_cost = cost; best = r; }
-    }
+    int best = choose_rows_r(M, N, rounds > 1, nullptr);
     if ((forced == 2 || forced == 4 || forced == 6 || forced == 8 || forced == 9 || forced == 10) && (M > 64 ? forced <= 4 : forced >= 4)) best = forced;
     if (rounds > 1 && (M > 64 || (M > 32 && best > 6)))
         return fail(LP_ERR_UNSUPPORTED, "lp_gemm_fp8_block: no decode kernel for K = %lld with %lld rows and %d weight rows per workgroup",

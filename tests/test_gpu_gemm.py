@@ -95,6 +95,8 @@ DENSE_SHAPES = [
     # rounds, every kernel of the family), and shapes the rule leaves to the tiled kernels
     (1, 4096, 14336), (16, 7168, 8192), (64, 5120, 7296), (40, 6144, 9216), (128, 7168, 8192), (8, 4096, 57344), (8, 256, 14336), (13, 18432, 8192),
     (64, 8192, 14336), (33, 7168, 18432), (48, 4096, 8192), (100, 3072, 9216),
+    # ... beyond 8192 weight rows: up to 32 rows every cut, above only cuts of at most 48 rows that fill their rounds of workgroups
+    (24, 12288, 8192), (40, 12288, 9216), (20, 18432, 8192), (48, 18432, 8192),
 ]
 
 
