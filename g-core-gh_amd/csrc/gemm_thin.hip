@@ -839,6 +839,10 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
                ((M + 127) / 128) * ((N + 31) / 32) <= 256;
     }
     if (M > 64) return M <= max_m && N / 16 >= wide_min_groups && N <= wide_max_n;
+    // up to 16 rows the 16-row ring kernel stays ahead while it has at most two workgroups per CU and K is short (9 .. 16 x 5120 ..
+    // 8192 x 4096: 8.8 .. 9.1 -> 8.1 .. 8.6 us, x 2048: level to 0.4 ahead; at K = 7168 and 16 rows the many-rows kernel leads, 14.1 -> 13.0)
+    static const bool min_m_given = getenv("LP_GEMM_THIN_ROWS_MIN_M") != nullptr;
+    if (M <= 16 && N <= 8192 && K <= 4096 && !min_m_given) return false;
     return M >= min_m && N / 16 > min_groups;
 }
 

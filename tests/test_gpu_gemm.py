@@ -97,6 +97,8 @@ DENSE_SHAPES = [
     (64, 8192, 14336), (33, 7168, 18432), (48, 4096, 8192), (100, 3072, 9216),
     # ... beyond 8192 weight rows: up to 32 rows every cut, above only cuts of at most 48 rows that fill their rounds of workgroups
     (24, 12288, 8192), (40, 12288, 9216), (20, 18432, 8192), (48, 18432, 8192),
+    # 9 .. 16 rows either side of the hand-over between the 16-row ring kernel and the many-rows kernel
+    (12, 7168, 4096), (16, 8192, 2048), (9, 5120, 4096), (16, 8320, 4096), (12, 8192, 4224),
 ]
 
 
