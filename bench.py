@@ -454,7 +454,10 @@ def main():
         for tag, probe_tag, M3, N3, K3, sets in (("c3_skinny_gemm", "c3_floor_probe", 64, 4096, 7168, 12),
                                                  ("decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", 64, 18432, 7168, 4),
                                                  ("decode_gemm_64x7168x18432", "decode_64x7168x18432_floor_probe", 64, 7168, 18432, 4),
-                                                 ("decode_gemm_1x7168x18432", "decode_1x7168x18432_floor_probe", 1, 7168, 18432, 4)):
+                                                 ("decode_gemm_1x7168x18432", "decode_1x7168x18432_floor_probe", 1, 7168, 18432, 4),
+                                                 # the vocabulary projection as a decode step sees it: 927 MB of weights
+                                                 ("decode_gemm_1x129280x7168", "decode_1x129280x7168_floor_probe", 1, 129280, 7168, 1),
+                                                 ("decode_gemm_16x129280x7168", "decode_16x129280x7168_floor_probe", 16, 129280, 7168, 1)):
             a3 = randn(M3, K3)
             a3q = torch.empty(M3, K3, dtype=torch.uint8, device=dev)
             a3s = torch.empty(M3, K3 // 128, dtype=torch.float32, device=dev)

@@ -126,7 +126,8 @@ def bench_lines(b):
     for tag, v in ex.get("hipblaslt_fp8_tensorwise_scaled_mm", {}).items():
         if "ms" in v:
             L.append(f"  hipBLASLt, one scale per tensor, {tag}: {v['ms'] * 1e3:.1f} us = {v['tflops']:.0f} TFLOP/s ({v['mfma_frac']:.3f})")
-    for tag in ("c3_skinny_gemm", "decode_gemm_64x18432x7168", "decode_gemm_64x7168x18432", "decode_gemm_1x7168x18432"):
+    for tag in ("c3_skinny_gemm", "decode_gemm_64x18432x7168", "decode_gemm_64x7168x18432", "decode_gemm_1x7168x18432",
+                "decode_gemm_1x129280x7168", "decode_gemm_16x129280x7168"):
         if tag in ex:
             L.append(f"  {tag}: {ex[tag]['ms'] * 1e3:.2f} us = {ex[tag]['weight_GB/s']:.0f} GB/s of weights")
     c4 = ex.get("c4_grouped_gemm", {})
@@ -172,7 +173,9 @@ def floor_summary(b):
     for n, tag, ptag, what in (("2", "c3_skinny_gemm", "c3_floor_probe", "config 3: M = 64, N = 4096, K = 7168"),
                                ("3", "decode_gemm_64x18432x7168", "decode_64x18432x7168_floor_probe", "M = 64, N = 18432, K = 7168"),
                                ("3b", "decode_gemm_64x7168x18432", "decode_64x7168x18432_floor_probe", "M = 64, N = 7168, K = 18432: three rounds of K"),
-                               ("3c", "decode_gemm_1x7168x18432", "decode_1x7168x18432_floor_probe", "M = 1, N = 7168, K = 18432: three rounds of K")):
+                               ("3c", "decode_gemm_1x7168x18432", "decode_1x7168x18432_floor_probe", "M = 1, N = 7168, K = 18432: three rounds of K"),
+                               ("3d", "decode_gemm_1x129280x7168", "decode_1x129280x7168_floor_probe", "M = 1, N = 129280, K = 7168: the vocabulary projection"),
+                               ("3e", "decode_gemm_16x129280x7168", "decode_16x129280x7168_floor_probe", "M = 16, N = 129280, K = 7168")):
         if tag in ex and ptag in ex:
             pr = ex[ptag]
             L.append(f"{n}. Decode GEMM ({what}) against an empty launch and a bare read of its weight bytes")
