@@ -843,6 +843,14 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     // 8192 x 4096: 8.8 .. 9.1 -> 8.1 .. 8.6 us, x 2048: level to 0.4 ahead; at K = 7168 and 16 rows the many-rows kernel leads, 14.1 -> 13.0)
     static const bool min_m_given = getenv("LP_GEMM_THIN_ROWS_MIN_M") != nullptr;
     if (M <= 16 && N <= 8192 && K <= 4096 && !min_m_given) return false;
+    // above 32 rows a workgroup pulls as many activation bytes as weight bytes, and once the weight rows fill a round of 256
+    // x 256 tiles the tiled kernels, which share the activations between 256 weight rows, are ahead (us per call, this
+    // kernel -> tiles, 64 rows: 65536 x 4096 63.8 -> 42.3, 98304 x 7168 150.3 -> 127.7, 129280 x 7168 200.6 -> 168.3; 40
+    // rows: 65536 x 7168 86.2 -> 83.1, 129280 x 7168 178.0 -> 162.6, 98304 x 4096 85.1 -> 91.6; at 49152 weight rows, 192
+    // tiles, it depends on K: 64 x 49152 x 4096 49.0 -> 41.1, x 7168 73.3 -> 78.0; 32 rows level, 24 rows 153.1 -> 160.0).
+    // LP_GEMM_THIN_ROWS_TILED_FROM_N = n (tuning aid): from n weight rows.
+    static const int64_t tiled_from_n = getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N") ? atoll(getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N")) : 65536;
+    if (M > 32 && N >= tiled_from_n) return false;
     return M >= min_m && N / 16 > min_groups;
 }
 

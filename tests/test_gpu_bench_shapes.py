@@ -115,13 +115,13 @@ def test_gemm_at_the_reference_benchmarks_largest_shape(G, pow2):
 @pytest.mark.parametrize("pow2", [False, True], ids=["f32scale", "e8m0scale"])
 def test_decode_rows_against_the_vocabulary_projection(G, pow2):
     """1 ... 64 rows x 129280 x 7168: the same vocabulary weight as a decode step sees it (8080 workgroups of 16 weight rows
-    on the ring kernel up to 8 rows, rounds of 256 workgroups on the many-rows kernel above), one weight quantised once,
+    on the ring kernel up to 8 rows, rounds of 256 workgroups on the many-rows kernel up to 32, the tiled kernels above), one weight quantised once,
     checked slab by slab against fp32 dequantise-then-matmul."""
     N, K = 129280, 7168
     w = _randn(N, K, 0.02, 32)
     wq, ws = G.quant_fp8_e4m3_scale_e8m0(w, (128, 128)) if pow2 else G.quant_2d(w)
     del w
-    for M in (1, 7, 16, 24, 64):
+    for M in (1, 7, 16, 24, 40, 64):
         x = _randn(M, K, 1.0, 40 + M)
         xq, xs = G.quant_fp8_e4m3_scale_e8m0(x, (1, 128)) if pow2 else G.quant_1d(x)
         say("decode rows x vocabulary projection", (M, N, K), "e8m0" if pow2 else "f32")
