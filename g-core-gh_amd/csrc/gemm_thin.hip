@@ -843,13 +843,17 @@ bool thin_rows_ok(int64_t M, int64_t N, int64_t K)
     // 8192 x 4096: 8.8 .. 9.1 -> 8.1 .. 8.6 us, x 2048: level to 0.4 ahead; at K = 7168 and 16 rows the many-rows kernel leads, 14.1 -> 13.0)
     static const bool min_m_given = getenv("LP_GEMM_THIN_ROWS_MIN_M") != nullptr;
     if (M <= 16 && N <= 8192 && K <= 4096 && !min_m_given) return false;
-    // above 32 rows a workgroup pulls as many activation bytes as weight bytes, and once the weight rows fill a round of 256
-    // x 256 tiles the tiled kernels, which share the activations between 256 weight rows, are ahead (us per call, this
-    // kernel -> tiles, 64 rows: 65536 x 4096 63.8 -> 42.3, 98304 x 7168 150.3 -> 127.7, 129280 x 7168 200.6 -> 168.3; 40
-    // rows: 65536 x 7168 86.2 -> 83.1, 129280 x 7168 178.0 -> 162.6, 98304 x 4096 85.1 -> 91.6; at 49152 weight rows, 192
-    // tiles, it depends on K: 64 x 49152 x 4096 49.0 -> 41.1, x 7168 73.3 -> 78.0; 32 rows level, 24 rows 153.1 -> 160.0).
-    // LP_GEMM_THIN_ROWS_TILED_FROM_N = n (tuning aid): from n weight rows.
-    static const int64_t tiled_from_n = getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N") ? atoll(getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N")) : 65536;
+    // above 32 rows a workgroup pulls as many activation bytes as weight bytes, and from about a round of 256 x 256 tiles on
+    // the tiled kernels, which share the activations between 256 weight rows, are ahead (us per call, this kernel -> tiles,
+    // 64 rows: 65536 x 4096 63.8 -> 42.3, 98304 x 7168 150.3 -> 127.7, 129280 x 7168 200.6 -> 168.3, 57344 x 7168 113.4 ->
+    // 81.1, 53248 x 7168 86.1 -> 79.9, but 49152 x 7168 72.9 -> 77.0 and 40960 x 7168 61.6 -> 69.8; 40 rows: 129280 x 7168
+    // 178.0 -> 162.6, 53248 x 7168 77.0 -> 75.7).  With K <= 4096 from 24576 weight rows already (64 rows: 24576 x 4096
+    // 29.4 -> 24.9, 32768 x 4096 33.2 -> 25.0, 57344 x 4096 73.6 -> 41.1, 32768 x 2048 19.4 -> 16.8, 24576 x 2048 16.9 -> 16.2,
+    // but 18432 x 4096 20.1 -> 24.2; 40 rows: 24576 x 4096 26.5 -> 24.2, 57344 x 2048 36.9 -> 23.6, 98304 x 4096 85.1 -> 91.6).
+    // 32 rows level at 129280 x 7168, 24 rows 153.1 -> 160.0.  LP_GEMM_THIN_ROWS_TILED_FROM_N = n (tuning aid): from n
+    // weight rows whatever K.
+    static const int64_t tiled_from_env = getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N") ? atoll(getenv("LP_GEMM_THIN_ROWS_TILED_FROM_N")) : 0;
+    const int64_t tiled_from_n = tiled_from_env > 0 ? tiled_from_env : K <= 4096 ? 24576 : 53248;
     if (M > 32 && N >= tiled_from_n) return false;
     return M >= min_m && N / 16 > min_groups;
 }

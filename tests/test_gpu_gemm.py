@@ -99,6 +99,8 @@ DENSE_SHAPES = [
     (24, 12288, 8192), (40, 12288, 9216), (20, 18432, 8192), (48, 18432, 8192),
     # 9 .. 16 rows either side of the hand-over between the 16-row ring kernel and the many-rows kernel
     (12, 7168, 4096), (16, 8192, 2048), (9, 5120, 4096), (16, 8320, 4096), (12, 8192, 4224),
+    # 33 .. 64 rows either side of the weight-row count from which the tiled kernels take them
+    (48, 24576, 2048), (48, 24448, 2048), (32, 24576, 2048),
 ]
 
 
